@@ -1,0 +1,163 @@
+// Channel-mixing linear layers on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
+//
+//   OUT[n, m, :] = X[n, m, :] . W[g(n)][l(m)] / sqrt(K)
+//
+// One wavefront owns a tile of 32 nodes x one component m x all Nout columns, so every row of the
+// tile uses the same K x Nout weight block.  The X rows of the tile (K contiguous floats each) are
+// brought in with fully coalesced 16-byte loads and staged in LDS in chunks of 64 columns; the
+// weight operand is read as 16-byte pieces of the TRANSPOSED weights ([Nout, K], which the caller
+// already keeps for the backward) straight from L1/L2 -- the whole weight set is at most a few
+// hundred KB.  Native fp32 MFMA needs no split-precision compensation.  All (group, m, tile)
+// combinations go out in a single launch; per-element weights are selected through a node
+// permutation that lists the nodes group by group, without any host synchronisation.
+#include <algorithm>
+#include <cmath>
+
+#include "common.hpp"
+
+namespace cm {
+namespace {
+
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kTileNodes = 32;  // MFMA M
+constexpr int kKC = 64;         // columns of X staged per step
+constexpr int kLdA = kKC + 4;   // padded LDS row stride (floats)
+
+template <int NT>  // Nout = 32 * NT
+__global__ __launch_bounds__(kWave) void linear_kernel(const float *__restrict__ X, const float *__restrict__ WT,
+                                                       const int32_t *__restrict__ node_perm,
+                                                       const int32_t *__restrict__ group_offsets, int nnodes,
+                                                       int ngroups, int K, float scale, float *__restrict__ OUT) {
+  constexpr int NOUT = 32 * NT;
+  __shared__ __attribute__((aligned(16))) float sA[kTileNodes * kLdA];
+  __shared__ int sNode[kTileNodes];
+
+  const int lane = threadIdx.x;
+  const int m = blockIdx.y;  // component 0..15
+  const int l = l_of_m(m);
+
+  // locate (group, first position in the grouped node order) of this tile
+  int tile = blockIdx.x;
+  int g = 0, pos0 = 0, gend = nnodes;
+  if (group_offsets) {
+    bool found = false;
+    for (g = 0; g < ngroups; ++g) {
+      const int lo = group_offsets[g], hi = group_offsets[g + 1];
+      const int tiles = (hi - lo + kTileNodes - 1) / kTileNodes;
+      if (tile < tiles) {
+        pos0 = lo + tile * kTileNodes;
+        gend = hi;
+        found = true;
+        break;
+      }
+      tile -= tiles;
+    }
+    if (!found) return;
+  } else {
+    pos0 = tile * kTileNodes;
+    if (pos0 >= nnodes) return;
+  }
+  const int nrows = min(kTileNodes, gend - pos0);
+
+  if (lane < kTileNodes) {
+    int node = -1;
+    if (lane < nrows) {
+      node = node_perm ? node_perm[pos0 + lane] : pos0 + lane;
+      if (static_cast<unsigned>(node) >= static_cast<unsigned>(nnodes)) node = -1;
+    }
+    sNode[lane] = node;
+  }
+  __syncthreads();
+
+  const float *Wg = WT + (static_cast<int64_t>(g) * 4 + l) * NOUT * K;  // [NOUT, K]
+
+  v16f acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+
+  // staging map: 16 lanes x 16 bytes cover the 64 staged columns of a row, 4 rows per load
+  const int srow = lane / 16;
+  const int scol = (lane % 16) * 4;
+  // MFMA operand map: row / column within the tile and which half of the 8-wide k step
+  const int mrow = lane % 32;
+  const int half = lane / 32;
+
+  for (int kc = 0; kc < K; kc += kKC) {
+    const int kw = min(kKC, K - kc);  // multiple of 32
+    f4 pre[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = 4 * i + srow;
+      const int node = sNode[row];
+      pre[i] = zero4();
+      if (node >= 0 && scol < kw) pre[i] = ld4_stream(X + (static_cast<int64_t>(node) * 16 + m) * K + kc + scol);
+    }
+    __syncthreads();  // previous chunk fully consumed
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<f4 *>(sA + (4 * i + srow) * kLdA + scol) = pre[i];
+    __syncthreads();
+
+    for (int kb = 0; kb < kw; kb += 8) {
+      const f4 a = *reinterpret_cast<const f4 *>(sA + mrow * kLdA + kb + 4 * half);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const f4 b = ld4(Wg + static_cast<int64_t>(32 * t + mrow) * K + kc + kb + 4 * half);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc[t], 0, 0, 0);
+      }
+    }
+  }
+
+  // accumulator r of a lane is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the 32x32 block
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = 8 * (r / 4) + 4 * half + (r % 4);
+    const int node = sNode[row];
+    if (node >= 0) {
+      float *op = OUT + (static_cast<int64_t>(node) * 16 + m) * NOUT + mrow;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+    }
+  }
+}
+
+template <int NT>
+int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
+           int K, float *OUT, hipStream_t st) {
+  const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
+  hipLaunchKernelGGL(linear_kernel<NT>, dim3(static_cast<unsigned>(tiles), 16), dim3(kWave), 0, st, X, WT, perm, offs,
+                     static_cast<int>(nnodes), ngroups, K, 1.0f / std::sqrt(static_cast<float>(K)), OUT);
+  return check_launch("cm_linear");
+}
+
+}  // namespace
+}  // namespace cm
+
+extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_perm, const int32_t *group_offsets,
+                         int64_t nnodes, int ngroups, int K, int Nout, float *OUT, cm_stream_t stream) {
+  CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 16, "cm_linear: nnodes out of range");
+  CM_REQUIRE(K >= 32 && K <= 256 && K % 32 == 0, "cm_linear: K=%d must be a multiple of 32 in [32, 256]", K);
+  CM_REQUIRE(Nout >= 32 && Nout <= 256 && Nout % 32 == 0, "cm_linear: Nout=%d must be a multiple of 32 in [32, 256]", Nout);
+  CM_REQUIRE(ngroups >= 1, "cm_linear: ngroups must be at least 1");
+  CM_REQUIRE((node_perm == nullptr) == (group_offsets == nullptr), "cm_linear: node_perm and group_offsets go together");
+  CM_REQUIRE(group_offsets != nullptr || ngroups == 1, "cm_linear: ngroups > 1 needs node_perm / group_offsets");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(X && W_T && OUT, "cm_linear: NULL pointer");
+  hipStream_t st = cm::as_stream(stream);
+  switch (Nout / 32) {
+    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+  }
+  return CM_EINVAL;
+}

@@ -1,0 +1,222 @@
+// Symmetric contraction (correlation 3, scalar output) and its analytic gradient.
+//
+// The cubic form is evaluated over monomials x_i x_j x_k with i <= j <= k whose coefficients
+// T3[e, t, c] (and T2, T1 for the quadratic and linear parts) are folded once per call from the
+// sparse coupling tables and the per-element weights; that removes every permuted duplicate of the
+// packed table from the inner loop.  Nodes are processed grouped by element so that a workgroup
+// works with one coefficient set; a thread owns one channel, the node's 16 inputs and 16 gradient
+// accumulators sit in LDS columns private to that thread (dynamic component indices, no bank
+// conflicts, no synchronisation inside the monomial loop).
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace cm {
+namespace {
+
+// T[e, t, c] = sum over the CSR row t of val * W[e, path, c]
+__global__ void fold_tables_kernel(const int32_t *__restrict__ off, const int32_t *__restrict__ path,
+                                   const float *__restrict__ val, int nmono, const float *__restrict__ W, int ne, int P,
+                                   int C, float *__restrict__ T) {
+  const int64_t idx = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (idx >= static_cast<int64_t>(ne) * nmono * C) return;
+  const int c = idx % C;
+  const int t = (idx / C) % nmono;
+  const int e = idx / (static_cast<int64_t>(C) * nmono);
+  float acc = 0.f;
+  for (int q = off[t]; q < off[t + 1]; ++q) {
+    const int p = path[q];
+    if (static_cast<unsigned>(p) < static_cast<unsigned>(P)) acc += val[q] * W[(static_cast<int64_t>(e) * P + p) * C + c];
+  }
+  T[idx] = acc;
+}
+
+__global__ void copy_w1_kernel(const float *__restrict__ W1, int ne, int P1, int C, float *__restrict__ T1) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= ne * C) return;
+  T1[idx] = W1[(static_cast<int64_t>(idx / C) * P1) * C + idx % C];
+}
+
+// Workgroup: blockDim.x = C threads (one per channel), NB nodes of one element at a time.
+template <int NB, bool GRAD>
+__global__ void symcon_forward_kernel(const float *__restrict__ X, const int32_t *__restrict__ node_perm,
+                                      const int32_t *__restrict__ group_offsets, const int32_t *__restrict__ mono3,
+                                      int n3, const int32_t *__restrict__ mono2, int n2, const float *__restrict__ T3,
+                                      const float *__restrict__ T2, const float *__restrict__ T1, int nnodes, int ne,
+                                      float *__restrict__ out, float *__restrict__ grad) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int C = blockDim.x;
+  const int c = threadIdx.x;
+  float *sx = smem;                 // [NB][16][C]
+  float *sg = smem + NB * 16 * C;   // [NB][16][C] (GRAD only)
+
+  int tile = blockIdx.x;
+  int e = 0, pos0 = 0, gend = 0;
+  bool found = false;
+  for (e = 0; e < ne; ++e) {
+    const int lo = group_offsets[e], hi = group_offsets[e + 1];
+    const int tiles = (hi - lo + NB - 1) / NB;
+    if (tile < tiles) {
+      pos0 = lo + tile * NB;
+      gend = hi;
+      found = true;
+      break;
+    }
+    tile -= tiles;
+  }
+  if (!found) return;
+  const int nb = min(NB, gend - pos0);
+
+  int node[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    node[b] = -1;
+    if (b < nb) {
+      const int n = node_perm[pos0 + b];
+      if (static_cast<unsigned>(n) < static_cast<unsigned>(nnodes)) node[b] = n;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      sx[(b * 16 + i) * C + c] = node[b] >= 0 ? X[(static_cast<int64_t>(node[b]) * 16 + i) * C + c] : 0.f;
+      if (GRAD) sg[(b * 16 + i) * C + c] = 0.f;
+    }
+  }
+  // every thread reads and writes only its own column c of sx / sg: no barrier needed
+
+  float acc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) acc[b] = 0.f;
+
+  const float *t3 = T3 + static_cast<int64_t>(e) * n3 * C + c;
+  for (int t = 0; t < n3; ++t) {
+    const int ijk = mono3[t];
+    const int i = ijk & 0xFF, j = (ijk >> 8) & 0xFF, k = (ijk >> 16) & 0xFF;
+    const float w = t3[static_cast<int64_t>(t) * C];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const float xi = sx[(b * 16 + i) * C + c], xj = sx[(b * 16 + j) * C + c], xk = sx[(b * 16 + k) * C + c];
+      const float wjk = w * xj * xk;
+      acc[b] = fmaf(wjk, xi, acc[b]);
+      if (GRAD) {
+        sg[(b * 16 + i) * C + c] += wjk;
+        sg[(b * 16 + j) * C + c] += w * xi * xk;
+        sg[(b * 16 + k) * C + c] += w * xi * xj;
+      }
+    }
+  }
+  const float *t2 = T2 + static_cast<int64_t>(e) * n2 * C + c;
+  for (int t = 0; t < n2; ++t) {
+    const int ij = mono2[t];
+    const int i = ij & 0xFF, j = (ij >> 8) & 0xFF;
+    const float w = t2[static_cast<int64_t>(t) * C];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const float xi = sx[(b * 16 + i) * C + c], xj = sx[(b * 16 + j) * C + c];
+      acc[b] = fmaf(w * xi, xj, acc[b]);
+      if (GRAD) {
+        sg[(b * 16 + i) * C + c] += w * xj;
+        sg[(b * 16 + j) * C + c] += w * xi;
+      }
+    }
+  }
+  const float w1 = T1[static_cast<int64_t>(e) * C + c];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    if (node[b] < 0) continue;
+    out[static_cast<int64_t>(node[b]) * C + c] = fmaf(w1, sx[(b * 16) * C + c], acc[b]);
+    if (GRAD) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        grad[(static_cast<int64_t>(node[b]) * 16 + i) * C + c] = sg[(b * 16 + i) * C + c] + (i == 0 ? w1 : 0.f);
+    }
+  }
+}
+
+__global__ void symcon_backward_kernel(const float *__restrict__ grad, const float *__restrict__ gout, int64_t nnodes,
+                                       int C, float *__restrict__ gX) {
+  const int C4 = C / 4;
+  const int64_t t = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (t >= nnodes * 16 * C4) return;
+  const int c4 = t % C4;
+  const int64_t n = t / (16 * C4);
+  const f4 g = ld4(gout + n * C + 4 * c4);
+  st4(gX + 4 * t, ld4_stream(grad + 4 * t) * g);
+}
+
+template <int NB>
+void launch_fwd(bool want_grad, unsigned grid, int C, hipStream_t st, const float *X, const int32_t *perm,
+                const int32_t *offs, const int32_t *mono3, int n3, const int32_t *mono2, int n2, const float *T3,
+                const float *T2, const float *T1, int nnodes, int ne, float *out, float *grad) {
+  const size_t lds = static_cast<size_t>(NB) * 16 * C * sizeof(float) * (want_grad ? 2 : 1);
+  if (want_grad)
+    hipLaunchKernelGGL((symcon_forward_kernel<NB, true>), dim3(grid), dim3(C), lds, st, X, perm, offs, mono3, n3, mono2,
+                       n2, T3, T2, T1, nnodes, ne, out, grad);
+  else
+    hipLaunchKernelGGL((symcon_forward_kernel<NB, false>), dim3(grid), dim3(C), lds, st, X, perm, offs, mono3, n3, mono2,
+                       n2, T3, T2, T1, nnodes, ne, out, grad);
+}
+
+}  // namespace
+}  // namespace cm
+
+extern "C" int cm_symcon_tables(const int32_t *term3_off, const int32_t *term3_path, const float *term3_val, int n3,
+                                const int32_t *term2_off, const int32_t *term2_path, const float *term2_val, int n2,
+                                const float *W3, const float *W2, const float *W1, int nelements, int P3, int P2,
+                                int P1, int channels, float *T3, float *T2, float *T1, cm_stream_t stream) {
+  CM_REQUIRE(n3 >= 0 && n2 >= 0 && nelements >= 1 && P3 >= 1 && P2 >= 1 && P1 >= 1 && channels >= 1,
+             "cm_symcon_tables: bad sizes");
+  CM_REQUIRE(term3_off && term2_off && W3 && W2 && W1 && T1, "cm_symcon_tables: NULL pointer");
+  CM_REQUIRE((n3 == 0 || T3) && (n2 == 0 || T2), "cm_symcon_tables: NULL output table");
+  hipStream_t st = cm::as_stream(stream);
+  const int block = 256;
+  if (n3 > 0) {
+    const int64_t tot = static_cast<int64_t>(nelements) * n3 * channels;
+    hipLaunchKernelGGL(cm::fold_tables_kernel, dim3(static_cast<unsigned>(cm::ceil_div(tot, block))), dim3(block), 0, st,
+                       term3_off, term3_path, term3_val, n3, W3, nelements, P3, channels, T3);
+  }
+  if (n2 > 0) {
+    const int64_t tot = static_cast<int64_t>(nelements) * n2 * channels;
+    hipLaunchKernelGGL(cm::fold_tables_kernel, dim3(static_cast<unsigned>(cm::ceil_div(tot, block))), dim3(block), 0, st,
+                       term2_off, term2_path, term2_val, n2, W2, nelements, P2, channels, T2);
+  }
+  hipLaunchKernelGGL(cm::copy_w1_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nelements * channels, block))),
+                     dim3(block), 0, st, W1, nelements, P1, channels, T1);
+  return cm::check_launch("cm_symcon_tables");
+}
+
+extern "C" int cm_symcon_forward(const float *X, const int32_t *node_perm, const int32_t *group_offsets,
+                                 const int32_t *mono3_ijk, int n3, const int32_t *mono2_ij, int n2, const float *T3,
+                                 const float *T2, const float *T1, int64_t nnodes, int nelements, int channels,
+                                 float *out, float *grad, cm_stream_t stream) {
+  CM_REQUIRE(cm_channels_supported(channels), "cm_symcon_forward: channels=%d must be a multiple of 32 in [32, 256]", channels);
+  CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 16, "cm_symcon_forward: nnodes out of range");
+  CM_REQUIRE(nelements >= 1 && n3 >= 0 && n2 >= 0, "cm_symcon_forward: bad sizes");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(X && node_perm && group_offsets && T1 && out, "cm_symcon_forward: NULL pointer");
+  CM_REQUIRE((n3 == 0 || (mono3_ijk && T3)) && (n2 == 0 || (mono2_ij && T2)), "cm_symcon_forward: NULL table");
+  hipStream_t st = cm::as_stream(stream);
+  // LDS per workgroup is held to 32 KB (two [NB][16][C] fp32 arrays) so that several fit a CU
+  if (channels <= 128) {
+    const unsigned grid = static_cast<unsigned>(cm::ceil_div(nnodes, 2) + nelements);
+    cm::launch_fwd<2>(grad != nullptr, grid, channels, st, X, node_perm, group_offsets, mono3_ijk, n3, mono2_ij, n2, T3,
+                      T2, T1, static_cast<int>(nnodes), nelements, out, grad);
+  } else {
+    const unsigned grid = static_cast<unsigned>(nnodes + nelements);
+    cm::launch_fwd<1>(grad != nullptr, grid, channels, st, X, node_perm, group_offsets, mono3_ijk, n3, mono2_ij, n2, T3,
+                      T2, T1, static_cast<int>(nnodes), nelements, out, grad);
+  }
+  return cm::check_launch("cm_symcon_forward");
+}
+
+extern "C" int cm_symcon_backward(const float *grad, const float *grad_out, int64_t nnodes, int channels, float *gX,
+                                  cm_stream_t stream) {
+  CM_REQUIRE(channels >= 4 && channels % 4 == 0, "cm_symcon_backward: channels must be a multiple of 4");
+  CM_REQUIRE(nnodes >= 0, "cm_symcon_backward: negative size");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(grad && grad_out && gX, "cm_symcon_backward: NULL pointer");
+  const int block = 256;
+  const int64_t threads = nnodes * 16 * (channels / 4);
+  hipLaunchKernelGGL(cm::symcon_backward_kernel, dim3(static_cast<unsigned>(cm::ceil_div(threads, block))), dim3(block), 0,
+                     cm::as_stream(stream), grad, grad_out, nnodes, channels, gX);
+  return cm::check_launch("cm_symcon_backward");
+}

@@ -1,0 +1,259 @@
+"""ctypes binding of libcuda_mace_hip.so (the C ABI declared in include/cuda_mace_hip.h).
+
+Torch is used only to own device memory and to name the current HIP stream; every compute call
+goes through the C entry points.  There is no fallback: if the library is missing the import
+fails, and if a call is given host tensors it raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+_HERE = os.path.realpath(os.path.dirname(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libcuda_mace_hip.so")
+
+if not os.path.isfile(LIB_PATH):
+    raise ImportError(
+        "Could not find the HIP kernel library at %s; build it with `python cuda-mace_amd/build.py`" % LIB_PATH
+    )
+
+lib = ctypes.CDLL(LIB_PATH)
+
+_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_i32 = ctypes.c_int
+_f32 = ctypes.c_float
+_sz = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/cuda_mace_hip.h one to one
+SIGNATURES = {
+    "cm_abi_version": (_i32, []),
+    "cm_last_error": (ctypes.c_char_p, []),
+    "cm_channels_supported": (_i32, [_i32]),
+    "cm_first_occurences": (_i32, [_p, _i64, _i64, _p, _p]),
+    "cm_stable_key_sort_workspace": (_sz, [_i64, _i64]),
+    "cm_stable_key_sort": (_i32, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),
+    "cm_mp_forward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _p, _p]),
+    "cm_mp_backward": (_i32, [_p] * 8 + [_i64, _i64, _i32] + [_p] * 5),
+    "cm_sh_forward": (_i32, [_p, _i64, _p, _p]),
+    "cm_sh_backward": (_i32, [_p, _p, _i64, _p, _p]),
+    "cm_spline_forward": (_i32, [_p, _p, _p, _i64, _i32, _i32, _f32, _f32, _p, _p, _p]),
+    "cm_spline_backward": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _f32, _f32, _p, _p]),
+    "cm_linear": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _p, _p]),
+    "cm_symcon_tables": (_i32, [_p, _p, _p, _i32, _p, _p, _p, _i32, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _p, _p, _p]),
+    "cm_symcon_forward": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
+    "cm_symcon_backward": (_i32, [_p, _p, _i64, _i32, _p, _p]),
+}
+
+for _name, (_res, _args) in SIGNATURES.items():
+    _fn = getattr(lib, _name)
+    _fn.restype = _res
+    _fn.argtypes = _args
+
+
+class CudaMaceError(RuntimeError):
+    pass
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise CudaMaceError("%s (code %d)" % (lib.cm_last_error().decode(), rc))
+
+
+def _dev(t: Optional[torch.Tensor], dtype: torch.dtype, name: str) -> Optional[int]:
+    """Device address of a contiguous tensor after checking what the C side assumes."""
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise CudaMaceError("%s must live on the GPU (got a %s tensor)" % (name, t.device))
+    if t.dtype != dtype:
+        raise CudaMaceError("%s must be %s (got %s)" % (name, dtype, t.dtype))
+    if not t.is_contiguous():
+        raise CudaMaceError("%s must be contiguous" % name)
+    return t.data_ptr() if t.numel() > 0 else None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+F32, I32 = torch.float32, torch.int32
+
+
+# ---- index kernels ---------------------------------------------------------------------------
+def first_occurences(receiver: torch.Tensor, nnodes: int) -> torch.Tensor:
+    out = torch.empty(2 * nnodes, dtype=I32, device=receiver.device)
+    _check(lib.cm_first_occurences(_dev(receiver, I32, "receiver_list"), receiver.numel(), nnodes, _dev(out, I32, "out"), _stream()))
+    return out
+
+
+def stable_key_sort(keys: torch.Tensor, nkeys: int):
+    n = keys.numel()
+    perm = torch.empty(n, dtype=I32, device=keys.device)
+    offsets = torch.empty(nkeys + 1, dtype=I32, device=keys.device)
+    nbytes = lib.cm_stable_key_sort_workspace(n, nkeys)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=keys.device)
+    _check(
+        lib.cm_stable_key_sort(
+            _dev(keys, I32, "keys"), n, nkeys, _dev(perm, I32, "perm"), _dev(offsets, I32, "offsets"),
+            ws.data_ptr(), nbytes, _stream(),
+        )
+    )
+    return perm, offsets
+
+
+# ---- message passing --------------------------------------------------------------------------
+def mp_forward(X, Y, R, sender, first_occ, nnodes: int) -> torch.Tensor:
+    C = X.shape[-1]
+    E = sender.numel()
+    if Y.shape != (16, E):
+        raise CudaMaceError("Y must be [16, nedges] = [16, %d], got %s" % (E, tuple(Y.shape)))
+    if R.numel() != E * 4 * C:
+        raise CudaMaceError("radial must hold nedges*4*channels = %d values, got %d" % (E * 4 * C, R.numel()))
+    if X.shape[0] != nnodes:
+        raise CudaMaceError("X must be [nnodes, channels]")
+    out = torch.empty(nnodes, 16, C, dtype=F32, device=X.device)
+    _check(
+        lib.cm_mp_forward(
+            _dev(X, F32, "X"), _dev(Y, F32, "Y"), _dev(R, F32, "radial"), _dev(sender, I32, "sender_list"),
+            _dev(first_occ, I32, "first_occurences"), nnodes, E, C, _dev(out, F32, "out"), _stream(),
+        )
+    )
+    return out
+
+
+def mp_backward(X, Y, R, grad_out, sender, first_occ, sender_perm, sender_offsets, nnodes: int,
+                need_gX: bool = True, need_gY: bool = True, need_gR: bool = True):
+    C = X.shape[-1]
+    E = sender.numel()
+    dev = X.device
+    gX = torch.empty(nnodes, C, dtype=F32, device=dev) if need_gX else None
+    gY = torch.empty(16, E, dtype=F32, device=dev) if need_gY else None
+    gR = torch.empty(E, 4, C, dtype=F32, device=dev) if need_gR else None
+    scratch = torch.empty(E, C, dtype=F32, device=dev) if need_gX else None
+    _check(
+        lib.cm_mp_backward(
+            _dev(X, F32, "X"), _dev(Y, F32, "Y"), _dev(R, F32, "radial"), _dev(grad_out, F32, "grad_out"),
+            _dev(sender, I32, "sender_list"), _dev(first_occ, I32, "first_occurences"),
+            _dev(sender_perm, I32, "sender_perm") if need_gX else None,
+            _dev(sender_offsets, I32, "sender_offsets") if need_gX else None,
+            nnodes, E, C, _dev(gX, F32, "gX"), _dev(gY, F32, "gY"), _dev(gR, F32, "gR"), _dev(scratch, F32, "scratch"), _stream(),
+        )
+    )
+    return gX, gY, gR
+
+
+# ---- spherical harmonics ------------------------------------------------------------------------
+def sh_forward(xyz: torch.Tensor) -> torch.Tensor:
+    E = xyz.shape[0]
+    Y = torch.empty(16, E, dtype=F32, device=xyz.device)
+    _check(lib.cm_sh_forward(_dev(xyz, F32, "xyz"), E, _dev(Y, F32, "Y"), _stream()))
+    return Y
+
+
+def sh_backward(xyz: torch.Tensor, grad_Y: torch.Tensor) -> torch.Tensor:
+    E = xyz.shape[0]
+    g = torch.empty(E, 3, dtype=F32, device=xyz.device)
+    _check(lib.cm_sh_backward(_dev(xyz, F32, "xyz"), _dev(grad_Y, F32, "grad_Y"), E, _dev(g, F32, "grad_xyz"), _stream()))
+    return g
+
+
+# ---- cubic spline ---------------------------------------------------------------------------------
+def spline_forward(r, r_knots, coeffs, r_width: float, r_max: float, want_deriv: bool = False):
+    E = r.numel()
+    J = coeffs.shape[-1]
+    nknots = r_knots.numel()
+    if coeffs.shape[0] != nknots - 1 or coeffs.shape[1] != 4:
+        raise CudaMaceError("coeffs must be [nknots-1, 4, noutputs]")
+    R = torch.empty(E, J, dtype=F32, device=r.device)
+    dR = torch.empty(E, J, dtype=F32, device=r.device) if want_deriv else None
+    _check(
+        lib.cm_spline_forward(
+            _dev(r, F32, "r"), _dev(r_knots, F32, "r_knots"), _dev(coeffs, F32, "coeffs"), E, nknots, J,
+            float(r_width), float(r_max), _dev(R, F32, "R_out"), _dev(dR, F32, "R_deriv"), _stream(),
+        )
+    )
+    return (R, dR) if want_deriv else R
+
+
+def spline_backward(r, r_knots, coeffs, grad_R, r_width: float, r_max: float) -> torch.Tensor:
+    E = r.numel()
+    J = coeffs.shape[-1]
+    out = torch.empty(E, dtype=F32, device=r.device)
+    _check(
+        lib.cm_spline_backward(
+            _dev(r, F32, "r"), _dev(r_knots, F32, "r_knots"), _dev(coeffs, F32, "coeffs"), _dev(grad_R, F32, "grad_R"),
+            E, r_knots.numel(), J, float(r_width), float(r_max), _dev(out, F32, "grad_r"), _stream(),
+        )
+    )
+    return out
+
+
+# ---- linears ------------------------------------------------------------------------------------------
+def linear(X, W_T, node_perm=None, group_offsets=None) -> torch.Tensor:
+    """X [N,16,K]; W_T [4,N',K] or [ngroups,4,N',K] (transposed weight blocks)."""
+    if W_T.dim() == 3:
+        W_T = W_T.unsqueeze(0)
+    ngroups, four, Nout, K = W_T.shape
+    if four != 4 or X.dim() != 3 or X.shape[1] != 16 or X.shape[2] != K:
+        raise CudaMaceError("linear: X must be [N,16,K] and W_T [(ngroups,)4,N',K]")
+    N = X.shape[0]
+    grouped = node_perm is not None
+    OUT = (torch.zeros if grouped else torch.empty)(N, 16, Nout, dtype=F32, device=X.device)
+    _check(
+        lib.cm_linear(
+            _dev(X, F32, "X"), _dev(W_T, F32, "W_T"), _dev(node_perm, I32, "node_perm"),
+            _dev(group_offsets, I32, "group_offsets"), N, ngroups, K, Nout, _dev(OUT, F32, "OUT"), _stream(),
+        )
+    )
+    return OUT
+
+
+# ---- symmetric contraction -----------------------------------------------------------------------------
+def symcon_tables(term3_off, term3_path, term3_val, term2_off, term2_path, term2_val, W3, W2, W1):
+    ne, P3, C = W3.shape
+    P2 = W2.shape[1]
+    P1 = W1.shape[1]
+    n3 = term3_off.numel() - 1
+    n2 = term2_off.numel() - 1
+    dev = W3.device
+    T3 = torch.empty(ne, n3, C, dtype=F32, device=dev)
+    T2 = torch.empty(ne, n2, C, dtype=F32, device=dev)
+    T1 = torch.empty(ne, C, dtype=F32, device=dev)
+    _check(
+        lib.cm_symcon_tables(
+            _dev(term3_off, I32, "term3_off"), _dev(term3_path, I32, "term3_path"), _dev(term3_val, F32, "term3_val"), n3,
+            _dev(term2_off, I32, "term2_off"), _dev(term2_path, I32, "term2_path"), _dev(term2_val, F32, "term2_val"), n2,
+            _dev(W3, F32, "W3"), _dev(W2, F32, "W2"), _dev(W1, F32, "W1"), ne, P3, P2, P1, C,
+            _dev(T3, F32, "T3"), _dev(T2, F32, "T2"), _dev(T1, F32, "T1"), _stream(),
+        )
+    )
+    return T3, T2, T1
+
+
+def symcon_forward(X, node_perm, group_offsets, mono3, mono2, T3, T2, T1, want_grad: bool = True):
+    N, sixteen, C = X.shape
+    if sixteen != 16:
+        raise CudaMaceError("symmetric contraction: X must be [N,16,C]")
+    ne = T1.shape[0]
+    out = torch.zeros(N, C, dtype=F32, device=X.device)
+    grad = torch.zeros(N, 16, C, dtype=F32, device=X.device) if want_grad else None
+    _check(
+        lib.cm_symcon_forward(
+            _dev(X, F32, "X"), _dev(node_perm, I32, "node_perm"), _dev(group_offsets, I32, "group_offsets"),
+            _dev(mono3, I32, "mono3"), mono3.numel(), _dev(mono2, I32, "mono2"), mono2.numel(),
+            _dev(T3, F32, "T3"), _dev(T2, F32, "T2"), _dev(T1, F32, "T1"), N, ne, C,
+            _dev(out, F32, "out"), _dev(grad, F32, "grad"), _stream(),
+        )
+    )
+    return out, grad
+
+
+def symcon_backward(grad, grad_out) -> torch.Tensor:
+    N, _, C = grad.shape
+    gX = torch.empty_like(grad)
+    _check(lib.cm_symcon_backward(_dev(grad, F32, "grad"), _dev(grad_out, F32, "grad_out"), N, C, _dev(gX, F32, "gX"), _stream()))
+    return gX

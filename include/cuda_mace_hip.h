@@ -1,0 +1,184 @@
+/*
+ * C ABI of libcuda_mace_hip.so: the invariant-MACE hot path as hand-written HIP kernels for
+ * gfx950 (MI355X).  Plain pointers and sizes only; every pointer is DEVICE memory unless a
+ * comment says otherwise; every tensor is contiguous row-major fp32 / int32.  Each entry point
+ * enqueues its kernels on `stream` (a hipStream_t passed as void*, NULL = the default stream),
+ * returns without synchronising, and returns 0 on success or a negative CM_E* code after
+ * storing a message retrievable with cm_last_error().  Argument checking happens on the host
+ * before anything is launched; no entry point allocates or frees device memory.
+ *
+ * The reference exposes this path as TorchScript custom classes whose C++ launchers are the
+ * jit_* free functions cited below (paths relative to the reference tree); each entry point
+ * here replaces the launcher + kernel pair named in its comment.
+ */
+#ifndef CUDA_MACE_HIP_H
+#define CUDA_MACE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CM_OK 0
+#define CM_EINVAL (-22)   /* bad shape / null pointer / unsupported channel count */
+#define CM_ELAUNCH (-5)   /* the HIP runtime refused a launch */
+#define CM_ENOSPC (-28)   /* caller's workspace too small */
+
+typedef void *cm_stream_t;
+
+/* ABI version, bumped on any signature change. */
+int cm_abi_version(void);
+/* Message of the calling thread's most recent failure ("" if none). Host pointer, do not free. */
+const char *cm_last_error(void);
+/* 1 if `channels` is a supported feature width (multiple of 32, 32..256), else 0. */
+int cm_channels_supported(int channels);
+
+/* ---------------------------------------------------------------------------------------------
+ * CSR offsets of a non-decreasing receiver list.
+ * Replaces jit_calculate_first_occurences (jit_wrappers/src/invariant_message_passing_wrapper.cpp:19-70)
+ * and calculate_first_occurences_kernel_ptr (cuda/src/invariant_message_passing_impl.cu:8-72).
+ *   receiver   int32 [nedges], non-decreasing, values in [0, nnodes)
+ *   first_occ  int32 [2 * nnodes]: [n] = first edge of node n, [nnodes + n] = one past its last.
+ * Nodes without edges get start == end == insertion point (the reference leaves them undefined).
+ */
+int cm_first_occurences(const int32_t *receiver, int64_t nedges, int64_t nnodes,
+                        int32_t *first_occ, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Stable counting sort of item indices by key: perm lists items by non-decreasing key, ties in
+ * original order; offsets[k] = number of items with key < k (offsets has nkeys + 1 entries).
+ * Used for the sender-sorted view of the edge list, which takes the place of the reference's
+ * N x N reverse-edge table (jit_wrappers/src/invariant_message_passing_wrapper.cpp:91-93;
+ * cuda/src/invariant_message_passing_impl.cu:112-116, 331-336), and for grouping nodes by
+ * element, which takes the place of the per-element torch::where + host sync in
+ * jit_elemental_linear (jit_wrappers/src/linear_wrapper.cpp:137-145).
+ *   keys int32 [n] in [0, nkeys); perm int32 [n]; offsets int32 [nkeys + 1];
+ *   workspace: cm_stable_key_sort_workspace(n, nkeys) bytes of device memory.
+ */
+size_t cm_stable_key_sort_workspace(int64_t n, int64_t nkeys);
+int cm_stable_key_sort(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm,
+                       int32_t *offsets, void *workspace, size_t workspace_bytes,
+                       cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Invariant message passing, forward.
+ * Replaces jit_forward_message_passing (jit_wrappers/src/invariant_message_passing_wrapper.cpp:72-155)
+ * and inv_tp_kernel_ptr (cuda/src/invariant_message_passing_impl.cu:74-165).
+ *   out[n, m, c] = sum_{e in [first_occ[n], first_occ[nnodes + n])} X[sender[e], c] * Y[m, e] * R[e, l(m), c]
+ *   X [nnodes, channels]; Y [16, nedges]; R [nedges, 4, channels]; sender int32 [nedges];
+ *   first_occ from cm_first_occurences; out [nnodes, 16, channels] (rows of edgeless nodes = 0).
+ * No N x N side table is produced.
+ */
+int cm_mp_forward(const float *X, const float *Y, const float *R, const int32_t *sender,
+                  const int32_t *first_occ, int64_t nnodes, int64_t nedges, int channels,
+                  float *out, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Invariant message passing, backward.
+ * Replaces jit_backward_message_passing (jit_wrappers/src/invariant_message_passing_wrapper.cpp:157-284),
+ * backward_edge_inv_tp_kernel_ptr (cuda/src/invariant_message_passing_impl.cu:167-294) and
+ * backward_node_inv_tp_kernel_ptr (:296-399).
+ *   grad_out [nnodes, 16, channels]
+ *   gY [16, nedges]           (may be NULL: not computed)
+ *   gR [nedges, 4, channels]  (may be NULL: not computed)
+ *   gX [nnodes, channels]     (may be NULL: not computed).  When gX is wanted the caller also
+ *      passes the sender-sorted view (sender_perm [nedges], sender_offsets [nnodes + 1] from
+ *      cm_stable_key_sort(sender, nedges, nnodes, ...)) and edge_scratch, fp32
+ *      [nedges, channels], which receives the per-edge contributions that the second kernel
+ *      sums per sender.  Works for any directed multigraph.
+ */
+int cm_mp_backward(const float *X, const float *Y, const float *R, const float *grad_out,
+                   const int32_t *sender, const int32_t *first_occ, const int32_t *sender_perm,
+                   const int32_t *sender_offsets, int64_t nnodes, int64_t nedges, int channels,
+                   float *gX, float *gY, float *gR, float *edge_scratch, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Real spherical harmonics l <= 3 of normalised edge vectors, sqrt(4 pi) ("component")
+ * normalisation, input axes permuted as (x, y, z) = (in[2], in[0], in[1]).
+ * Replaces jit_spherical_harmonics / jit_spherical_harmonics_backward
+ * (jit_wrappers/src/spherical_harmonics_wrapper.cpp:15-83, 85-137) and
+ * spherical_harmonics_kernel_ptr / spherical_harmonics_backward_kernel_ptr
+ * (cuda/src/spherical_harmonics_impl.cu:21-282, 284-334).
+ *   xyz [nedges, 3] -> Y [16, nedges];  backward: grad_Y [16, nedges] -> grad_xyz [nedges, 3]
+ * The backward recomputes the Jacobian from xyz instead of reading a stored [16, 3, nedges] one.
+ */
+int cm_sh_forward(const float *xyz, int64_t nedges, float *Y, cm_stream_t stream);
+int cm_sh_backward(const float *xyz, const float *grad_Y, int64_t nedges, float *grad_xyz,
+                   cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Tabulated radial functions: natural cubic spline, R[e, j] = a + b x + c x^2 + d x^3 with
+ * x = r[e] - r_knots[idx], idx = clamp(int(r[e] / r_width), 0, nknots - 2); zero when r[e] > r_max.
+ * Replaces jit_evaluate_spline / jit_backward_spline (jit_wrappers/src/cubic_spline_wrapper.cpp:14-97,
+ * 99-153) and evaluate_spline_kernel_ptr / backward_spline_kernel_ptr
+ * (cuda/src/cubic_spline_impl.cu:5-66, 68-107).
+ *   r [nedges]; r_knots [nknots]; coeffs [nknots - 1, 4, noutputs]; R_out [nedges, noutputs];
+ *   R_deriv [nedges, noutputs] or NULL.  noutputs must be a multiple of 4.
+ * Backward: grad_r[e] = sum_j grad_R[e, j] * dR/dr[e, j], with dR/dr recomputed from the table.
+ */
+int cm_spline_forward(const float *r, const float *r_knots, const float *coeffs, int64_t nedges,
+                      int nknots, int noutputs, float r_width, float r_max, float *R_out,
+                      float *R_deriv, cm_stream_t stream);
+int cm_spline_backward(const float *r, const float *r_knots, const float *coeffs,
+                       const float *grad_R, int64_t nedges, int nknots, int noutputs,
+                       float r_width, float r_max, float *grad_r, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Channel-mixing linear layers on fp32 MFMA: OUT[n, m, :] = X[n, m, :] . W[g(n)][l(m)] / sqrt(K).
+ * Replaces jit_linear and jit_elemental_linear (jit_wrappers/src/linear_wrapper.cpp:23-95, 97-191) and
+ * linear_kernel_ptr / elemental_linear_kernel_ptr (cuda/src/linear_impl.cu:16-133, 134-255).
+ *   X [nnodes, 16, K]; OUT [nnodes, 16, Nout];
+ *   W_T [ngroups, 4, Nout, K]: the TRANSPOSED weight blocks, W_T[g][l][j][k] = W[g][l][k][j].  The
+ *   reference keeps both W and W_T as module buffers (ops/linear.py:47-51); the forward passes its
+ *   weights_transposed buffer here and the backward with respect to X passes its weights buffer.
+ *   Plain linear: ngroups = 1, node_perm = group_offsets = NULL.
+ *   Per-element linear: node_perm int32 [nnodes] lists nodes grouped by element and
+ *   group_offsets int32 [ngroups + 1] delimits the groups (cm_stable_key_sort on the element
+ *   index); rows of nodes that are in no group are not written.
+ *   K and Nout: multiples of 32 in [32, 256].
+ */
+int cm_linear(const float *X, const float *W_T, const int32_t *node_perm,
+              const int32_t *group_offsets, int64_t nnodes, int ngroups, int K, int Nout,
+              float *OUT, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Symmetric contraction, correlation 3, scalar (L = 0) output, with its analytic gradient.
+ * Replaces jit_symmetric_contraction_forward / _backward
+ * (jit_wrappers/src/symmetric_contraction_wrapper.cpp:15-156, 158-205) and
+ * symmetric_contraction_kernel / symm_contraction_backward_kernel
+ * (cuda/src/symmetric_contraction_impl.cu:6-196, 198-234).
+ *
+ * The cubic form is evaluated over monomials x_i x_j x_k, i <= j <= k:
+ *   out[n, c] = sum_t T3[e, t, c] x_i(t) x_j(t) x_k(t) + sum_q T2[e, q, c] x_i(q) x_j(q)
+ *             + T1[e, c] x_0,     e = atom_types[n], x_i = X[n, i, c]
+ * cm_symcon_tables builds T3/T2/T1 on the device from the reference's packed sparse U tables and
+ * its per-element weights (ops/symmetric_contraction.py:91-232): for every monomial the packed
+ * entries (i, j, k, path) that map onto it are listed in CSR form by the host.
+ *   mono3_ijk  int32 [n3]  : i | j << 8 | k << 16, sorted triples
+ *   term3_off  int32 [n3+1], term3_path int32 [nt3], term3_val fp32 [nt3]: CSR of (path, U value)
+ *   same for the quadratic part (mono2_ij: i | j << 8).
+ *   W3 [ne, P3, C], W2 [ne, P2, C], W1 [ne, P1, C] (only path 0 of W1 is used, as in the reference)
+ *   T3 [ne, n3, C], T2 [ne, n2, C], T1 [ne, C]
+ */
+int cm_symcon_tables(const int32_t *term3_off, const int32_t *term3_path, const float *term3_val,
+                     int n3, const int32_t *term2_off, const int32_t *term2_path,
+                     const float *term2_val, int n2, const float *W3, const float *W2,
+                     const float *W1, int nelements, int P3, int P2, int P1, int channels,
+                     float *T3, float *T2, float *T1, cm_stream_t stream);
+/*   X [nnodes, 16, C]; atom_types int32 [nnodes] in [0, nelements);
+ *   node_perm / group_offsets: nodes grouped by element (cm_stable_key_sort on atom_types);
+ *   out [nnodes, C]; grad [nnodes, 16, C] or NULL (d out[n, c] / d X[n, i, c]). */
+int cm_symcon_forward(const float *X, const int32_t *node_perm, const int32_t *group_offsets,
+                      const int32_t *mono3_ijk, int n3, const int32_t *mono2_ij, int n2,
+                      const float *T3, const float *T2, const float *T1, int64_t nnodes,
+                      int nelements, int channels, float *out, float *grad, cm_stream_t stream);
+/*   gX[n, i, c] = grad_out[n, c] * grad[n, i, c] */
+int cm_symcon_backward(const float *grad, const float *grad_out, int64_t nnodes, int channels,
+                       float *gX, cm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUDA_MACE_HIP_H */

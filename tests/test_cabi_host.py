@@ -1,0 +1,54 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports every symbol the
+header declares, and the ctypes table covers exactly those symbols."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "cuda_mace_hip.h")
+LIB = os.path.join(ROOT, "cuda-mace_amd", "cuda_mace", "lib", "libcuda_mace_hip.so")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.isfile(LIB), "build the library first: python cuda-mace_amd/build.py"
+    lib = ctypes.CDLL(LIB)
+    names = _declared()
+    assert len(names) >= 15
+    for name in names:
+        assert hasattr(lib, name), name
+
+
+def test_ctypes_table_matches_header():
+    from cuda_mace import _cabi
+
+    assert sorted(_cabi.SIGNATURES) == _declared()
+
+
+def test_host_side_validation_needs_no_gpu():
+    lib = ctypes.CDLL(LIB)
+    lib.cm_last_error.restype = ctypes.c_char_p
+    assert lib.cm_abi_version() >= 1
+    assert lib.cm_channels_supported(128) == 1 and lib.cm_channels_supported(48) == 0
+    lib.cm_mp_forward.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    rc = lib.cm_mp_forward(None, None, None, None, None, 10, 10, 48, None, None)
+    assert rc == -22 and b"multiple of 32" in lib.cm_last_error()
+    rc = lib.cm_mp_forward(None, None, None, None, None, 10, 10, 64, None, None)
+    assert rc == -22 and b"NULL" in lib.cm_last_error()
+    lib.cm_stable_key_sort_workspace.restype = ctypes.c_size_t
+    lib.cm_stable_key_sort_workspace.argtypes = [ctypes.c_int64, ctypes.c_int64]
+    assert lib.cm_stable_key_sort_workspace(100, 10) >= 4 * 120
+
+
+def test_binding_rejects_host_tensors():
+    import pytest
+    import torch
+    from cuda_mace import _cabi
+
+    with pytest.raises(RuntimeError, match="GPU"):
+        _cabi.sh_forward(torch.zeros(4, 3))

@@ -1,0 +1,301 @@
+"""GPU parity of every C-ABI entry point against the fp64 CPU oracle on the same seeded inputs.
+
+Tolerances (fp32 kernels vs fp64 oracle): relative 2e-5 with an absolute floor of 2e-6 of the
+largest expected magnitude for sums of O(50) N(0,1) products; index kernels must be bit-exact.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ops as O
+from tests.util import close, mp_inputs, random_graph
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 2e-5
+ATOL = 2e-6
+DEV = "cuda"
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+# ------------------------------------------------------------------------------------------------
+# index kernels: bit-exact
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize(
+    "nnodes,avg,iso,seed",
+    [(1, 1, 0.0, 0), (7, 3, 0.5, 1), (1000, 30, 0.0, 2), (4097, 5, 0.3, 3), (300, 700, 0.1, 4), (50, 0, 0.0, 5)],
+)
+def test_first_occurences_exact(cabi, nnodes, avg, iso, seed):
+    _say("first_occurences", nnodes, avg, iso, seed)
+    _, recv = random_graph(nnodes, avg, seed, isolated_frac=iso)
+    ref = O.first_occurences(recv, nnodes)
+    got = cabi.first_occurences(recv.to(DEV), nnodes).cpu()
+    assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize("n,nkeys,seed", [(0, 5, 0), (1, 1, 1), (1000, 10, 2), (122880, 4096, 3), (5000, 1, 4), (3000, 10000, 5)])
+def test_stable_key_sort_exact(cabi, n, nkeys, seed):
+    _say("stable_key_sort", n, nkeys, seed)
+    keys = torch.from_numpy(np.random.default_rng(seed).integers(0, nkeys, n).astype(np.int32))
+    perm_ref, off_ref = O.stable_key_sort(keys, nkeys)
+    perm, off = cabi.stable_key_sort(keys.to(DEV), nkeys)
+    assert torch.equal(off.cpu(), off_ref)
+    assert torch.equal(perm.cpu(), perm_ref)
+
+
+# ------------------------------------------------------------------------------------------------
+# message passing
+# ------------------------------------------------------------------------------------------------
+MP_CASES = [
+    # nnodes, avg degree, channels, degree mode, isolated fraction, seed
+    (64, 8, 32, "poisson", 0.2, 0),
+    (200, 30, 64, "poisson", 0.0, 1),
+    (512, 30, 96, "fixed", 0.0, 2),
+    (300, 52, 128, "poisson", 0.05, 3),
+    (40, 150, 128, "poisson", 0.0, 4),  # segments longer than one 64-edge chunk
+    (100, 20, 160, "poisson", 0.1, 5),
+    (150, 40, 192, "poisson", 0.0, 6),
+    (60, 10, 224, "poisson", 0.0, 7),
+    (80, 25, 256, "poisson", 0.3, 8),
+    (3, 1, 128, "fixed", 0.0, 9),
+]
+
+
+def _mp_case(nnodes, avg, C, mode, iso, seed):
+    snd, rcv = random_graph(nnodes, avg, seed, degree_mode=mode, isolated_frac=iso)
+    E = snd.numel()
+    X, v, R, G = mp_inputs(nnodes, E, C, seed)
+    Y = O.spherical_harmonics(v) if E else torch.zeros(16, 0, dtype=torch.float64)
+    return snd, rcv, X, Y.contiguous(), R, G
+
+
+@pytest.mark.parametrize("case", MP_CASES, ids=lambda c: "N%d_d%d_C%d_%s_s%d" % (c[0], c[1], c[2], c[3], c[5]))
+def test_mp_forward(cabi, case):
+    _say("mp_forward", case)
+    nnodes = case[0]
+    snd, rcv, X, Y, R, _ = _mp_case(*case)
+    ref = O.mp_forward(X, Y, R, snd, rcv, nnodes)
+    fo = cabi.first_occurences(rcv.to(DEV), nnodes)
+    out = cabi.mp_forward(X.float().to(DEV), Y.float().to(DEV), R.float().to(DEV), snd.to(DEV), fo, nnodes)
+    close(out, ref, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("case", MP_CASES, ids=lambda c: "N%d_d%d_C%d_%s_s%d" % (c[0], c[1], c[2], c[3], c[5]))
+def test_mp_backward(cabi, case):
+    _say("mp_backward", case)
+    nnodes = case[0]
+    snd, rcv, X, Y, R, G = _mp_case(*case)
+    gX_ref, gY_ref, gR_ref = O.mp_backward(X, Y, R, G, snd, rcv)
+    d = lambda t: t.float().to(DEV)
+    fo = cabi.first_occurences(rcv.to(DEV), nnodes)
+    perm, off = cabi.stable_key_sort(snd.to(DEV), nnodes)
+    gX, gY, gR = cabi.mp_backward(d(X), d(Y), d(R), d(G), snd.to(DEV), fo, perm, off, nnodes)
+    close(gR, gR_ref, RTOL, ATOL)
+    close(gY, gY_ref, RTOL, ATOL)
+    close(gX, gX_ref, RTOL, ATOL)
+
+
+def test_mp_backward_subsets(cabi):
+    """Only the requested gradients are produced; each equals the full computation."""
+    case = (120, 20, 128, "poisson", 0.1, 21)
+    _say("mp_backward_subsets", case)
+    nnodes = case[0]
+    snd, rcv, X, Y, R, G = _mp_case(*case)
+    d = lambda t: t.float().to(DEV)
+    fo = cabi.first_occurences(rcv.to(DEV), nnodes)
+    perm, off = cabi.stable_key_sort(snd.to(DEV), nnodes)
+    full = cabi.mp_backward(d(X), d(Y), d(R), d(G), snd.to(DEV), fo, perm, off, nnodes)
+    for mask in range(1, 7):
+        need = dict(need_gX=bool(mask & 1), need_gY=bool(mask & 2), need_gR=bool(mask & 4))
+        part = cabi.mp_backward(d(X), d(Y), d(R), d(G), snd.to(DEV), fo, perm, off, nnodes, **need)
+        for got, want, on in zip(part, full, (need["need_gX"], need["need_gY"], need["need_gR"])):
+            if on:
+                assert torch.equal(got, want)
+            else:
+                assert got is None
+
+
+def test_mp_reproducible_bitwise(cabi):
+    """No atomics: two runs give identical bits."""
+    case = (256, 30, 96, "poisson", 0.0, 31)
+    nnodes = case[0]
+    snd, rcv, X, Y, R, G = _mp_case(*case)
+    d = lambda t: t.float().to(DEV)
+    fo = cabi.first_occurences(rcv.to(DEV), nnodes)
+    perm, off = cabi.stable_key_sort(snd.to(DEV), nnodes)
+    a = cabi.mp_forward(d(X), d(Y), d(R), snd.to(DEV), fo, nnodes)
+    b = cabi.mp_forward(d(X), d(Y), d(R), snd.to(DEV), fo, nnodes)
+    assert torch.equal(a, b)
+    ga = cabi.mp_backward(d(X), d(Y), d(R), d(G), snd.to(DEV), fo, perm, off, nnodes)
+    gb = cabi.mp_backward(d(X), d(Y), d(R), d(G), snd.to(DEV), fo, perm, off, nnodes)
+    for u, v in zip(ga, gb):
+        assert torch.equal(u, v)
+
+
+def test_mp_rejects_bad_arguments(cabi):
+    X = torch.zeros(4, 48, device=DEV)
+    Y = torch.zeros(16, 0, device=DEV)
+    R = torch.zeros(0, 4, 48, device=DEV)
+    snd = torch.zeros(0, dtype=torch.int32, device=DEV)
+    fo = torch.zeros(8, dtype=torch.int32, device=DEV)
+    with pytest.raises(RuntimeError, match="multiple of 32"):
+        cabi.mp_forward(X, Y, R, snd, fo, 4)
+    with pytest.raises(RuntimeError, match="GPU"):
+        cabi.mp_forward(torch.zeros(4, 32), Y, R, snd, fo, 4)
+
+
+# ------------------------------------------------------------------------------------------------
+# spherical harmonics
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("E,seed", [(1, 0), (1000, 1), (100003, 2)])
+def test_sh_forward_backward(cabi, E, seed):
+    _say("sh", E, seed)
+    g = torch.Generator().manual_seed(seed)
+    xyz = torch.randn(E, 3, generator=g, dtype=torch.float64) * 2.5
+    gY = torch.randn(16, E, generator=g, dtype=torch.float64)
+    ref = O.spherical_harmonics(xyz)
+    gref = O.spherical_harmonics_backward(xyz, gY)
+    Y = cabi.sh_forward(xyz.float().to(DEV))
+    gx = cabi.sh_backward(xyz.float().to(DEV), gY.float().to(DEV))
+    close(Y, ref, 1e-5, 2e-6)
+    close(gx, gref, 2e-5, 2e-6)
+
+
+# ------------------------------------------------------------------------------------------------
+# spline
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("E,J,seed", [(1, 128, 0), (777, 384, 1), (5000, 512, 2), (300, 768, 3)])
+def test_spline_forward_backward(cabi, E, J, seed):
+    _say("spline", E, J, seed)
+    g = torch.Generator().manual_seed(seed)
+    r_max = 5.0
+    knots_np, h = np.linspace(1e-12, r_max + 1.0, 256, retstep=True)
+    knots = torch.from_numpy(knots_np)
+    table = torch.sin(knots[:, None] * torch.linspace(0.3, 3.0, J, dtype=torch.float64)[None, :]) * torch.randn(
+        1, J, generator=g, dtype=torch.float64
+    )
+    coeffs = O.spline_coefficients(knots, table)
+    r = torch.rand(E, generator=g, dtype=torch.float64) * 5.6 + 0.4  # some beyond r_max
+    gR = torch.randn(E, J, generator=g, dtype=torch.float64)
+    # evaluate the oracle at the fp32-rounded radii the kernel sees
+    r32 = r.float()
+    val_ref, der_ref = O.spline_eval(r32.double(), knots, coeffs, float(h), r_max, deriv=True)
+    gr_ref = O.spline_backward(gR, der_ref)
+    d = lambda t: t.float().to(DEV)
+    val, der = cabi.spline_forward(d(r), d(knots), d(coeffs), float(h), r_max, want_deriv=True)
+    val_only = cabi.spline_forward(d(r), d(knots), d(coeffs), float(h), r_max)
+    gr = cabi.spline_backward(d(r), d(knots), d(coeffs), d(gR), float(h), r_max)
+    assert torch.equal(val, val_only)
+    close(val, val_ref, 2e-5, 2e-6)
+    close(der, der_ref, 2e-5, 5e-6)
+    close(gr, gr_ref, 2e-5, 5e-6)
+    assert float(val[(r32 > r_max).to(DEV)].abs().sum()) == 0.0
+
+
+# ------------------------------------------------------------------------------------------------
+# linears (fp32 MFMA)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("N,K,Nout,seed", [(1, 32, 32, 0), (33, 64, 64, 1), (1000, 128, 128, 2), (257, 96, 96, 3), (100, 192, 192, 4), (70, 256, 256, 5), (50, 64, 128, 6), (50, 160, 96, 7)])
+def test_linear(cabi, N, K, Nout, seed):
+    _say("linear", N, K, Nout, seed)
+    g = torch.Generator().manual_seed(seed)
+    X = torch.randn(N, 16, K, generator=g, dtype=torch.float64)
+    W = torch.randn(4, K, Nout, generator=g, dtype=torch.float64)
+    ref = O.linear(X, W)
+    WT = W.transpose(-1, -2).contiguous()
+    out = cabi.linear(X.float().to(DEV), WT.float().to(DEV))
+    close(out, ref, 1e-5, 2e-6)
+    # the reference's own acceptance threshold (tests/linear.py:142-143): mean abs error < 5e-5
+    assert float((out.double().cpu() - ref).abs().mean()) < 5e-5
+
+
+@pytest.mark.parametrize("N,C,ne,seed", [(1, 32, 1, 0), (500, 128, 10, 1), (333, 96, 4, 2), (64, 192, 10, 3)])
+def test_elemental_linear(cabi, N, C, ne, seed):
+    _say("elemental_linear", N, C, ne, seed)
+    g = torch.Generator().manual_seed(seed)
+    X = torch.randn(N, 16, C, generator=g, dtype=torch.float64)
+    W = torch.randn(ne, 4, C, C, generator=g, dtype=torch.float64)
+    elem = torch.randint(0, ne, (N,), generator=g)
+    one_hot = torch.nn.functional.one_hot(elem, ne).double()
+    ref = O.elemental_linear(X, W, one_hot)
+    perm, off = cabi.stable_key_sort(elem.int().to(DEV), ne)
+    WT = W.transpose(-1, -2).contiguous()
+    out = cabi.linear(X.float().to(DEV), WT.float().to(DEV), perm, off)
+    close(out, ref, 1e-5, 2e-6)
+
+
+# ------------------------------------------------------------------------------------------------
+# symmetric contraction with synthetic sparse tables
+# ------------------------------------------------------------------------------------------------
+def _random_tables(seed, n3=40, n2=10, P3=23, P2=4):
+    """Random monomial lists with 1-3 (path, value) terms each, plus the dense U they stand for."""
+    rng = np.random.default_rng(seed)
+    triples = set()
+    while len(triples) < n3:
+        triples.add(tuple(sorted(rng.integers(0, 16, 3).tolist())))
+    pairs = set()
+    while len(pairs) < n2:
+        pairs.add(tuple(sorted(rng.integers(0, 16, 2).tolist())))
+    U3 = torch.zeros(16, 16, 16, P3, dtype=torch.float64)
+    U2 = torch.zeros(16, 16, P2, dtype=torch.float64)
+    mono3, off3, path3, val3 = [], [0], [], []
+    for (i, j, k) in sorted(triples):
+        mono3.append(i | (j << 8) | (k << 16))
+        for _ in range(int(rng.integers(1, 4))):
+            p, v = int(rng.integers(0, P3)), float(rng.normal())
+            U3[i, j, k, p] += v  # the whole coefficient sits on the sorted position
+            path3.append(p)
+            val3.append(v)
+        off3.append(len(path3))
+    mono2, off2, path2, val2 = [], [0], [], []
+    for (i, j) in sorted(pairs):
+        mono2.append(i | (j << 8))
+        p, v = int(rng.integers(0, P2)), float(rng.normal())
+        U2[i, j, p] += v
+        path2.append(p)
+        val2.append(v)
+        off2.append(len(path2))
+    ti = lambda a: torch.tensor(a, dtype=torch.int32)
+    tf = lambda a: torch.tensor(a, dtype=torch.float32)
+    return U3, U2, ti(mono3), ti(off3), ti(path3), tf(val3), ti(mono2), ti(off2), ti(path2), tf(val2)
+
+
+@pytest.mark.parametrize("N,C,ne,seed", [(1, 32, 1, 0), (37, 128, 10, 1), (20, 96, 3, 2), (9, 192, 4, 3), (5, 256, 2, 4)])
+def test_symcon_synthetic_tables(cabi, N, C, ne, seed):
+    _say("symcon", N, C, ne, seed)
+    U3, U2, mono3, off3, path3, val3, mono2, off2, path2, val2 = _random_tables(seed)
+    g = torch.Generator().manual_seed(seed)
+    X = torch.randn(N, 16, C, generator=g, dtype=torch.float64)
+    W3 = torch.randn(ne, 23, C, generator=g, dtype=torch.float64)
+    W2 = torch.randn(ne, 4, C, generator=g, dtype=torch.float64)
+    W1 = torch.randn(ne, 1, C, generator=g, dtype=torch.float64)
+    types = torch.randint(0, ne, (N,), generator=g).int()
+    gout = torch.randn(N, C, generator=g, dtype=torch.float64)
+    # the oracle sees the fp32-rounded table values
+    U3r, U2r = torch.zeros_like(U3), torch.zeros_like(U2)
+    for t in range(mono3.numel()):
+        w = int(mono3[t])
+        for q in range(int(off3[t]), int(off3[t + 1])):
+            U3r[w & 255, (w >> 8) & 255, (w >> 16) & 255, int(path3[q])] += float(val3[q])
+    for t in range(mono2.numel()):
+        w = int(mono2[t])
+        for q in range(int(off2[t]), int(off2[t + 1])):
+            U2r[w & 255, (w >> 8) & 255, int(path2[q])] += float(val2[q])
+    Xa = X.clone().requires_grad_(True)
+    ref = O.symmetric_contraction(Xa, types, U3r, U2r, W3, W2, W1)
+    (ref * gout).sum().backward()
+    d = lambda t: t.to(DEV)
+    f = lambda t: t.float().to(DEV)
+    T3, T2, T1 = cabi.symcon_tables(d(off3), d(path3), d(val3), d(off2), d(path2), d(val2), f(W3), f(W2), f(W1))
+    perm, offs = cabi.stable_key_sort(d(types), ne)
+    out, grad = cabi.symcon_forward(f(X), perm, offs, d(mono3), d(mono2), T3, T2, T1)
+    out_nograd, none = cabi.symcon_forward(f(X), perm, offs, d(mono3), d(mono2), T3, T2, T1, want_grad=False)
+    gX = cabi.symcon_backward(grad, f(gout))
+    assert none is None and torch.equal(out, out_nograd)
+    close(out, ref.detach(), 3e-5, 3e-6)
+    close(gX, Xa.grad, 3e-5, 3e-6)

@@ -1,0 +1,197 @@
+"""Pins of the CPU oracle against closed forms, library routines and brute force (no GPU).
+
+A wrong sign, index, transposed operand or dropped term in oracle/ops.py fails at least one of
+these; none of them re-types the oracle's own formula.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ops as O
+from tests.util import mp_inputs, random_graph
+
+torch.set_default_dtype(torch.float64)
+
+
+# ---- index kernels -------------------------------------------------------------------------------
+def test_first_occurences_brute_force():
+    recv = torch.tensor([0, 0, 2, 2, 2, 5], dtype=torch.int32)
+    fo = O.first_occurences(recv, 7)
+    assert fo[:7].tolist() == [0, 2, 2, 5, 5, 5, 6]
+    assert fo[7:].tolist() == [2, 2, 5, 5, 5, 6, 6]
+    for n in range(7):  # python scan
+        idx = [e for e in range(6) if recv[e] == n]
+        if idx:
+            assert fo[n] == idx[0] and fo[7 + n] == idx[-1] + 1
+        else:
+            assert fo[n] == fo[7 + n]
+    assert O.first_occurences(torch.zeros(0, dtype=torch.int32), 3).tolist() == [0] * 6
+
+
+def test_stable_key_sort_matches_torch_sort():
+    keys = torch.from_numpy(np.random.default_rng(0).integers(0, 13, 500).astype(np.int32))
+    perm, off = O.stable_key_sort(keys, 13)
+    _, ref = torch.sort(keys.long(), stable=True)
+    assert torch.equal(perm.long(), ref)
+    assert off[0] == 0 and off[-1] == 500
+    for k in range(13):
+        assert int(off[k + 1] - off[k]) == int((keys == k).sum())
+
+
+# ---- message passing ---------------------------------------------------------------------------------
+def test_mp_forward_brute_force_loops():
+    """Python loops over edges on a tiny non-symmetric multigraph with an isolated node."""
+    N, C = 5, 3
+    sender = torch.tensor([1, 1, 4, 0, 2, 2], dtype=torch.int32)  # duplicate edge 1->0
+    receiver = torch.tensor([0, 0, 0, 2, 3, 3], dtype=torch.int32)  # node 1 and 4 receive nothing
+    X, v, R, _ = mp_inputs(N, 6, C, 0)
+    Y = torch.randn(16, 6)
+    out = O.mp_forward(X, Y, R, sender, receiver, N)
+    ref = torch.zeros(N, 16, C)
+    for e in range(6):
+        for m in range(16):
+            l = int(math.floor(math.sqrt(m)))
+            for c in range(C):
+                ref[receiver[e], m, c] += X[sender[e], c] * Y[m, e] * R[e, l, c]
+    torch.testing.assert_close(out, ref)
+    assert float(out[1].abs().sum()) == 0.0 and float(out[4].abs().sum()) == 0.0
+
+
+def test_mp_backward_is_autograd_of_forward():
+    snd, rcv = random_graph(40, 5, 3, isolated_frac=0.2)
+    X, v, R, G = mp_inputs(40, snd.numel(), 8, 3)
+    Y = torch.randn(16, snd.numel())
+    Xa, Ya, Ra = (t.clone().requires_grad_(True) for t in (X, Y, R))
+    (O.mp_forward(Xa, Ya, Ra, snd, rcv, 40) * G).sum().backward()
+    gX, gY, gR = O.mp_backward(X, Y, R, G, snd, rcv)
+    torch.testing.assert_close(gX, Xa.grad)
+    torch.testing.assert_close(gY, Ya.grad)
+    torch.testing.assert_close(gR, Ra.grad)
+
+
+# ---- spherical harmonics -------------------------------------------------------------------------------
+def test_sh_against_scipy_closed_form():
+    """sqrt(4 pi) x real harmonics built from scipy's complex ones, without Condon-Shortley sign:
+    m=0: Re;  m>0: sqrt2 (-1)^m Re;  m<0: sqrt2 (-1)^m Im, on (x,y,z) = (in2, in0, in1)."""
+    from scipy.special import sph_harm_y
+
+    xyz = torch.randn(200, 3) * 3.0
+    out = O.spherical_harmonics(xyz).numpy()
+    v = (xyz / xyz.norm(dim=1, keepdim=True)).numpy()
+    x, y, z = v[:, 2], v[:, 0], v[:, 1]
+    theta, phi = np.arccos(np.clip(z, -1, 1)), np.arctan2(y, x)
+    row = 0
+    for l in range(4):
+        for m in range(-l, l + 1):
+            c = sph_harm_y(l, abs(m), theta, phi)
+            if m == 0:
+                val = c.real
+            elif m > 0:
+                val = math.sqrt(2) * (-1) ** m * c.real
+            else:
+                val = math.sqrt(2) * (-1) ** m * c.imag
+            np.testing.assert_allclose(out[row], math.sqrt(4 * math.pi) * val, atol=1e-12)
+            row += 1
+
+
+def test_sh_sum_rule_and_l1():
+    xyz = torch.randn(50, 3)
+    Y = O.spherical_harmonics(xyz)
+    for l in range(4):
+        torch.testing.assert_close((Y[l * l:(l + 1) ** 2] ** 2).sum(0), torch.full((50,), 2.0 * l + 1))
+    torch.testing.assert_close(Y[1:4].t(), math.sqrt(3) * xyz / xyz.norm(dim=1, keepdim=True))
+
+
+def test_sh_parity_and_scale_invariance():
+    xyz = torch.randn(20, 3)
+    Y, Ym, Ys = O.spherical_harmonics(xyz), O.spherical_harmonics(-xyz), O.spherical_harmonics(3.7 * xyz)
+    sign = torch.tensor([(-1.0) ** int(math.isqrt(m)) for m in range(16)])[:, None]
+    torch.testing.assert_close(Ym, sign * Y)
+    torch.testing.assert_close(Ys, Y)
+
+
+def test_sh_backward_finite_differences_and_radial_null():
+    xyz = torch.randn(10, 3) + 0.5
+    g = torch.randn(16, 10)
+    gx = O.spherical_harmonics_backward(xyz, g)
+    h = 1e-6
+    for k in range(3):
+        d = torch.zeros(10, 3)
+        d[:, k] = h
+        fd = ((O.spherical_harmonics(xyz + d) - O.spherical_harmonics(xyz - d)) * g).sum(0) / (2 * h)
+        torch.testing.assert_close(gx[:, k], fd, rtol=1e-6, atol=1e-7)
+    # homogeneous of degree 0: the gradient has no radial component
+    torch.testing.assert_close((gx * xyz).sum(1), torch.zeros(10), atol=1e-12, rtol=0)
+
+
+# ---- spline ---------------------------------------------------------------------------------------------
+def test_spline_against_scipy_and_boundary_conditions():
+    from scipy.interpolate import CubicSpline
+
+    knots_np, h = np.linspace(1e-12, 6.0, 256, retstep=True)
+    knots = torch.from_numpy(knots_np)
+    table = torch.stack([torch.sin(knots * 1.3), torch.exp(-knots), knots ** 2, torch.cos(3 * knots)], dim=1)
+    co = O.spline_coefficients(knots, table)
+    assert co.shape == (255, 4, 4)
+    torch.testing.assert_close(co[:, 0], table[:-1])  # a_k = y_k
+    torch.testing.assert_close(co[0, 2], torch.zeros(4), atol=1e-9, rtol=0)  # natural: c_0 = 0
+    r = torch.rand(300) * 5.9
+    val, der = O.spline_eval(r, knots, co, float(h), 5.0, deriv=True)
+    cs = CubicSpline(knots_np, table.numpy(), bc_type="natural")
+    inside = (r <= 5.0).numpy()
+    np.testing.assert_allclose(val.numpy()[inside], cs(r.numpy())[inside], atol=1e-10)
+    np.testing.assert_allclose(der.numpy()[inside], cs(r.numpy(), 1)[inside], atol=1e-9)
+    assert float(val[~torch.from_numpy(inside)].abs().sum()) == 0.0
+    # interpolates a smooth function to O(h^4)
+    np.testing.assert_allclose(val[:, 0].numpy()[inside], np.sin(1.3 * r.numpy())[inside], atol=1e-6)
+    torch.testing.assert_close(O.spline_backward(torch.ones(300, 4), der), der.sum(1))
+
+
+# ---- linears ---------------------------------------------------------------------------------------------
+def test_linear_loops():
+    X = torch.randn(3, 16, 4)
+    W = torch.randn(4, 4, 5)
+    out = O.linear(X, W)
+    for n in range(3):
+        for m in range(16):
+            l = math.isqrt(m)
+            torch.testing.assert_close(out[n, m], X[n, m] @ W[l] / 2.0)
+    Wel = torch.randn(3, 4, 4, 5)
+    one_hot = torch.tensor([[0., 1, 0], [1, 0, 0], [0, 0, 0]])
+    oe = O.elemental_linear(X, Wel, one_hot)
+    torch.testing.assert_close(oe[0], O.linear(X[:1], Wel[1])[0])
+    torch.testing.assert_close(oe[1], O.linear(X[1:2], Wel[0])[0])
+    assert float(oe[2].abs().sum()) == 0.0
+
+
+# ---- symmetric contraction ----------------------------------------------------------------------------
+def test_symmetric_contraction_brute_force():
+    N, C, ne = 3, 2, 2
+    U3 = torch.zeros(16, 16, 16, 5)
+    U2 = torch.zeros(16, 16, 3)
+    rng = np.random.default_rng(0)
+    for _ in range(30):
+        i, j, k = rng.integers(0, 16, 3)
+        U3[i, j, k, rng.integers(0, 5)] = rng.normal()
+    for _ in range(10):
+        i, j = rng.integers(0, 16, 2)
+        U2[i, j, rng.integers(0, 3)] = rng.normal()
+    X = torch.randn(N, 16, C)
+    W3, W2, W1 = torch.randn(ne, 5, C), torch.randn(ne, 3, C), torch.randn(ne, 1, C)
+    types = torch.tensor([1, 0, 1])
+    out = O.symmetric_contraction(X, types, U3, U2, W3, W2, W1)
+    ref = torch.zeros(N, C)
+    nz3 = U3.nonzero().tolist()
+    nz2 = U2.nonzero().tolist()
+    for n in range(N):
+        e = int(types[n])
+        for c in range(C):
+            s = W1[e, 0, c] * X[n, 0, c]
+            for (i, j, k, p) in nz3:
+                s += U3[i, j, k, p] * W3[e, p, c] * X[n, i, c] * X[n, j, c] * X[n, k, c]
+            for (i, j, p) in nz2:
+                s += U2[i, j, p] * W2[e, p, c] * X[n, i, c] * X[n, j, c]
+            ref[n, c] = s
+    torch.testing.assert_close(out, ref)
