@@ -1,6 +1,6 @@
 // Channel-mixing linear layers on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
 //
-//   OUT[n, m, :] = X[n, m, :] . W[g(n)][l(m)] / sqrt(K)
+//   OUT[n, m, :] = scale * X[n, m, :] . W[g(n)][l(m)]      (scale = 1/sqrt(K) in the model)
 //
 // One wavefront owns a tile of 32 nodes x one component m x all Nout columns, so every row of the
 // tile uses the same K x Nout weight block.  The X rows of the tile (K contiguous floats each) are
@@ -128,10 +128,10 @@ __global__ __launch_bounds__(kWave) void linear_kernel(const float *__restrict__
 
 template <int NT>
 int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
-           int K, float *OUT, hipStream_t st) {
+           int K, float scale, float *OUT, hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
   hipLaunchKernelGGL(linear_kernel<NT>, dim3(static_cast<unsigned>(tiles), 16), dim3(kWave), 0, st, X, WT, perm, offs,
-                     static_cast<int>(nnodes), ngroups, K, 1.0f / std::sqrt(static_cast<float>(K)), OUT);
+                     static_cast<int>(nnodes), ngroups, K, scale, OUT);
   return check_launch("cm_linear");
 }
 
@@ -139,7 +139,7 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
 }  // namespace cm
 
 extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_perm, const int32_t *group_offsets,
-                         int64_t nnodes, int ngroups, int K, int Nout, float *OUT, cm_stream_t stream) {
+                         int64_t nnodes, int ngroups, int K, int Nout, float scale, float *OUT, cm_stream_t stream) {
   CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 16, "cm_linear: nnodes out of range");
   CM_REQUIRE(K >= 32 && K <= 256 && K % 32 == 0, "cm_linear: K=%d must be a multiple of 32 in [32, 256]", K);
   CM_REQUIRE(Nout >= 32 && Nout <= 256 && Nout % 32 == 0, "cm_linear: Nout=%d must be a multiple of 32 in [32, 256]", Nout);
@@ -150,14 +150,14 @@ extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_p
   CM_REQUIRE(X && W_T && OUT, "cm_linear: NULL pointer");
   hipStream_t st = cm::as_stream(stream);
   switch (Nout / 32) {
-    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
-    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
-    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
-    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
-    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
-    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
-    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
-    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, OUT, st);
+    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
+    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
+    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
+    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
+    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
+    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
+    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
+    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
   }
   return CM_EINVAL;
 }

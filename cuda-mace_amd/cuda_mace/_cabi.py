@@ -42,7 +42,7 @@ SIGNATURES = {
     "cm_sh_backward": (_i32, [_p, _p, _i64, _p, _p]),
     "cm_spline_forward": (_i32, [_p, _p, _p, _i64, _i32, _i32, _f32, _f32, _p, _p, _p]),
     "cm_spline_backward": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _f32, _f32, _p, _p]),
-    "cm_linear": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _p, _p]),
+    "cm_linear": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _f32, _p, _p]),
     "cm_symcon_tables": (_i32, [_p, _p, _p, _i32, _p, _p, _p, _i32, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _p, _p, _p]),
     "cm_symcon_forward": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
     "cm_symcon_backward": (_i32, [_p, _p, _i64, _i32, _p, _p]),
@@ -193,8 +193,8 @@ def spline_backward(r, r_knots, coeffs, grad_R, r_width: float, r_max: float) ->
 
 
 # ---- linears ------------------------------------------------------------------------------------------
-def linear(X, W_T, node_perm=None, group_offsets=None) -> torch.Tensor:
-    """X [N,16,K]; W_T [4,N',K] or [ngroups,4,N',K] (transposed weight blocks)."""
+def linear(X, W_T, node_perm=None, group_offsets=None, scale=None) -> torch.Tensor:
+    """X [N,16,K]; W_T [4,N',K] or [ngroups,4,N',K] (transposed weight blocks); scale defaults to 1/sqrt(K)."""
     if W_T.dim() == 3:
         W_T = W_T.unsqueeze(0)
     ngroups, four, Nout, K = W_T.shape
@@ -206,7 +206,8 @@ def linear(X, W_T, node_perm=None, group_offsets=None) -> torch.Tensor:
     _check(
         lib.cm_linear(
             _dev(X, F32, "X"), _dev(W_T, F32, "W_T"), _dev(node_perm, I32, "node_perm"),
-            _dev(group_offsets, I32, "group_offsets"), N, ngroups, K, Nout, _dev(OUT, F32, "OUT"), _stream(),
+            _dev(group_offsets, I32, "group_offsets"), N, ngroups, K, Nout,
+            float(scale) if scale is not None else 1.0 / float(K) ** 0.5, _dev(OUT, F32, "OUT"), _stream(),
         )
     )
     return OUT

@@ -1,0 +1,272 @@
+"""OptimizedInvariantMACE: an invariant MACE model whose hot path runs on the gfx950 HIP kernels.
+
+Drop-in for the reference's cuda_mace/models/InvariantMACE.py: same class names, same constructor
+argument (an upstream-like model object whose attribute tree is read, see :168-244 there), same
+`forward(data, training, compute_force, compute_virials, compute_stress, compute_displacement)` and the
+same output dictionary (:366-377).  The pieces the reference borrows from upstream `mace`
+(`scatter_sum`, `get_edge_vectors_and_lengths`, `get_outputs`, `get_symmetric_displacement`) are small
+torch functions here, because upstream is not a dependency.
+"""
+from __future__ import annotations
+
+from copy import deepcopy
+from math import sqrt
+from typing import Dict, Optional, Tuple
+
+import numpy as np
+import torch
+
+from cuda_mace.ops.cubic_spline import CubicSpline
+from cuda_mace.ops.invariant_message_passing import InvariantMessagePassingTP
+from cuda_mace.ops.linear import ElementalLinear, Linear
+from cuda_mace.ops.spherical_harmonics import SphericalHarmonics
+from cuda_mace.ops.symmetric_contraction import SymmetricContraction as CUDAContraction
+from cuda_mace.utils.irreps import Instruction
+
+
+# ---- the few upstream helpers the forward needs ------------------------------------------------------
+def scatter_sum(src: torch.Tensor, index: torch.Tensor, dim: int = -1, dim_size: Optional[int] = None) -> torch.Tensor:
+    dim = dim % src.dim()
+    size = list(src.shape)
+    size[dim] = int(dim_size) if dim_size is not None else int(index.max()) + 1
+    out = torch.zeros(size, dtype=src.dtype, device=src.device)
+    return out.index_add_(dim, index, src)
+
+
+def get_edge_vectors_and_lengths(positions, edge_index, shifts) -> Tuple[torch.Tensor, torch.Tensor]:
+    """vectors = positions[edge_index[1]] - positions[edge_index[0]] + shifts (upstream convention)."""
+    vectors = positions[edge_index[1]] - positions[edge_index[0]] + shifts
+    return vectors, torch.linalg.norm(vectors, dim=-1, keepdim=True)
+
+
+def get_symmetric_displacement(positions, unit_shifts, cell, edge_index, num_graphs, batch):
+    """Applies a symmetric strain (zero, but differentiable) to positions and cell so that
+    d energy / d displacement gives the virial."""
+    if cell is None:
+        cell = torch.zeros(num_graphs * 3, 3, dtype=positions.dtype, device=positions.device)
+    sender = edge_index[0]
+    displacement = torch.zeros((num_graphs, 3, 3), dtype=positions.dtype, device=positions.device)
+    displacement.requires_grad_(True)
+    symmetric = 0.5 * (displacement + displacement.transpose(-1, -2))
+    positions = positions + torch.einsum("be,bec->bc", positions, symmetric[batch])
+    cell = cell.view(-1, 3, 3)
+    cell = cell + torch.matmul(cell, symmetric)
+    shifts = torch.einsum("be,bec->bc", unit_shifts, cell[batch[sender]])
+    return positions, shifts, displacement, cell
+
+
+def get_outputs(energy, positions, displacement, cell, training=False, compute_force=True, compute_virials=False,
+                compute_stress=False):
+    """forces = -dE/dpositions; virials = -dE/ddisplacement; stress = -virials / volume."""
+    forces = virials = stress = None
+    grad_outputs = [torch.ones_like(energy)]
+    want_virials = compute_virials or compute_stress
+    if compute_force and want_virials:
+        gp, gd = torch.autograd.grad([energy], [positions, displacement], grad_outputs=grad_outputs,
+                                     retain_graph=training, create_graph=training, allow_unused=True)
+        forces = -gp
+        virials = -gd if gd is not None else torch.zeros_like(displacement)
+    elif compute_force:
+        (gp,) = torch.autograd.grad([energy], [positions], grad_outputs=grad_outputs, retain_graph=training,
+                                    create_graph=training, allow_unused=True)
+        forces = -gp if gp is not None else torch.zeros_like(positions)
+    if compute_stress and virials is not None and cell is not None:
+        cell3 = cell.view(-1, 3, 3)
+        volume = torch.linalg.det(cell3).abs().view(-1, 1, 1)
+        stress = -virials / volume
+    return forces, virials, stress, None, None
+
+
+# ---- model pieces -----------------------------------------------------------------------------------------
+class SymmetricContractionWrapper(torch.nn.Module):
+    def __init__(self, symmetric_contractions):
+        super().__init__()
+        self.symmetric_contractions = symmetric_contractions
+
+    def forward(self, x, y):
+        # y: one-hot [nnodes, nelements] as upstream passes it, or already the int32 element index
+        if y.dim() == 2:
+            y = y.argmax(dim=-1).int()
+        return self.symmetric_contractions(x, y).squeeze(1)
+
+
+class linear_matmul(torch.nn.Module):
+    """x @ W / sqrt(fan_in) for scalar features, from an e3nn-Linear-like module (reference :41-53)."""
+
+    def __init__(self, linear_e3nn):
+        super().__init__()
+        n_in = linear_e3nn.__dict__["irreps_in"].num_irreps
+        n_out = linear_e3nn.__dict__["irreps_out"].num_irreps
+        self.register_buffer("weights", (linear_e3nn.weight.data.reshape(n_in, n_out) / n_in ** 0.5).float())
+
+    def forward(self, x):
+        return torch.matmul(x, self.weights)
+
+
+def element_linear_to_cuda(skip_tp):
+    """Per-element, per-l weight blocks of the first layer's skip tensor product (reference :56-74)."""
+    num_elements = skip_tp.__dict__["irreps_in2"].dim
+    n_channels = skip_tp.__dict__["irreps_in1"][0].dim
+    lmax = skip_tp.__dict__["irreps_in1"].lmax
+    ws = skip_tp.weight.data.float().reshape([lmax + 1, n_channels, num_elements, n_channels]).permute(2, 0, 1, 3)
+    ws = ws.flatten(1) / sqrt(num_elements)
+    instructions = [Instruction(l, l, (n_channels, n_channels), 1.0 / sqrt(n_channels)) for l in range(lmax + 1)]
+    return ElementalLinear(skip_tp.__dict__["irreps_in1"], skip_tp.__dict__["irreps_out"], instructions, ws, num_elements)
+
+
+class _FloatLinearView:
+    """Presents an e3nn-Linear-like module with fp32 weights without converting the module in place."""
+
+    def __init__(self, linear):
+        self.irreps_in, self.irreps_out = linear.irreps_in, linear.irreps_out
+        self.instructions = linear.instructions
+        self.weight = linear.weight.data.float()
+
+
+class InvariantInteraction(torch.nn.Module):
+    """First layer: linear_up, message passing, per-l linear, per-element linear."""
+
+    def __init__(self, mace_model):
+        super().__init__()
+        inter = mace_model.interactions[0]
+        self.linear_up = linear_matmul(inter.linear_up)
+        self.linear = Linear(_FloatLinearView(inter.linear))
+        self.tp = InvariantMessagePassingTP()
+        self.skip_tp = element_linear_to_cuda(inter.skip_tp)
+        self.avg_num_neighbors = inter.avg_num_neighbors
+
+    def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None):
+        if sender is None:
+            sender, receiver = edge_index[1].int(), edge_index[0].int()
+        node_feats = self.linear_up(node_feats)
+        message = self.tp.forward(node_feats, edge_attrs, edge_feats.view(edge_feats.shape[0], -1, node_feats.shape[-1]),
+                                  sender, receiver, node_feats.shape[0])
+        message = self.linear(message) / self.avg_num_neighbors
+        message = self.skip_tp(message, node_attrs)
+        return message, None
+
+
+class InvariantResidualInteraction(torch.nn.Module):
+    """Second layer: residual skip connection on the scalar features, linear_up, message passing, per-l linear."""
+
+    def __init__(self, mace_model):
+        super().__init__()
+        inter = mace_model.interactions[1]
+        self.linear_up = linear_matmul(inter.linear_up)
+        self.linear = Linear(_FloatLinearView(inter.linear))
+        self.tp = InvariantMessagePassingTP()
+        self.skip_tp = deepcopy(inter.skip_tp).float()
+        self.avg_num_neighbors = inter.avg_num_neighbors
+
+    def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None):
+        if sender is None:
+            sender, receiver = edge_index[1].int(), edge_index[0].int()
+        sc = self.skip_tp(node_feats, node_attrs)
+        node_feats = self.linear_up(node_feats)
+        message = self.tp.forward(node_feats, edge_attrs, edge_feats.view(edge_feats.shape[0], -1, node_feats.shape[-1]),
+                                  sender, receiver, node_feats.shape[0])
+        message = self.linear(message) / self.avg_num_neighbors
+        return message, sc
+
+
+class OptimizedInvariantMACE(torch.nn.Module):
+    def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256):
+        super().__init__()
+        assert int(mace_model.num_interactions) == 2, "exactly two interaction layers are supported"
+        self.register_buffer("atomic_numbers", deepcopy(mace_model.atomic_numbers))
+        self.register_buffer("r_max", deepcopy(mace_model.r_max))
+        self.register_buffer("num_interactions", deepcopy(mace_model.num_interactions))
+
+        self.node_embedding = deepcopy(mace_model.node_embedding)
+        self.radial_embedding = deepcopy(mace_model.radial_embedding)
+        self.spherical_harmonics = SphericalHarmonics()
+        self.atomic_energies_fn = deepcopy(mace_model.atomic_energies_fn)
+
+        self.interactions = torch.nn.ModuleList([InvariantInteraction(mace_model), InvariantResidualInteraction(mace_model)])
+        self.products = deepcopy(mace_model.products)
+        self.readouts = deepcopy(mace_model.readouts).to(torch.float64)
+
+        for i in range(int(mace_model.num_interactions)):
+            contraction = CUDAContraction(mace_model.products[i].symmetric_contractions, device=device)
+            self.products[i].symmetric_contractions = SymmetricContractionWrapper(contraction)
+            self.products[i].linear = linear_matmul(mace_model.products[i].linear)
+
+        # tabulate R(r) = conv_tp_weights(radial_embedding(r)) of each layer in fp64, spline it in fp32
+        r_np, h = np.linspace(1e-12, float(self.r_max) + 1.0, num_spline_knots, retstep=True)
+        r = torch.tensor(r_np, dtype=torch.float64)
+        with torch.no_grad():
+            radial = deepcopy(mace_model.radial_embedding).double().cpu()
+            bessel_j = radial(r.unsqueeze(-1), None, None, None)
+            if isinstance(bessel_j, tuple):
+                bessel_j = bessel_j[0]
+            edge_splines = []
+            for interaction in mace_model.interactions:
+                R = deepcopy(interaction.conv_tp_weights).double().cpu()(bessel_j)
+                edge_splines.append(CubicSpline(r.float(), R.float(), float(h), float(self.r_max)))
+        self.edge_splines = torch.nn.ModuleList(edge_splines)
+
+        self.scale_shift = deepcopy(mace_model.scale_shift).double()
+        self.orig_model = mace_model
+        self.to(device)
+
+    def forward(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
+                compute_virials: bool = False, compute_stress: bool = False,
+                compute_displacement: bool = False) -> Dict[str, Optional[torch.Tensor]]:
+        data["positions"].requires_grad_(True)
+        positions = data["positions"]
+        node_attrs = data["node_attrs"]
+        batch = data["batch"]
+        node_heads = data["head"][batch] if "head" in data else torch.zeros_like(batch)
+        num_atoms_arange = torch.arange(positions.shape[0], device=positions.device)
+        num_graphs = data["ptr"].numel() - 1
+        shifts = data["shifts"]
+        cell = data.get("cell")
+
+        displacement = torch.zeros((num_graphs, 3, 3), dtype=positions.dtype, device=positions.device)
+        if compute_virials or compute_stress or compute_displacement:
+            positions, shifts, displacement, cell = get_symmetric_displacement(
+                positions=positions, unit_shifts=data["unit_shifts"], cell=cell, edge_index=data["edge_index"],
+                num_graphs=num_graphs, batch=batch)
+
+        node_e0 = self.atomic_energies_fn(node_attrs.double())[num_atoms_arange, node_heads]
+        e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs)
+        node_feats = self.node_embedding(node_attrs.double())
+
+        vectors, lengths = get_edge_vectors_and_lengths(positions=positions, edge_index=data["edge_index"], shifts=shifts)
+        edge_attrs = self.spherical_harmonics.forward(vectors.float())
+        lengths32 = lengths.squeeze(-1).float()
+
+        # index structures shared by both layers: one int32 copy of the edge lists (their CSR offsets and
+        # sender-sorted view are cached on these tensor objects) and one element index per node
+        receiver = data["edge_index"][0].int()
+        sender = data["edge_index"][1].int()
+        node_attrs32 = node_attrs.float()
+        atom_types = node_attrs.argmax(dim=-1).int()
+
+        node_es_list, node_feats_list = [], []
+        for interaction, product, readout, edge_spline in zip(self.interactions, self.products, self.readouts, self.edge_splines):
+            edge_feats = edge_spline.forward(lengths32)
+            node_feats, sc = interaction(node_attrs=node_attrs32, node_feats=node_feats.float(), edge_attrs=edge_attrs,
+                                         edge_feats=edge_feats, edge_index=data["edge_index"], sender=sender,
+                                         receiver=receiver)
+            node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types).double()
+            node_feats_list.append(node_feats)
+            node_es_list.append(readout(node_feats, node_heads)[num_atoms_arange, node_heads])
+
+        node_feats_out = torch.cat(node_feats_list, dim=-1)
+        node_inter_es = torch.sum(torch.stack(node_es_list, dim=0), dim=0)
+        node_inter_es = self.scale_shift(node_inter_es, node_heads)
+        inter_e = scatter_sum(src=node_inter_es.double(), index=batch, dim=-1, dim_size=num_graphs)
+
+        total_energy = e0 + inter_e
+        node_energy = node_e0 + node_inter_es
+
+        forces, virials, stress, hessian, edge_forces = get_outputs(
+            energy=inter_e, positions=data["positions"], displacement=displacement, cell=cell, training=training,
+            compute_force=compute_force, compute_virials=compute_virials, compute_stress=compute_stress)
+
+        return {
+            "energy": total_energy, "node_energy": node_energy, "interaction_energy": inter_e, "forces": forces,
+            "virials": virials, "stress": stress, "hessian": hessian, "displacement": displacement,
+            "node_feats": node_feats_out, "edge_forces": edge_forces,
+        }

@@ -1,0 +1,20 @@
+import torch
+
+from . import classes
+
+
+class InvariantMessagePassingTP(torch.nn.Module):
+    """out[n, m, c] = sum over edges received by n of node_feats[sender, c] * edge_attrs[m, e] * tp_weights[e, l(m), c].
+
+    Same module name and call signature as the reference (ops/invariant_message_passing.py:3-22).
+    Shapes as the kernels take them: node_feats [nnodes, C], edge_attrs [16, nedges] (the reference's
+    comment says [nedges, 16]; its kernels index [16, nedges]), tp_weights [nedges, 4, C], both edge
+    lists int32 with receiver_list non-decreasing; returns [nnodes, 16, C].
+    """
+
+    def __init__(self):
+        super().__init__()
+        self.cuda_obj = classes.inv_message_passing.InvariantMessagePassingTP()
+
+    def forward(self, node_feats, edge_attrs, tp_weights, sender_list, receiver_list, nnodes):
+        return self.cuda_obj.forward(node_feats, edge_attrs, tp_weights, sender_list, receiver_list, int(nnodes))

@@ -126,7 +126,9 @@ int cm_spline_backward(const float *r, const float *r_knots, const float *coeffs
                        float r_width, float r_max, float *grad_r, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
- * Channel-mixing linear layers on fp32 MFMA: OUT[n, m, :] = X[n, m, :] . W[g(n)][l(m)] / sqrt(K).
+ * Channel-mixing linear layers on fp32 MFMA: OUT[n, m, :] = scale * X[n, m, :] . W[g(n)][l(m)].
+ * The reference hard-codes scale = 1/sqrt(K) (cuda/src/linear_impl.cu:33), also in the backward, where
+ * that is the true gradient only for square layers; here the caller passes the factor.
  * Replaces jit_linear and jit_elemental_linear (jit_wrappers/src/linear_wrapper.cpp:23-95, 97-191) and
  * linear_kernel_ptr / elemental_linear_kernel_ptr (cuda/src/linear_impl.cu:16-133, 134-255).
  *   X [nnodes, 16, K]; OUT [nnodes, 16, Nout];
@@ -141,7 +143,7 @@ int cm_spline_backward(const float *r, const float *r_knots, const float *coeffs
  */
 int cm_linear(const float *X, const float *W_T, const int32_t *node_perm,
               const int32_t *group_offsets, int64_t nnodes, int ngroups, int K, int Nout,
-              float *OUT, cm_stream_t stream);
+              float scale, float *OUT, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Symmetric contraction, correlation 3, scalar (L = 0) output, with its analytic gradient.

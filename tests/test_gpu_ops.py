@@ -193,7 +193,9 @@ def test_spline_forward_backward(cabi, E, J, seed):
     assert torch.equal(val, val_only)
     close(val, val_ref, 2e-5, 2e-6)
     close(der, der_ref, 2e-5, 5e-6)
-    close(gr, gr_ref, 2e-5, 5e-6)
+    # a sum of J signed terms: the error bound scales with the sum of their magnitudes
+    bound = 2e-6 * (gR.abs() * der_ref.abs()).sum(-1) + 1e-30
+    assert bool(((gr.double().cpu() - gr_ref).abs() <= bound).all())
     assert float(val[(r32 > r_max).to(DEV)].abs().sum()) == 0.0
 
 

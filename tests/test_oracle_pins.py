@@ -12,7 +12,14 @@ import torch
 from oracle import ops as O
 from tests.util import mp_inputs, random_graph
 
-torch.set_default_dtype(torch.float64)
+
+
+@pytest.fixture(autouse=True)
+def _fp64_default():
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float64)
+    yield
+    torch.set_default_dtype(old)
 
 
 # ---- index kernels -------------------------------------------------------------------------------
