@@ -29,6 +29,9 @@ def scatter_sum(src: torch.Tensor, index: torch.Tensor, dim: int = -1, dim_size:
     dim = dim % src.dim()
     size = list(src.shape)
     size[dim] = int(dim_size) if dim_size is not None else int(index.max()) + 1
+    if size[dim] == 1:
+        # single graph: a plain reduction, whose summation order does not vary from run to run
+        return src.sum(dim=dim, keepdim=True)
     out = torch.zeros(size, dtype=src.dtype, device=src.device)
     return out.index_add_(dim, index, src)
 
@@ -206,8 +209,15 @@ class OptimizedInvariantMACE(torch.nn.Module):
         self.edge_splines = torch.nn.ModuleList(edge_splines)
 
         self.scale_shift = deepcopy(mace_model.scale_shift).double()
-        self.orig_model = mace_model
         self.to(device)
+        # inference model: the custom ops differentiate with respect to features and geometry only, so no weight
+        # needs a gradient; frozen weights also let autograd skip dX of the first layer, whose input depends on
+        # the species alone
+        for p in self.parameters():
+            p.requires_grad_(False)
+        # kept for reference like upstream does, but not as a registered sub-module: moving or casting the
+        # optimised model must not touch the caller's original model
+        object.__setattr__(self, "orig_model", mace_model)
 
     def forward(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
                 compute_virials: bool = False, compute_stress: bool = False,
