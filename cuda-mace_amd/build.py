@@ -20,7 +20,7 @@ OBJ_DIR = os.path.join(HERE, "build")
 LIB_DIR = os.path.join(HERE, "cuda_mace", "lib")
 LIB_NAME = "libcuda_mace_hip.so"
 
-SOURCES = ["error.cpp", "mp.hip", "sort.hip", "sh.hip", "spline.hip", "linear.hip", "symcon.hip"]
+SOURCES = ["error.cpp", "mp.hip", "sort.hip", "sh.hip", "geometry.hip", "spline.hip", "linear.hip", "symcon.hip"]
 
 HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 

@@ -38,6 +38,8 @@ SIGNATURES = {
     "cm_stable_key_sort": (_i32, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "cm_mp_forward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _p, _p]),
     "cm_mp_backward": (_i32, [_p] * 8 + [_i64, _i64, _i32] + [_p] * 5),
+    "cm_edge_geometry_forward": (_i32, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p]),
+    "cm_edge_geometry_backward": (_i32, [_p] * 9 + [_i64, _i64, _p, _p, _p]),
     "cm_sh_forward": (_i32, [_p, _i64, _p, _p]),
     "cm_sh_backward": (_i32, [_p, _p, _i64, _p, _p]),
     "cm_spline_forward": (_i32, [_p, _p, _p, _i64, _i32, _i32, _f32, _f32, _p, _p, _p]),
@@ -159,6 +161,43 @@ def sh_backward(xyz: torch.Tensor, grad_Y: torch.Tensor) -> torch.Tensor:
     g = torch.empty(E, 3, dtype=F32, device=xyz.device)
     _check(lib.cm_sh_backward(_dev(xyz, F32, "xyz"), _dev(grad_Y, F32, "grad_Y"), E, _dev(g, F32, "grad_xyz"), _stream()))
     return g
+
+
+# ---- edge geometry ------------------------------------------------------------------------------
+F64 = torch.float64
+
+
+def edge_geometry_forward(positions, row_a, row_b, shifts):
+    E = row_a.numel()
+    dev = positions.device
+    vec = torch.empty(E, 3, dtype=F32, device=dev)
+    length = torch.empty(E, dtype=F32, device=dev)
+    _check(
+        lib.cm_edge_geometry_forward(
+            _dev(positions, F64, "positions"), _dev(row_a, I32, "row_a"), _dev(row_b, I32, "row_b"),
+            _dev(shifts, F64, "shifts"), positions.shape[0], E, _dev(vec, F32, "vectors"), _dev(length, F32, "lengths"), _stream(),
+        )
+    )
+    return vec, length
+
+
+def edge_geometry_backward(positions, row_a, row_b, shifts, a_first_occ, b_perm, b_offsets, grad_vectors, grad_lengths,
+                           need_positions: bool = True, need_shifts: bool = False):
+    E = row_a.numel()
+    N = positions.shape[0]
+    dev = positions.device
+    gpos = torch.empty(N, 3, dtype=F64, device=dev) if need_positions else None
+    gshift = torch.empty(E, 3, dtype=F64, device=dev) if need_shifts else None
+    _check(
+        lib.cm_edge_geometry_backward(
+            _dev(positions, F64, "positions"), _dev(row_a, I32, "row_a"), _dev(row_b, I32, "row_b"),
+            _dev(shifts, F64, "shifts"), _dev(a_first_occ, I32, "a_first_occ"), _dev(b_perm, I32, "b_perm"),
+            _dev(b_offsets, I32, "b_offsets"), _dev(grad_vectors, F32, "grad_vectors"),
+            _dev(grad_lengths, F32, "grad_lengths"), N, E, _dev(gpos, F64, "grad_positions"),
+            _dev(gshift, F64, "grad_shifts"), _stream(),
+        )
+    )
+    return gpos, gshift
 
 
 # ---- cubic spline ---------------------------------------------------------------------------------

@@ -21,6 +21,7 @@ from cuda_mace.ops.invariant_message_passing import InvariantMessagePassingTP
 from cuda_mace.ops.linear import ElementalLinear, Linear
 from cuda_mace.ops.spherical_harmonics import SphericalHarmonics
 from cuda_mace.ops.symmetric_contraction import SymmetricContraction as CUDAContraction
+from cuda_mace.ops._autograd import EdgeGeometryAutograd, _cached
 from cuda_mace.utils.irreps import Instruction
 
 
@@ -118,12 +119,13 @@ def element_linear_to_cuda(skip_tp):
 
 
 class _FloatLinearView:
-    """Presents an e3nn-Linear-like module with fp32 weights without converting the module in place."""
+    """Presents an e3nn-Linear-like module with fp32 weights without converting the module in place; `divide_by`
+    folds the reference's `linear(message) / avg_num_neighbors` (models/InvariantMACE.py:114) into the weights."""
 
-    def __init__(self, linear):
+    def __init__(self, linear, divide_by: float = 1.0):
         self.irreps_in, self.irreps_out = linear.irreps_in, linear.irreps_out
         self.instructions = linear.instructions
-        self.weight = linear.weight.data.float()
+        self.weight = (linear.weight.data.double() / float(divide_by)).float()
 
 
 class InvariantInteraction(torch.nn.Module):
@@ -133,7 +135,7 @@ class InvariantInteraction(torch.nn.Module):
         super().__init__()
         inter = mace_model.interactions[0]
         self.linear_up = linear_matmul(inter.linear_up)
-        self.linear = Linear(_FloatLinearView(inter.linear))
+        self.linear = Linear(_FloatLinearView(inter.linear, divide_by=inter.avg_num_neighbors))
         self.tp = InvariantMessagePassingTP()
         self.skip_tp = element_linear_to_cuda(inter.skip_tp)
         self.avg_num_neighbors = inter.avg_num_neighbors
@@ -144,7 +146,7 @@ class InvariantInteraction(torch.nn.Module):
         node_feats = self.linear_up(node_feats)
         message = self.tp.forward(node_feats, edge_attrs, edge_feats.view(edge_feats.shape[0], -1, node_feats.shape[-1]),
                                   sender, receiver, node_feats.shape[0])
-        message = self.linear(message) / self.avg_num_neighbors
+        message = self.linear(message)  # 1/avg_num_neighbors is folded into its weights
         message = self.skip_tp(message, node_attrs)
         return message, None
 
@@ -156,7 +158,7 @@ class InvariantResidualInteraction(torch.nn.Module):
         super().__init__()
         inter = mace_model.interactions[1]
         self.linear_up = linear_matmul(inter.linear_up)
-        self.linear = Linear(_FloatLinearView(inter.linear))
+        self.linear = Linear(_FloatLinearView(inter.linear, divide_by=inter.avg_num_neighbors))
         self.tp = InvariantMessagePassingTP()
         self.skip_tp = deepcopy(inter.skip_tp).float()
         self.avg_num_neighbors = inter.avg_num_neighbors
@@ -168,7 +170,7 @@ class InvariantResidualInteraction(torch.nn.Module):
         node_feats = self.linear_up(node_feats)
         message = self.tp.forward(node_feats, edge_attrs, edge_feats.view(edge_feats.shape[0], -1, node_feats.shape[-1]),
                                   sender, receiver, node_feats.shape[0])
-        message = self.linear(message) / self.avg_num_neighbors
+        message = self.linear(message)  # 1/avg_num_neighbors is folded into its weights
         return message, sc
 
 
@@ -242,16 +244,18 @@ class OptimizedInvariantMACE(torch.nn.Module):
         e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs)
         node_feats = self.node_embedding(node_attrs.double())
 
-        vectors, lengths = get_edge_vectors_and_lengths(positions=positions, edge_index=data["edge_index"], shifts=shifts)
-        edge_attrs = self.spherical_harmonics.forward(vectors.float())
-        lengths32 = lengths.squeeze(-1).float()
+        # index structures shared by both layers, cached on the caller's tensors so that they are rebuilt only when
+        # the neighbour list / the species change: int32 edge lists (their CSR offsets and sender-sorted view are in
+        # turn cached on these), the fp32 one-hot matrix and the element index per node
+        edge_index = data["edge_index"]
+        receiver, sender = _cached(edge_index, "_cm_int32_rows", None,
+                                   lambda: (edge_index[0].int().contiguous(), edge_index[1].int().contiguous()))
+        node_attrs32, atom_types = _cached(node_attrs, "_cm_species", None,
+                                           lambda: (node_attrs.detach().float(), node_attrs.detach().argmax(dim=-1).int()))
 
-        # index structures shared by both layers: one int32 copy of the edge lists (their CSR offsets and
-        # sender-sorted view are cached on these tensor objects) and one element index per node
-        receiver = data["edge_index"][0].int()
-        sender = data["edge_index"][1].int()
-        node_attrs32 = node_attrs.float()
-        atom_types = node_attrs.argmax(dim=-1).int()
+        # vectors = positions[edge_index[1]] - positions[edge_index[0]] + shifts in fp64, rounded once to fp32
+        vectors32, lengths32 = EdgeGeometryAutograd.apply(positions, shifts, receiver, sender)
+        edge_attrs = self.spherical_harmonics.forward(vectors32)
 
         node_es_list, node_feats_list = [], []
         for interaction, product, readout, edge_spline in zip(self.interactions, self.products, self.readouts, self.edge_splines):

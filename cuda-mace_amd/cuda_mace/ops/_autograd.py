@@ -95,6 +95,43 @@ class InvariantMessagePassingTPAutograd(torch.autograd.Function):
 
 
 # ------------------------------------------------------------------------------------------------
+class EdgeGeometryAutograd(torch.autograd.Function):
+    """(positions [N,3], shifts [E,3], row_a int32 [E] non-decreasing, row_b int32 [E]) -> (vectors fp32 [E,3],
+    lengths fp32 [E]) with vectors = positions[row_b] - positions[row_a] + shifts evaluated in fp64.
+    Differentiable in positions and shifts; the backward scatters edge gradients to atoms over the CSR of row_a
+    and the sorted view of row_b (the same index structures message passing uses), in fp64, without atomics."""
+
+    @staticmethod
+    def forward(ctx, positions, shifts, row_a, row_b):
+        _require(row_a.dtype == I32 and row_b.dtype == I32, "edge geometry: int32 edge lists expected")
+        _require(positions.dim() == 2 and positions.shape[1] == 3, "edge geometry: positions must be [nnodes, 3]")
+        pos64 = positions.detach().double().contiguous()
+        sh64 = shifts.detach().double().contiguous()
+        vec, length = cabi.edge_geometry_forward(pos64, row_a, row_b, sh64)
+        ctx.save_for_backward(pos64, sh64, row_a, row_b)
+        ctx.dtypes = (positions.dtype, shifts.dtype)
+        ctx.mark_non_differentiable()
+        return vec, length
+
+    @staticmethod
+    def backward(ctx, grad_vec, grad_len):
+        pos64, sh64, row_a, row_b = ctx.saved_tensors
+        need_pos, need_shift = ctx.needs_input_grad[:2]
+        nnodes = pos64.shape[0]
+        first_occ = csr_of(row_a, nnodes)
+        perm, off = sender_view_of(row_b, nnodes)
+        gv = grad_vec.contiguous() if grad_vec is not None else None
+        gl = grad_len.contiguous() if grad_len is not None else None
+        gpos, gshift = cabi.edge_geometry_backward(pos64, row_a, row_b, sh64, first_occ, perm, off, gv, gl,
+                                                   need_positions=need_pos, need_shifts=need_shift)
+        if gpos is not None:
+            gpos = gpos.to(ctx.dtypes[0])
+        if gshift is not None:
+            gshift = gshift.to(ctx.dtypes[1])
+        return gpos, gshift, None, None
+
+
+# ------------------------------------------------------------------------------------------------
 class SphericalHarmonicsAutograd(torch.autograd.Function):
     @staticmethod
     def forward(ctx, xyz):

@@ -109,6 +109,28 @@ int cm_sh_backward(const float *xyz, const float *grad_Y, int64_t nedges, float 
                    cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Edge vectors and lengths from positions, and the scatter of per-edge gradients back to atoms.
+ * Replaces the upstream helper the reference model calls at models/InvariantMACE.py:297-301
+ * (get_edge_vectors_and_lengths, positions[edge_index[1]] - positions[edge_index[0]] + shifts, evaluated
+ * there by generic indexing kernels whose backward is a sort-based index_put) and the casts at :303-304, :320.
+ *   positions fp64 [nnodes, 3]; row_a = edge_index[0] (non-decreasing), row_b = edge_index[1], int32 [nedges];
+ *   shifts fp64 [nedges, 3] -> vectors fp32 [nedges, 3] = pos[row_b] - pos[row_a] + shifts (computed in
+ *   fp64, rounded once), lengths fp32 [nedges].
+ * Backward: g = grad_vectors + grad_lengths * vec / |vec| per edge (either gradient may be NULL);
+ *   grad_positions[n] = sum_{e: row_b[e] = n} g - sum_{e: row_a[e] = n} g   (fp64 [nnodes, 3], may be NULL)
+ *   grad_shifts[e] = g                                                     (fp64 [nedges, 3], may be NULL)
+ *   a_first_occ = cm_first_occurences(row_a); b_perm / b_offsets = cm_stable_key_sort(row_b, nedges, nnodes).
+ */
+int cm_edge_geometry_forward(const double *positions, const int32_t *row_a, const int32_t *row_b,
+                             const double *shifts, int64_t nnodes, int64_t nedges, float *vectors,
+                             float *lengths, cm_stream_t stream);
+int cm_edge_geometry_backward(const double *positions, const int32_t *row_a, const int32_t *row_b,
+                              const double *shifts, const int32_t *a_first_occ, const int32_t *b_perm,
+                              const int32_t *b_offsets, const float *grad_vectors,
+                              const float *grad_lengths, int64_t nnodes, int64_t nedges,
+                              double *grad_positions, double *grad_shifts, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Tabulated radial functions: natural cubic spline, R[e, j] = a + b x + c x^2 + d x^3 with
  * x = r[e] - r_knots[idx], idx = clamp(int(r[e] / r_width), 0, nknots - 2); zero when r[e] > r_max.
  * Replaces jit_evaluate_spline / jit_backward_spline (jit_wrappers/src/cubic_spline_wrapper.cpp:14-97,

@@ -236,3 +236,13 @@ def symmetric_contraction(X, atom_types, U3, U2, W3, W2, W1):
     out = out + torch.einsum("nijc,nic,njc->nc", c2, X, X)
     out = out + W1[e][:, 0, :] * X[:, 0, :]
     return out
+
+
+# ----------------------------------------------------------------------------------------
+# edge geometry
+# ----------------------------------------------------------------------------------------
+def edge_geometry(positions, row_a, row_b, shifts):
+    """vectors = positions[row_b] - positions[row_a] + shifts and their lengths; the upstream helper the reference
+    model calls at models/InvariantMACE.py:297-301.  Gradients by torch.autograd on this expression."""
+    vec = positions[row_b.long()] - positions[row_a.long()] + shifts
+    return vec, vec.norm(dim=-1)

@@ -301,3 +301,35 @@ def test_symcon_synthetic_tables(cabi, N, C, ne, seed):
     assert none is None and torch.equal(out, out_nograd)
     close(out, ref.detach(), 3e-5, 3e-6)
     close(gX, Xa.grad, 3e-5, 3e-6)
+
+
+# ------------------------------------------------------------------------------------------------
+# edge geometry (vectors, lengths, scatter of edge gradients to atoms)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("nnodes,avg,iso,seed", [(1, 2, 0.0, 0), (50, 8, 0.3, 1), (3000, 52, 0.0, 2), (20, 200, 0.0, 3)])
+def test_edge_geometry(cabi, nnodes, avg, iso, seed):
+    _say("edge_geometry", nnodes, avg, iso, seed)
+    row_b, row_a = random_graph(nnodes, avg, seed, isolated_frac=iso)  # row_a sorted
+    E = row_a.numel()
+    g = torch.Generator().manual_seed(seed)
+    pos = (torch.rand(nnodes, 3, generator=g, dtype=torch.float64) * 20).requires_grad_(True)
+    shifts = (torch.randn(E, 3, generator=g, dtype=torch.float64) * 3).requires_grad_(True)
+    gv = torch.randn(E, 3, generator=g, dtype=torch.float64)
+    gl = torch.randn(E, generator=g, dtype=torch.float64)
+    vec_ref, len_ref = O.edge_geometry(pos, row_a, row_b, shifts)
+    # the kernel receives fp32 gradients: give the oracle the same rounded values
+    ((vec_ref * gv.float().double()).sum() + (len_ref * gl.float().double()).sum()).backward()
+    d = lambda t: t.detach().to(DEV)
+    fo = cabi.first_occurences(d(row_a), nnodes)
+    perm, off = cabi.stable_key_sort(d(row_b), nnodes)
+    vec, length = cabi.edge_geometry_forward(d(pos), d(row_a), d(row_b), d(shifts))
+    gpos, gshift = cabi.edge_geometry_backward(d(pos), d(row_a), d(row_b), d(shifts), fo, perm, off, d(gv).float(), d(gl).float(),
+                                               need_positions=True, need_shifts=True)
+    assert torch.equal(vec.cpu(), vec_ref.detach().float()) and torch.equal(length.cpu(), len_ref.detach().float())
+    close(gpos, pos.grad, 1e-12, 1e-13)
+    close(gshift, shifts.grad, 1e-12, 1e-13)
+    only_vec, _ = cabi.edge_geometry_backward(d(pos), d(row_a), d(row_b), d(shifts), fo, perm, off, d(gv).float(), None)
+    pos.grad = None
+    vec2, _ = O.edge_geometry(pos, row_a, row_b, shifts)
+    (vec2 * gv.float().double()).sum().backward()
+    close(only_vec, pos.grad, 1e-12, 1e-13)
