@@ -2,14 +2,15 @@
 //
 //   OUT[n, m, :] = scale * X[n, m, :] . W[g(n)][l(m)]      (scale = 1/sqrt(K) in the model)
 //
-// One wavefront owns a tile of 32 nodes x one component m x all Nout columns, so every row of the
-// tile uses the same K x Nout weight block.  The X rows of the tile (K contiguous floats each) are
-// brought in with fully coalesced 16-byte loads and staged in LDS in chunks of 64 columns; the
-// weight operand is read as 16-byte pieces of the TRANSPOSED weights ([Nout, K], which the caller
-// already keeps for the backward) straight from L1/L2 -- the whole weight set is at most a few
-// hundred KB.  Native fp32 MFMA needs no split-precision compensation.  All (group, m, tile)
-// combinations go out in a single launch; per-element weights are selected through a node
-// permutation that lists the nodes group by group, without any host synchronisation.
+// A workgroup of four wavefronts owns a tile of 128 nodes x one component m x all Nout columns, so
+// every row of the tile uses the same K x Nout weight block W[g][l(m)].  K is walked in chunks of 32:
+// the X rows of the tile (each chunk of a row is one 128-byte line) and the matching columns of the
+// TRANSPOSED weights ([Nout, K], which the caller already keeps for the backward) are staged in LDS
+// with coalesced 16-byte loads, and each wave feeds the matrix cores with 16-byte LDS reads -- one A
+// read per 4*NT MFMAs, one B read per 4.  Weights therefore cross L2 once per 128 rows instead of once
+// per 32.  Native fp32 MFMA needs no split-precision compensation.  All (group, m, tile) combinations
+// go out in a single launch; per-element weights are selected through a node permutation that lists
+// the nodes group by group, without any host synchronisation.
 #include <algorithm>
 #include <cmath>
 
@@ -20,20 +21,25 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kTileNodes = 32;  // MFMA M
-constexpr int kKC = 64;         // columns of X staged per step
-constexpr int kLdA = kKC + 4;   // padded LDS row stride (floats)
+constexpr int kWaves = 4;
+constexpr int kTileNodes = 32 * kWaves;  // rows per workgroup (MFMA M = 32 per wave)
+constexpr int kKC = 32;                  // K columns staged per step
+constexpr int kLd = kKC + 4;             // padded LDS row stride (floats)
 
 template <int NT>  // Nout = 32 * NT
-__global__ __launch_bounds__(kWave) void linear_kernel(const float *__restrict__ X, const float *__restrict__ WT,
-                                                       const int32_t *__restrict__ node_perm,
-                                                       const int32_t *__restrict__ group_offsets, int nnodes,
-                                                       int ngroups, int K, float scale, float *__restrict__ OUT) {
+__global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__restrict__ X, const float *__restrict__ WT,
+                                                               const int32_t *__restrict__ node_perm,
+                                                               const int32_t *__restrict__ group_offsets, int nnodes,
+                                                               int ngroups, int K, float scale,
+                                                               float *__restrict__ OUT) {
   constexpr int NOUT = 32 * NT;
-  __shared__ __attribute__((aligned(16))) float sA[kTileNodes * kLdA];
+  __shared__ __attribute__((aligned(16))) float sA[kTileNodes * kLd];
+  __shared__ __attribute__((aligned(16))) float sB[NOUT * kLd];
   __shared__ int sNode[kTileNodes];
 
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = tid / kWave;
   const int m = blockIdx.y;  // component 0..15
   const int l = l_of_m(m);
 
@@ -60,13 +66,13 @@ __global__ __launch_bounds__(kWave) void linear_kernel(const float *__restrict__
   }
   const int nrows = min(kTileNodes, gend - pos0);
 
-  if (lane < kTileNodes) {
+  if (tid < kTileNodes) {
     int node = -1;
-    if (lane < nrows) {
-      node = node_perm ? node_perm[pos0 + lane] : pos0 + lane;
+    if (tid < nrows) {
+      node = node_perm ? node_perm[pos0 + tid] : pos0 + tid;
       if (static_cast<unsigned>(node) >= static_cast<unsigned>(nnodes)) node = -1;
     }
-    sNode[lane] = node;
+    sNode[tid] = node;
   }
   __syncthreads();
 
@@ -78,33 +84,43 @@ __global__ __launch_bounds__(kWave) void linear_kernel(const float *__restrict__
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
 
-  // staging map: 16 lanes x 16 bytes cover the 64 staged columns of a row, 4 rows per load
-  const int srow = lane / 16;
-  const int scol = (lane % 16) * 4;
-  // MFMA operand map: row / column within the tile and which half of the 8-wide k step
+  // staging map: 8 threads x 16 bytes cover the 32 staged columns of a row; 32 rows per pass
+  const int srow = tid / 8;
+  const int scol = (tid % 8) * 4;
+  // MFMA operand map: row / column within the 32-wide block and which half of the 8-wide k step
   const int mrow = lane % 32;
   const int half = lane / 32;
 
-  for (int kc = 0; kc < K; kc += kKC) {
-    const int kw = min(kKC, K - kc);  // multiple of 32
-    f4 pre[8];
+  constexpr int A_PASSES = kTileNodes / 32;
+  constexpr int B_PASSES = NOUT / 32;
+  f4 pa[A_PASSES], pb[B_PASSES];
+  // global -> register prefetch of one K chunk; the next chunk is in flight while the current one is multiplied
+  auto prefetch = [&](int kc) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int row = 4 * i + srow;
-      const int node = sNode[row];
-      pre[i] = zero4();
-      if (node >= 0 && scol < kw) pre[i] = ld4_stream(X + (static_cast<int64_t>(node) * 16 + m) * K + kc + scol);
+    for (int i = 0; i < A_PASSES; ++i) {
+      const int node = sNode[32 * i + srow];
+      pa[i] = zero4();
+      if (node >= 0) pa[i] = ld4_stream(X + (static_cast<int64_t>(node) * 16 + m) * K + kc + scol);
     }
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i) pb[i] = ld4(Wg + static_cast<int64_t>(32 * i + srow) * K + kc + scol);
+  };
+  prefetch(0);
+  for (int kc = 0; kc < K; kc += kKC) {
     __syncthreads();  // previous chunk fully consumed
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<f4 *>(sA + (4 * i + srow) * kLdA + scol) = pre[i];
+    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<f4 *>(sA + (32 * i + srow) * kLd + scol) = pa[i];
+#pragma unroll
+    for (int i = 0; i < B_PASSES; ++i) *reinterpret_cast<f4 *>(sB + (32 * i + srow) * kLd + scol) = pb[i];
     __syncthreads();
+    if (kc + kKC < K) prefetch(kc + kKC);
 
-    for (int kb = 0; kb < kw; kb += 8) {
-      const f4 a = *reinterpret_cast<const f4 *>(sA + mrow * kLdA + kb + 4 * half);
+#pragma unroll
+    for (int kb = 0; kb < kKC; kb += 8) {
+      const f4 a = *reinterpret_cast<const f4 *>(sA + (32 * wave + mrow) * kLd + kb + 4 * half);
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        const f4 b = ld4(Wg + static_cast<int64_t>(32 * t + mrow) * K + kc + kb + 4 * half);
+        const f4 b = *reinterpret_cast<const f4 *>(sB + (32 * t + mrow) * kLd + kb + 4 * half);
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc[t], 0, 0, 0);
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc[t], 0, 0, 0);
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc[t], 0, 0, 0);
@@ -113,10 +129,10 @@ __global__ __launch_bounds__(kWave) void linear_kernel(const float *__restrict__
     }
   }
 
-  // accumulator r of a lane is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the 32x32 block
+  // accumulator r of a lane is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the wave's 32x32 block
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
-    const int row = 8 * (r / 4) + 4 * half + (r % 4);
+    const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
     const int node = sNode[row];
     if (node >= 0) {
       float *op = OUT + (static_cast<int64_t>(node) * 16 + m) * NOUT + mrow;
@@ -130,8 +146,8 @@ template <int NT>
 int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
            int K, float scale, float *OUT, hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
-  hipLaunchKernelGGL(linear_kernel<NT>, dim3(static_cast<unsigned>(tiles), 16), dim3(kWave), 0, st, X, WT, perm, offs,
-                     static_cast<int>(nnodes), ngroups, K, scale, OUT);
+  hipLaunchKernelGGL(linear_kernel<NT>, dim3(static_cast<unsigned>(tiles), 16), dim3(kWaves * kWave), 0, st, X, WT, perm,
+                     offs, static_cast<int>(nnodes), ngroups, K, scale, OUT);
   return check_launch("cm_linear");
 }
 

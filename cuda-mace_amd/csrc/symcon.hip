@@ -10,6 +10,7 @@
 #include <algorithm>
 
 #include "common.hpp"
+#include "symcon_lmax3.inc"
 
 namespace cm {
 namespace {
@@ -132,6 +133,88 @@ __global__ void symcon_forward_kernel(const float *__restrict__ X, const int32_t
   }
 }
 
+// Specialised forward for the l_max = 3 structure known at build time: the monomial lists are unrolled, so a
+// thread (= one channel) keeps its 77 + 16 + 1 coefficients, the node's 16 inputs and 16 gradient accumulators in
+// registers and streams over kNodesPerBlock nodes of one element.  No LDS; loads and stores are coalesced rows.
+constexpr int kNodesPerBlock = 16;
+
+template <bool GRAD>
+__global__ __launch_bounds__(kWave) void symcon_lmax3_kernel(const float *__restrict__ X,
+                                                            const int32_t *__restrict__ node_perm,
+                                                            const int32_t *__restrict__ group_offsets,
+                                                            const float *__restrict__ T3, const float *__restrict__ T2,
+                                                            const float *__restrict__ T1, int nnodes, int ne, int C,
+                                                            float *__restrict__ out, float *__restrict__ grad) {
+  const int c = blockIdx.y * kWave + threadIdx.x;
+  int tile = blockIdx.x;
+  int e = 0, pos0 = 0, gend = 0;
+  bool found = false;
+  for (e = 0; e < ne; ++e) {
+    const int lo = group_offsets[e], hi = group_offsets[e + 1];
+    const int tiles = (hi - lo + kNodesPerBlock - 1) / kNodesPerBlock;
+    if (tile < tiles) {
+      pos0 = lo + tile * kNodesPerBlock;
+      gend = hi;
+      found = true;
+      break;
+    }
+    tile -= tiles;
+  }
+  if (!found || c >= C) return;
+  const int nb = min(kNodesPerBlock, gend - pos0);
+
+  float t3[CM_SYMCON_N3], t2[CM_SYMCON_N2];
+#pragma unroll
+  for (int t = 0; t < CM_SYMCON_N3; ++t) t3[t] = T3[(static_cast<int64_t>(e) * CM_SYMCON_N3 + t) * C + c];
+#pragma unroll
+  for (int t = 0; t < CM_SYMCON_N2; ++t) t2[t] = T2[(static_cast<int64_t>(e) * CM_SYMCON_N2 + t) * C + c];
+  const float t1 = T1[static_cast<int64_t>(e) * C + c];
+
+  for (int b = 0; b < nb; ++b) {
+    const int node = node_perm[pos0 + b];
+    if (static_cast<unsigned>(node) >= static_cast<unsigned>(nnodes)) continue;
+    const float *xp = X + static_cast<int64_t>(node) * 16 * C + c;
+    float x[16], g[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      x[i] = xp[i * C];
+      g[i] = 0.f;
+    }
+    float acc = t1 * x[0];
+    g[0] = t1;
+#define CM_TERM3(t, i, j, k)                    \
+  {                                             \
+    const float w = t3[t];                      \
+    const float wjk = w * (x[j] * x[k]);        \
+    acc = fmaf(wjk, x[i], acc);                 \
+    if (GRAD) {                                 \
+      g[i] += wjk;                              \
+      g[j] = fmaf(w * x[i], x[k], g[j]);        \
+      g[k] = fmaf(w * x[i], x[j], g[k]);        \
+    }                                           \
+  }
+    CM_SYMCON_MONO3(CM_TERM3)
+#undef CM_TERM3
+#define CM_TERM2(t, i, j)                       \
+  {                                             \
+    const float w = t2[t];                      \
+    acc = fmaf(w * x[i], x[j], acc);            \
+    if (GRAD) {                                 \
+      g[i] = fmaf(w, x[j], g[i]);               \
+      g[j] = fmaf(w, x[i], g[j]);               \
+    }                                           \
+  }
+    CM_SYMCON_MONO2(CM_TERM2)
+#undef CM_TERM2
+    out[static_cast<int64_t>(node) * C + c] = acc;
+    if (GRAD) {
+      float *gp = grad + static_cast<int64_t>(node) * 16 * C + c;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) gp[i * C] = g[i];
+    }
+  }
+}
+
 __global__ void symcon_backward_kernel(const float *__restrict__ grad, const float *__restrict__ gout, int64_t nnodes,
                                        int C, float *__restrict__ gX) {
   const int C4 = C / 4;
@@ -193,8 +276,25 @@ extern "C" int cm_symcon_forward(const float *X, const int32_t *node_perm, const
   CM_REQUIRE(nelements >= 1 && n3 >= 0 && n2 >= 0, "cm_symcon_forward: bad sizes");
   if (nnodes == 0) return CM_OK;
   CM_REQUIRE(X && node_perm && group_offsets && T1 && out, "cm_symcon_forward: NULL pointer");
-  CM_REQUIRE((n3 == 0 || (mono3_ijk && T3)) && (n2 == 0 || (mono2_ij && T2)), "cm_symcon_forward: NULL table");
+  const bool builtin = mono3_ijk == nullptr && mono2_ij == nullptr;
+  CM_REQUIRE(builtin || ((n3 == 0 || (mono3_ijk && T3)) && (n2 == 0 || (mono2_ij && T2))), "cm_symcon_forward: NULL table");
   hipStream_t st = cm::as_stream(stream);
+  if (mono3_ijk == nullptr && mono2_ij == nullptr) {
+    // built-in l_max = 3 structure: unrolled register kernel
+    CM_REQUIRE(n3 == CM_SYMCON_N3 && n2 == CM_SYMCON_N2,
+               "cm_symcon_forward: built-in structure has %d cubic and %d quadratic monomials, got %d and %d", CM_SYMCON_N3,
+               CM_SYMCON_N2, n3, n2);
+    CM_REQUIRE(T3 && T2, "cm_symcon_forward: NULL table");
+    const dim3 grid(static_cast<unsigned>(cm::ceil_div(nnodes, cm::kNodesPerBlock) + nelements),
+                    static_cast<unsigned>(cm::ceil_div(channels, cm::kWave)));
+    if (grad)
+      hipLaunchKernelGGL(cm::symcon_lmax3_kernel<true>, grid, dim3(cm::kWave), 0, st, X, node_perm, group_offsets, T3, T2, T1,
+                         static_cast<int>(nnodes), nelements, channels, out, grad);
+    else
+      hipLaunchKernelGGL(cm::symcon_lmax3_kernel<false>, grid, dim3(cm::kWave), 0, st, X, node_perm, group_offsets, T3, T2, T1,
+                         static_cast<int>(nnodes), nelements, channels, out, grad);
+    return cm::check_launch("cm_symcon_forward");
+  }
   // LDS per workgroup is held to 32 KB (two [NB][16][C] fp32 arrays) so that several fit a CU
   if (channels <= 128) {
     const unsigned grid = static_cast<unsigned>(cm::ceil_div(nnodes, 2) + nelements);
@@ -206,6 +306,31 @@ extern "C" int cm_symcon_forward(const float *X, const int32_t *node_perm, const
                       T2, T1, static_cast<int>(nnodes), nelements, out, grad);
   }
   return cm::check_launch("cm_symcon_forward");
+}
+
+extern "C" int cm_symcon_builtin_structure(int32_t *mono3_ijk, int capacity3, int32_t *mono2_ij, int capacity2,
+                                           int *n3, int *n2) {
+  static const int32_t k3[] = {
+#define CM_PACK3(t, i, j, k) ((i) | ((j) << 8) | ((k) << 16)),
+      CM_SYMCON_MONO3(CM_PACK3)
+#undef CM_PACK3
+  };
+  static const int32_t k2[] = {
+#define CM_PACK2(t, i, j) ((i) | ((j) << 8)),
+      CM_SYMCON_MONO2(CM_PACK2)
+#undef CM_PACK2
+  };
+  if (n3) *n3 = CM_SYMCON_N3;
+  if (n2) *n2 = CM_SYMCON_N2;
+  if (mono3_ijk) {
+    CM_REQUIRE(capacity3 >= CM_SYMCON_N3, "cm_symcon_builtin_structure: mono3 buffer too small");
+    for (int t = 0; t < CM_SYMCON_N3; ++t) mono3_ijk[t] = k3[t];
+  }
+  if (mono2_ij) {
+    CM_REQUIRE(capacity2 >= CM_SYMCON_N2, "cm_symcon_builtin_structure: mono2 buffer too small");
+    for (int t = 0; t < CM_SYMCON_N2; ++t) mono2_ij[t] = k2[t];
+  }
+  return CM_OK;
 }
 
 extern "C" int cm_symcon_backward(const float *grad, const float *grad_out, int64_t nnodes, int channels, float *gX,

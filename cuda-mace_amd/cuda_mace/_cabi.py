@@ -47,6 +47,7 @@ SIGNATURES = {
     "cm_linear": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _f32, _p, _p]),
     "cm_symcon_tables": (_i32, [_p, _p, _p, _i32, _p, _p, _p, _i32, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _p, _p, _p]),
     "cm_symcon_forward": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
+    "cm_symcon_builtin_structure": (_i32, [_p, _i32, _p, _i32, _p, _p]),
     "cm_symcon_backward": (_i32, [_p, _p, _i64, _i32, _p, _p]),
 }
 
@@ -274,7 +275,20 @@ def symcon_tables(term3_off, term3_path, term3_val, term2_off, term2_path, term2
     return T3, T2, T1
 
 
-def symcon_forward(X, node_perm, group_offsets, mono3, mono2, T3, T2, T1, want_grad: bool = True):
+def symcon_builtin_structure():
+    """(mono3, mono2) int32 numpy arrays of the monomial lists compiled into the library."""
+    import numpy as np
+
+    n3, n2 = ctypes.c_int(0), ctypes.c_int(0)
+    _check(lib.cm_symcon_builtin_structure(None, 0, None, 0, ctypes.byref(n3), ctypes.byref(n2)))
+    m3 = np.zeros(n3.value, dtype=np.int32)
+    m2 = np.zeros(n2.value, dtype=np.int32)
+    _check(lib.cm_symcon_builtin_structure(m3.ctypes.data, n3.value, m2.ctypes.data, n2.value, None, None))
+    return m3, m2
+
+
+def symcon_forward(X, node_perm, group_offsets, mono3, mono2, T3, T2, T1, want_grad: bool = True, builtin: bool = False):
+    """builtin=True: the monomial lists are the ones compiled into the library; the unrolled kernel is used."""
     N, sixteen, C = X.shape
     if sixteen != 16:
         raise CudaMaceError("symmetric contraction: X must be [N,16,C]")
@@ -284,7 +298,8 @@ def symcon_forward(X, node_perm, group_offsets, mono3, mono2, T3, T2, T1, want_g
     _check(
         lib.cm_symcon_forward(
             _dev(X, F32, "X"), _dev(node_perm, I32, "node_perm"), _dev(group_offsets, I32, "group_offsets"),
-            _dev(mono3, I32, "mono3"), mono3.numel(), _dev(mono2, I32, "mono2"), mono2.numel(),
+            None if builtin else _dev(mono3, I32, "mono3"), mono3.numel(),
+            None if builtin else _dev(mono2, I32, "mono2"), mono2.numel(),
             _dev(T3, F32, "T3"), _dev(T2, F32, "T2"), _dev(T1, F32, "T1"), N, ne, C,
             _dev(out, F32, "out"), _dev(grad, F32, "grad"), _stream(),
         )

@@ -249,10 +249,12 @@ class SymmetricContractionAutograd(torch.autograd.Function):
         def build_structure():
             (m3, o3, p3, v3), (m2, o2, p2, v2) = monomials_from_packed(
                 U3_num_nonzero, U3_indices, U3_values, U2_num_nonzero, U2_indices, U2_values)
-            return tuple(torch.from_numpy(a).to(dev) for a in (m3, o3, p3, v3, m2, o2, p2, v2))
+            b3, b2 = cabi.symcon_builtin_structure()
+            builtin = bool(np.array_equal(m3, b3) and np.array_equal(m2, b2))
+            return tuple(torch.from_numpy(a).to(dev) for a in (m3, o3, p3, v3, m2, o2, p2, v2)) + (builtin,)
 
         key = tuple((t.data_ptr(), t._version) for t in (U3_num_nonzero, U3_values, U2_num_nonzero, U2_indices, U2_values))
-        m3, o3, p3, v3, m2, o2, p2, v2 = _cached(U3_indices, "_cm_monomials", key, build_structure)
+        m3, o3, p3, v3, m2, o2, p2, v2, builtin = _cached(U3_indices, "_cm_monomials", key, build_structure)
 
         # weights are [nlout = 1, nelements, npaths, C]; only the scalar output block exists
         w3 = W3.reshape(-1, W3.shape[-2], W3.shape[-1])[:, : int(W3_size)].contiguous()
@@ -264,7 +266,7 @@ class SymmetricContractionAutograd(torch.autograd.Function):
 
         perm, off = groups_of(atom_types, ne)
         want_grad = X.requires_grad
-        out, grad = cabi.symcon_forward(X.contiguous(), perm, off, m3, m2, T3, T2, T1, want_grad=want_grad)
+        out, grad = cabi.symcon_forward(X.contiguous(), perm, off, m3, m2, T3, T2, T1, want_grad=want_grad, builtin=builtin)
         if want_grad:
             ctx.save_for_backward(grad)
         return out.view(X.shape[0], 1, X.shape[2])

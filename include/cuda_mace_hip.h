@@ -198,6 +198,13 @@ int cm_symcon_forward(const float *X, const int32_t *node_perm, const int32_t *g
                       const int32_t *mono3_ijk, int n3, const int32_t *mono2_ij, int n2,
                       const float *T3, const float *T2, const float *T1, int64_t nnodes,
                       int nelements, int channels, float *out, float *grad, cm_stream_t stream);
+/* The monomial lists of the l_max = 3, scalar-output coupling tensors are also compiled into the library
+ * (sorted triples / pairs in lexicographic order).  Passing mono3_ijk = mono2_ij = NULL to cm_symcon_forward
+ * selects a kernel unrolled over that built-in structure (n3, n2 and the row order of T3, T2 must then be the
+ * built-in ones).  cm_symcon_builtin_structure copies the lists to HOST buffers (either may be NULL) and
+ * returns their lengths, so that a caller can check that the tables it was given have this structure. */
+int cm_symcon_builtin_structure(int32_t *mono3_ijk_host, int capacity3, int32_t *mono2_ij_host,
+                                int capacity2, int *n3, int *n2);
 /*   gX[n, i, c] = grad_out[n, c] * grad[n, i, c] */
 int cm_symcon_backward(const float *grad, const float *grad_out, int64_t nnodes, int channels,
                        float *gX, cm_stream_t stream);
