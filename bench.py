@@ -26,11 +26,15 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 
 def mp_algorithmic_bytes(N, E, C):
-    """Each operand touched once.  forward: X, Y, R, sender, CSR in; out.  backward edge pass without gX
-    (first layer): X, Y, R, grad_out, sender, CSR in; gY, gR out."""
+    """Each operand touched once.  Tabulated radial weights R[E,4,C] (the reference's op): forward reads X, Y, R,
+    sender, CSR and writes out; the backward edge pass without gX (first layer) reads X, Y, R, grad_out, sender, CSR and
+    writes gY, gR.  Fused radial spline: R, gR are replaced by the edge lengths / their gradient and the spline table."""
     fwd = 4 * (4 * E * C + 16 * E + 17 * N * C) + 4 * E + 8 * N
     bwd_edge = 4 * (8 * E * C + 32 * E + 17 * N * C) + 4 * E + 8 * N
-    return fwd, bwd_edge
+    table = 255 * 16 * C * 4
+    fwd_fused = 4 * (17 * E + 17 * N * C) + 4 * E + 8 * N + table
+    bwd_fused = 4 * (34 * E + 17 * N * C) + 4 * E + 8 * N + table
+    return fwd, bwd_edge, fwd_fused, bwd_fused
 
 
 def main():
@@ -42,6 +46,8 @@ def main():
     ap.add_argument("--channels", type=int, default=128)
     ap.add_argument("--elements", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--tabulated-radial", action="store_true",
+                    help="keep the reference's separate spline step (R[E,4,C] in HBM) instead of the fused kernels")
     ap.add_argument("--cpu-atoms", type=int, default=1500, help="size of the box the CPU baseline is timed on")
     args = ap.parse_args()
 
@@ -65,7 +71,8 @@ def main():
     data_cpu = make_system(N, ne, seed=0, density=0.1)
     E = int(data_cpu["edge_index"].shape[1])
     upstream = SyntheticInvariantMACE(channels=C, atomic_numbers=tuple(range(1, ne + 1)), avg_num_neighbors=E / N, seed=0)
-    model = OptimizedInvariantMACE(upstream, device="cuda")
+    fused = not args.tabulated_radial
+    model = OptimizedInvariantMACE(upstream, device="cuda", fused_radial=fused)
     data = to_device(data_cpu, "cuda")
     print("# setup %.1fs: N=%d E=%d C=%d" % (time.time() - t0, N, E, C), file=sys.stderr, flush=True)
 
@@ -77,10 +84,11 @@ def main():
         step()
     torch.cuda.synchronize()
 
-    # live timing of the dominant kernel: events on the launch stream around every backward edge pass that runs
-    # without the sender pass (first layer: one kernel per call) and around every forward launch
-    events = {"mp_backward_edge": [], "mp_forward": []}
-    orig_bwd, orig_fwd = cabi.mp_backward, cabi.mp_forward
+    # live timing of the message-passing kernels: events on the launch stream around every forward launch and around
+    # every backward edge pass that runs without the sender pass (first layer: one kernel per call)
+    fwd_name, bwd_name = ("mp_spline_forward", "mp_spline_backward") if fused else ("mp_forward", "mp_backward")
+    events = {fwd_name: [], bwd_name: []}
+    originals = {fwd_name: getattr(cabi, fwd_name), bwd_name: getattr(cabi, bwd_name)}
 
     def timed(name, fn, pred):
         def wrapper(*a, **k):
@@ -94,8 +102,8 @@ def main():
             return r
         return wrapper
 
-    cabi.mp_backward = timed("mp_backward_edge", orig_bwd, lambda k: not k.get("need_gX", True))
-    cabi.mp_forward = timed("mp_forward", orig_fwd, lambda k: True)
+    setattr(cabi, bwd_name, timed(bwd_name, originals[bwd_name], lambda k: not k.get("need_gX", True)))
+    setattr(cabi, fwd_name, timed(fwd_name, originals[fwd_name], lambda k: True))
 
     torch.cuda.synchronize()
     t_start = time.perf_counter()
@@ -103,7 +111,8 @@ def main():
         energy, forces = step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t_start
-    cabi.mp_backward, cabi.mp_forward = orig_bwd, orig_fwd
+    for name, fn in originals.items():
+        setattr(cabi, name, fn)
 
     ms_per_step = 1e3 * elapsed / args.steps
     value = N * args.steps / elapsed
@@ -113,21 +122,58 @@ def main():
         ts = [s.elapsed_time(e) for s, e in events[name]]
         return sum(ts) / len(ts) if ts else None
 
-    fwd_bytes, bwd_bytes = mp_algorithmic_bytes(N, E, C)
-    t_bwd, t_fwd = avg_ms("mp_backward_edge"), avg_ms("mp_forward")
-    achieved = bwd_bytes / (t_bwd * 1e-3) / 1e9
-    roofline = {
-        "kernel": "mp_backward_edge_kernel<%d,true,true,false>" % C,
-        "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-        "algorithmic_bytes_per_launch": bwd_bytes, "avg_launch_ms": round(t_bwd, 4),
-        "launches_timed": len(events["mp_backward_edge"]),
-    }
-    others = {
-        "mp_forward_kernel<%d>" % C: {
-            "achieved": round(fwd_bytes / (t_fwd * 1e-3) / 1e9, 1), "frac": round(fwd_bytes / (t_fwd * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "algorithmic_bytes_per_launch": fwd_bytes, "avg_launch_ms": round(t_fwd, 4), "unit": "GB/s"},
-    }
+    def entry(nbytes, ms, **extra):
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        d = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes_per_launch": nbytes,
+             "avg_launch_ms": round(ms, 4)}
+        d.update(extra)
+        return d
+
+    fwd_b, bwd_b, fwd_fb, bwd_fb = mp_algorithmic_bytes(N, E, C)
+    t_bwd, t_fwd = avg_ms(bwd_name), avg_ms(fwd_name)
+    if fused:
+        roofline = entry(bwd_fb, t_bwd, kernel="mp_spline_backward_edge_kernel<%d,true,true,false>" % C,
+                         launches_timed=len(events[bwd_name]),
+                         note="radial weights come from the 2 MB spline table in L2 (16 coefficient loads of 16 B per lane and "
+                              "edge), so this kernel is bounded by L2 bandwidth, not HBM; see roofline_other_kernels for the "
+                              "HBM-bound message passing with tabulated R[E,4,C]")
+        others = {"mp_spline_forward_kernel<%d>" % C: entry(fwd_fb, t_fwd)}
+    else:
+        roofline = entry(bwd_b, t_bwd, kernel="mp_backward_edge_kernel<%d,true,true,false>" % C,
+                         launches_timed=len(events[bwd_name]))
+        others = {"mp_forward_kernel<%d>" % C: entry(fwd_b, t_fwd)}
+
+    # the message-passing op with the reference's signature (tabulated R[E,4,C]) at the same shape, timed on its own
+    def isolated_mp():
+        g = torch.Generator(device="cuda").manual_seed(0)
+        X = torch.randn(N, C, device="cuda", generator=g)
+        Yt = torch.randn(16, E, device="cuda", generator=g)
+        R = torch.randn(E, 4, C, device="cuda", generator=g)
+        G = torch.randn(N, 16, C, device="cuda", generator=g)
+        rcv = data["edge_index"][0].int().contiguous()
+        snd = data["edge_index"][1].int().contiguous()
+        fo = cabi.first_occurences(rcv, N)
+
+        def time_it(fn, reps=10):
+            fn()
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for _ in range(reps):
+                fn()
+            e.record()
+            torch.cuda.synchronize()
+            return s.elapsed_time(e) / reps
+
+        tf = time_it(lambda: cabi.mp_forward(X, Yt, R, snd, fo, N))
+        tb = time_it(lambda: cabi.mp_backward(X, Yt, R, G, snd, fo, None, None, N, need_gX=False))
+        return tf, tb
+
+    if fused:
+        tf, tb = isolated_mp()
+        others["mp_forward_kernel<%d> (isolated op, tabulated R)" % C] = entry(fwd_b, tf)
+        others["mp_backward_edge_kernel<%d,true,true,false> (isolated op, tabulated R)" % C] = entry(bwd_b, tb)
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
@@ -157,7 +203,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "invariant MACE energy+forces, %d-atom periodic box at 0.1 atoms/A^3, %d edges, %dx0e, "
                                "l_max 3, correlation 3, %d elements, random-init weights (seed 0)" % (N, E, C, ne),
-                   "atoms": N, "edges": E, "channels": C},
+                   "atoms": N, "edges": E, "channels": C, "radial": "fused spline" if fused else "tabulated"},
         "roofline": roofline, "roofline_other_kernels": others, "cpu_baseline": cpu_baseline,
     }
     if cpu_baseline:

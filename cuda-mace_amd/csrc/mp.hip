@@ -11,26 +11,12 @@
 // bit for bit.
 #include <algorithm>
 
-#include "common.hpp"
+#include "mp_common.hpp"
 
 namespace cm {
 namespace {
 
-constexpr int kChunk = 64;  // edges whose Y / sender values are staged in LDS at a time
-
-constexpr int pow2ceil(int v) {
-  int p = 1;
-  while (p < v) p <<= 1;
-  return p;
-}
-
-template <int C>
-struct Cfg {
-  static constexpr int LPE = C / 4;          // lanes that carry one edge
-  static constexpr int SW = pow2ceil(LPE);   // slot width in lanes (power of two)
-  static constexpr int EPW = kWave / SW;     // edges in flight per wave
-  static_assert(C % 32 == 0 && C >= 32 && C <= 256, "channel count");
-};
+using namespace mp;
 
 // -----------------------------------------------------------------------------------------------
 // CSR offsets.  Thread e looks at receiver[e-1] -> receiver[e]; a change of value closes every
@@ -64,26 +50,6 @@ __global__ void first_occurences_kernel(const int32_t *__restrict__ receiver, in
       start[n] = nedges;
       end[n] = nedges;
     }
-  }
-}
-
-// Stages Y[0:16, base:base+cnt] (transposed to [edge][16]) and sender[base:base+cnt] in LDS.
-__device__ __forceinline__ void stage_chunk(const float *__restrict__ Y, const int32_t *__restrict__ sender,
-                                            int64_t nedges, int base, int cnt, int lane, float *sY,
-                                            int *sS) {
-  if (lane < cnt) {
-    const int64_t e = base + lane;
-    sS[lane] = sender[e];
-    f4 y[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      y[q].x = Y[(4 * q + 0) * nedges + e];
-      y[q].y = Y[(4 * q + 1) * nedges + e];
-      y[q].z = Y[(4 * q + 2) * nedges + e];
-      y[q].w = Y[(4 * q + 3) * nedges + e];
-    }
-#pragma unroll
-    for (int q = 0; q < 4; ++q) *reinterpret_cast<f4 *>(sY + lane * 16 + 4 * q) = y[q];
   }
 }
 
@@ -167,50 +133,6 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
 // -----------------------------------------------------------------------------------------------
 // backward, edge pass: gR, gY and the per-edge contribution to gX
 // -----------------------------------------------------------------------------------------------
-// Sums p[m] over the SW lanes of a slot.  Butterfly with halving: after the exchange over lane
-// bit b each lane keeps half of its values, so 16 values cost 8+4+2+1 exchanges instead of 16*4.
-// Returns, in every lane, the total for m = bitrev4(cl & 15) (SW >= 16), or for SW == 8 the two
-// totals m = bitrev3(cl) * 2 + {0, 1} in p[0], p[1].
-template <int SW>
-__device__ __forceinline__ void slot_reduce16(float (&p)[16], int cl) {
-  static_assert(SW >= 8, "slot width");
-  {
-    const bool hi = cl & 1;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const float keep = hi ? p[8 + k] : p[k];
-      const float send = hi ? p[k] : p[8 + k];
-      p[k] = keep + __shfl_xor(send, 1);
-    }
-  }
-  {
-    const bool hi = cl & 2;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const float keep = hi ? p[4 + k] : p[k];
-      const float send = hi ? p[k] : p[4 + k];
-      p[k] = keep + __shfl_xor(send, 2);
-    }
-  }
-  {
-    const bool hi = cl & 4;
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      const float keep = hi ? p[2 + k] : p[k];
-      const float send = hi ? p[k] : p[2 + k];
-      p[k] = keep + __shfl_xor(send, 4);
-    }
-  }
-  if constexpr (SW >= 16) {
-    const bool hi = cl & 8;
-    const float keep = hi ? p[1] : p[0];
-    const float send = hi ? p[0] : p[1];
-    p[0] = keep + __shfl_xor(send, 8);
-  }
-  if constexpr (SW >= 32) p[0] += __shfl_xor(p[0], 16);
-  if constexpr (SW >= 64) p[0] += __shfl_xor(p[0], 32);
-}
-
 template <int C, bool WANT_GY, bool WANT_GR, bool WANT_GX>
 __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
     const float *__restrict__ X, const float *__restrict__ Y, const float *__restrict__ R,
@@ -382,29 +304,28 @@ int launch_backward(const float *X, const float *Y, const float *R, const float 
   }
   int rc = check_launch("cm_mp_backward (edge pass)");
   if (rc != CM_OK) return rc;
-  if (gX) {
-    hipLaunchKernelGGL(mp_backward_sender_kernel<C>, dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st, gXe,
-                       perm, offsets, static_cast<int>(nnodes), nedges, gX);
-    rc = check_launch("cm_mp_backward (sender pass)");
-  }
+  if (gX) rc = mp::launch_sender_pass(C, gXe, perm, offsets, nnodes, nedges, gX, st);
   return rc;
 }
 
-}  // namespace
-}  // namespace cm
+template <int C>
+int launch_sender(const float *gXe, const int32_t *perm, const int32_t *offsets, int64_t nnodes, int64_t nedges,
+                  float *gX, hipStream_t st) {
+  hipLaunchKernelGGL(mp_backward_sender_kernel<C>, dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st, gXe, perm,
+                     offsets, static_cast<int>(nnodes), nedges, gX);
+  return check_launch("cm_mp_backward (sender pass)");
+}
 
-#define CM_DISPATCH_C(channels, CALL)                 \
-  switch (channels) {                                 \
-    case 32: { constexpr int C_ = 32; CALL; } break;   \
-    case 64: { constexpr int C_ = 64; CALL; } break;   \
-    case 96: { constexpr int C_ = 96; CALL; } break;   \
-    case 128: { constexpr int C_ = 128; CALL; } break; \
-    case 160: { constexpr int C_ = 160; CALL; } break; \
-    case 192: { constexpr int C_ = 192; CALL; } break; \
-    case 224: { constexpr int C_ = 224; CALL; } break; \
-    case 256: { constexpr int C_ = 256; CALL; } break; \
-    default: break;                                   \
-  }
+}  // namespace
+
+int mp::launch_sender_pass(int channels, const float *gXe, const int32_t *perm, const int32_t *offsets, int64_t nnodes,
+                           int64_t nedges, float *gX, hipStream_t st) {
+  int rc = CM_EINVAL;
+  CM_DISPATCH_C(channels, rc = launch_sender<C_>(gXe, perm, offsets, nnodes, nedges, gX, st));
+  return rc;
+}
+
+}  // namespace cm
 
 extern "C" int cm_channels_supported(int channels) {
   return channels >= 32 && channels <= 256 && channels % 32 == 0;

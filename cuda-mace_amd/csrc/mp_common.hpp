@@ -1,0 +1,132 @@
+// Pieces shared by the message-passing kernels (tabulated-radial and spline-fused variants).
+#pragma once
+
+#include "common.hpp"
+
+namespace cm {
+namespace mp {
+
+constexpr int kChunk = 64;  // edges whose Y / sender values are staged in LDS at a time
+
+constexpr int pow2ceil(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+template <int C>
+struct Cfg {
+  static constexpr int LPE = C / 4;          // lanes that carry one edge
+  static constexpr int SW = pow2ceil(LPE);   // slot width in lanes (power of two)
+  static constexpr int EPW = kWave / SW;     // edges in flight per wave
+  static_assert(C % 32 == 0 && C >= 32 && C <= 256, "channel count");
+};
+
+// Stages Y[0:16, base:base+cnt] (transposed to [edge][16]) and sender[base:base+cnt] in LDS.
+__device__ __forceinline__ void stage_chunk(const float *__restrict__ Y, const int32_t *__restrict__ sender,
+                                            int64_t nedges, int base, int cnt, int lane, float *sY,
+                                            int *sS) {
+  if (lane < cnt) {
+    const int64_t e = base + lane;
+    sS[lane] = sender[e];
+    f4 y[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      y[q].x = Y[(4 * q + 0) * nedges + e];
+      y[q].y = Y[(4 * q + 1) * nedges + e];
+      y[q].z = Y[(4 * q + 2) * nedges + e];
+      y[q].w = Y[(4 * q + 3) * nedges + e];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) *reinterpret_cast<f4 *>(sY + lane * 16 + 4 * q) = y[q];
+  }
+}
+
+// Sums p[m] over the SW lanes of a slot.  Butterfly with halving: after the exchange over lane
+// bit b each lane keeps half of its values, so 16 values cost 8+4+2+1 exchanges instead of 16*4.
+// Returns, in every lane, the total for m = bitrev4(cl & 15) (SW >= 16), or for SW == 8 the two
+// totals m = bitrev3(cl) * 2 + {0, 1} in p[0], p[1].
+template <int SW>
+__device__ __forceinline__ void slot_reduce16(float (&p)[16], int cl) {
+  static_assert(SW >= 8, "slot width");
+  {
+    const bool hi = cl & 1;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float keep = hi ? p[8 + k] : p[k];
+      const float send = hi ? p[k] : p[8 + k];
+      p[k] = keep + __shfl_xor(send, 1);
+    }
+  }
+  {
+    const bool hi = cl & 2;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float keep = hi ? p[4 + k] : p[k];
+      const float send = hi ? p[k] : p[4 + k];
+      p[k] = keep + __shfl_xor(send, 2);
+    }
+  }
+  {
+    const bool hi = cl & 4;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const float keep = hi ? p[2 + k] : p[k];
+      const float send = hi ? p[k] : p[2 + k];
+      p[k] = keep + __shfl_xor(send, 4);
+    }
+  }
+  if constexpr (SW >= 16) {
+    const bool hi = cl & 8;
+    const float keep = hi ? p[1] : p[0];
+    const float send = hi ? p[0] : p[1];
+    p[0] = keep + __shfl_xor(send, 8);
+  }
+  if constexpr (SW >= 32) p[0] += __shfl_xor(p[0], 16);
+  if constexpr (SW >= 64) p[0] += __shfl_xor(p[0], 32);
+}
+
+// Plain sum of one value over the SW lanes of a slot; every lane gets the total.
+template <int SW>
+__device__ __forceinline__ float slot_sum(float v) {
+#pragma unroll
+  for (int off = 1; off < SW; off <<= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+// Which m a lane (position cl in its slot) holds after slot_reduce16, SW >= 16.
+__device__ __forceinline__ int reduced_index16(int cl) {
+  return ((cl & 1) << 3) | ((cl & 2) << 1) | ((cl & 4) >> 1) | ((cl & 8) >> 3);
+}
+
+// Writes the reduced gY values of edge j into the LDS tile sGY[m][kChunk].
+template <int SW>
+__device__ __forceinline__ void store_reduced16(const float (&p)[16], int cl, int j, float *sGY) {
+  if constexpr (SW >= 16) {
+    if (cl < 16) sGY[reduced_index16(cl) * kChunk + j] = p[0];
+  } else {
+    const int m0 = (((cl & 1) << 2) | (cl & 2) | ((cl & 4) >> 2)) * 2;
+    sGY[m0 * kChunk + j] = p[0];
+    sGY[(m0 + 1) * kChunk + j] = p[1];
+  }
+}
+
+// Sender pass of the backward, shared by both variants (defined in mp.hip).
+int launch_sender_pass(int channels, const float *gXe, const int32_t *perm, const int32_t *offsets, int64_t nnodes,
+                       int64_t nedges, float *gX, hipStream_t st);
+
+}  // namespace mp
+}  // namespace cm
+
+#define CM_DISPATCH_C(channels, CALL)                 \
+  switch (channels) {                                 \
+    case 32: { constexpr int C_ = 32; CALL; } break;   \
+    case 64: { constexpr int C_ = 64; CALL; } break;   \
+    case 96: { constexpr int C_ = 96; CALL; } break;   \
+    case 128: { constexpr int C_ = 128; CALL; } break; \
+    case 160: { constexpr int C_ = 160; CALL; } break; \
+    case 192: { constexpr int C_ = 192; CALL; } break; \
+    case 224: { constexpr int C_ = 224; CALL; } break; \
+    case 256: { constexpr int C_ = 256; CALL; } break; \
+    default: break;                                   \
+  }

@@ -1,0 +1,327 @@
+// Invariant message passing with the radial weights evaluated inside the kernels from the cubic-spline
+// table, so that R[E, 4, C], its derivative and grad_R never exist in HBM.
+//
+//   out[n, m, c] = sum_{e -> n} X[sender[e], c] * Y[m, e] * R(r[e])[l(m), c],
+//   R(r)[j] = a + b x + c x^2 + d x^3,  (a, b, c, d) = coeffs[idx, :, j],  x = r - r_knots[idx]
+//
+// Same decomposition as the tabulated-radial kernels (one wave per receiver node, lane = 4 channels,
+// node-resident accumulators / gradients in registers, Y and sender staged in LDS); the per-edge knot
+// interval and offset are staged next to them.  The coefficient table (2 MB at C = 128) lives in L2:
+// per edge and l a lane reads its four 16-byte coefficient pieces, evaluates R_l (and dR_l/dr in the
+// backward) and drops them, so only 16 registers of radial data are live at a time.  The backward
+// returns the gradient with respect to the edge length directly:
+//   g_r[e] = sum_{l, c} X[s, c] * q_l[c] * dR_l/dr[c],   q_l = sum_{m in l} Y[m, e] * grad_out[n, m, c].
+#include <type_traits>
+
+#include "mp_common.hpp"
+
+namespace cm {
+namespace {
+
+using namespace mp;
+
+struct Spline {
+  const float *r;       // [E]
+  const float *knots;   // [nknots]
+  const float *coeffs;  // [nknots - 1, 4, 4C]
+  int nknots;
+  float r_width;
+  float r_max;
+};
+
+// Stages the knot interval (or -1 beyond the cutoff) and the offset inside it for the chunk's edges.
+__device__ __forceinline__ void stage_radial(const Spline &sp, int base, int cnt, int lane, int *sIdx, float *sXr) {
+  if (lane < cnt) {
+    const float re = sp.r[base + lane];
+    int idx = -1;
+    float x = 0.f;
+    if (re <= sp.r_max) {
+      idx = static_cast<int>(re / sp.r_width);
+      idx = idx < 0 ? 0 : (idx > sp.nknots - 2 ? sp.nknots - 2 : idx);
+      x = re - sp.knots[idx];
+    }
+    sIdx[lane] = idx;
+    sXr[lane] = x;
+  }
+}
+
+template <int L>
+struct MRange {
+  static constexpr int lo = L * L;
+  static constexpr int hi = (L + 1) * (L + 1);
+};
+
+// -----------------------------------------------------------------------------------------------
+// forward
+// -----------------------------------------------------------------------------------------------
+template <int C>
+__global__ __launch_bounds__(kWave) void mp_spline_forward_kernel(const float *__restrict__ X,
+                                                                 const float *__restrict__ Y, Spline sp,
+                                                                 const int32_t *__restrict__ sender,
+                                                                 const int32_t *__restrict__ first_occ, int nnodes,
+                                                                 int64_t nedges, float *__restrict__ out) {
+  using K = Cfg<C>;
+  __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
+  __shared__ int sS[kChunk];
+  __shared__ int sIdx[kChunk];
+  __shared__ float sXr[kChunk];
+
+  const int node = blockIdx.x;
+  const int lane = threadIdx.x;
+  const int slot = lane / K::SW;
+  const int cl = lane % K::SW;
+  const bool active = cl < K::LPE;
+  const int e0 = first_occ[node];
+  const int e1 = first_occ[nnodes + node];
+
+  f4 acc[16];
+#pragma unroll
+  for (int m = 0; m < 16; ++m) acc[m] = zero4();
+
+  for (int base = e0; base < e1; base += kChunk) {
+    const int cnt = min(kChunk, e1 - base);
+    __syncthreads();
+    stage_chunk(Y, sender, nedges, base, cnt, lane, sY, sS);
+    stage_radial(sp, base, cnt, lane, sIdx, sXr);
+    __syncthreads();
+    if (active) {
+      for (int j = slot; j < cnt; j += K::EPW) {
+        const int s = sS[j];
+        const int idx = sIdx[j];
+        if (idx < 0 || static_cast<unsigned>(s) >= static_cast<unsigned>(nnodes)) continue;
+        const float xr = sXr[j];
+        const f4 x = ld4(X + static_cast<int64_t>(s) * C + 4 * cl);
+        float y[16];
+        {
+          const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f4 v = yp[q];
+            y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
+          }
+        }
+        const float *cp = sp.coeffs + static_cast<int64_t>(idx) * (16 * C) + 4 * cl;
+        auto per_l = [&](auto lc) {
+          constexpr int L = decltype(lc)::value;
+          const f4 a = ld4(cp + L * C), b = ld4(cp + 4 * C + L * C), c = ld4(cp + 8 * C + L * C), d = ld4(cp + 12 * C + L * C);
+          const f4 t = x * (a + xr * (b + xr * (c + xr * d)));
+#pragma unroll
+          for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) acc[m] += y[m] * t;
+        };
+        per_l(std::integral_constant<int, 0>{});
+        per_l(std::integral_constant<int, 1>{});
+        per_l(std::integral_constant<int, 2>{});
+        per_l(std::integral_constant<int, 3>{});
+      }
+    }
+  }
+
+#pragma unroll
+  for (int off = kWave / 2; off >= K::SW; off >>= 1) {
+#pragma unroll
+    for (int m = 0; m < 16; ++m) acc[m] += shfl_down4(acc[m], off);
+  }
+  if (slot == 0 && active) {
+    float *op = out + static_cast<int64_t>(node) * (16 * C) + 4 * cl;
+#pragma unroll
+    for (int m = 0; m < 16; ++m) st4(op + m * C, acc[m]);
+  }
+}
+
+// -----------------------------------------------------------------------------------------------
+// backward, edge pass: gY, g_r and the per-edge contribution to gX
+// -----------------------------------------------------------------------------------------------
+template <int C, bool WANT_GY, bool WANT_GR, bool WANT_GX>
+__global__ __launch_bounds__(kWave) void mp_spline_backward_edge_kernel(
+    const float *__restrict__ X, const float *__restrict__ Y, Spline sp, const float *__restrict__ G,
+    const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges,
+    float *__restrict__ gY, float *__restrict__ g_r, float *__restrict__ gXe) {
+  using K = Cfg<C>;
+  __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
+  __shared__ int sS[kChunk];
+  __shared__ int sIdx[kChunk];
+  __shared__ float sXr[kChunk];
+  __shared__ float sGY[16 * kChunk];  // [m][edge]
+  __shared__ float sGr[kChunk];
+
+  const int node = blockIdx.x;
+  const int lane = threadIdx.x;
+  const int slot = lane / K::SW;
+  const int cl = lane % K::SW;
+  const bool active = cl < K::LPE;
+  const int e0 = first_occ[node];
+  const int e1 = first_occ[nnodes + node];
+  if (e0 >= e1) return;
+
+  f4 g[16];
+  {
+    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + 4 * cl;
+#pragma unroll
+    for (int m = 0; m < 16; ++m) g[m] = active ? ld4(gp + m * C) : zero4();
+  }
+
+  for (int base = e0; base < e1; base += kChunk) {
+    const int cnt = min(kChunk, e1 - base);
+    __syncthreads();
+    stage_chunk(Y, sender, nedges, base, cnt, lane, sY, sS);
+    stage_radial(sp, base, cnt, lane, sIdx, sXr);
+    __syncthreads();
+    // every lane of a slot takes part in the reductions, so the loop bound is slot-uniform
+    for (int j = slot; j < cnt; j += K::EPW) {
+      const int64_t e = base + j;
+      const int s = sS[j];
+      const int idx = sIdx[j];
+      const bool live = active && idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
+      const float xr = sXr[j];
+      f4 x = zero4();
+      if (live) x = ld4(X + static_cast<int64_t>(s) * C + 4 * cl);
+      float y[16];
+      {
+        const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const f4 v = yp[q];
+          y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
+        }
+      }
+      const float *cp = sp.coeffs + static_cast<int64_t>(idx < 0 ? 0 : idx) * (16 * C) + 4 * cl;
+      float p[16];
+      f4 gxe = zero4();
+      f4 gr4 = zero4();
+      auto per_l = [&](auto lc) {
+        constexpr int L = decltype(lc)::value;
+        f4 rl = zero4(), drl = zero4();
+        if (live) {
+          const f4 a = ld4(cp + L * C), b = ld4(cp + 4 * C + L * C), c = ld4(cp + 8 * C + L * C), d = ld4(cp + 12 * C + L * C);
+          rl = a + xr * (b + xr * (c + xr * d));
+          drl = b + xr * (2.f * c + (3.f * xr) * d);
+        }
+        f4 q = zero4();
+#pragma unroll
+        for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) q += y[m] * g[m];
+        if constexpr (WANT_GY) {
+          const f4 t = x * rl;
+#pragma unroll
+          for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) p[m] = hsum4(g[m] * t);
+        }
+        if constexpr (WANT_GX) gxe += rl * q;
+        if constexpr (WANT_GR) gr4 += (x * q) * drl;
+      };
+      per_l(std::integral_constant<int, 0>{});
+      per_l(std::integral_constant<int, 1>{});
+      per_l(std::integral_constant<int, 2>{});
+      per_l(std::integral_constant<int, 3>{});
+
+      if constexpr (WANT_GX) {
+        if (active) st4(gXe + e * C + 4 * cl, gxe);
+      }
+      if constexpr (WANT_GR) {
+        const float tot = slot_sum<K::SW>(hsum4(gr4));
+        if (cl == 0) sGr[j] = tot;
+      }
+      if constexpr (WANT_GY) {
+        slot_reduce16<K::SW>(p, cl);
+        store_reduced16<K::SW>(p, cl, j, sGY);
+      }
+    }
+    if constexpr (WANT_GY || WANT_GR) {
+      __syncthreads();
+      if (lane < cnt) {
+        const int64_t e = base + lane;
+        if constexpr (WANT_GY) {
+#pragma unroll
+          for (int m = 0; m < 16; ++m) gY[m * nedges + e] = sGY[m * kChunk + lane];
+        }
+        if constexpr (WANT_GR) g_r[e] = sGr[lane];
+      }
+    }
+  }
+}
+
+template <int C>
+int launch_forward(const float *X, const float *Y, const Spline &sp, const int32_t *sender, const int32_t *first_occ,
+                   int64_t nnodes, int64_t nedges, float *out, hipStream_t st) {
+  hipLaunchKernelGGL(mp_spline_forward_kernel<C>, dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st, X, Y, sp, sender,
+                     first_occ, static_cast<int>(nnodes), nedges, out);
+  return check_launch("cm_mp_spline_forward");
+}
+
+template <int C, bool GY, bool GR, bool GX>
+void launch_edge(const float *X, const float *Y, const Spline &sp, const float *G, const int32_t *sender,
+                 const int32_t *first_occ, int64_t nnodes, int64_t nedges, float *gY, float *g_r, float *gXe,
+                 hipStream_t st) {
+  hipLaunchKernelGGL((mp_spline_backward_edge_kernel<C, GY, GR, GX>), dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st,
+                     X, Y, sp, G, sender, first_occ, static_cast<int>(nnodes), nedges, gY, g_r, gXe);
+}
+
+template <int C>
+int launch_backward(const float *X, const float *Y, const Spline &sp, const float *G, const int32_t *sender,
+                    const int32_t *first_occ, const int32_t *perm, const int32_t *offsets, int64_t nnodes, int64_t nedges,
+                    float *gX, float *gY, float *g_r, float *gXe, hipStream_t st) {
+  const int key = (gY ? 4 : 0) | (g_r ? 2 : 0) | (gX ? 1 : 0);
+  switch (key) {
+    case 7: launch_edge<C, true, true, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+    case 6: launch_edge<C, true, true, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+    case 5: launch_edge<C, true, false, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+    case 4: launch_edge<C, true, false, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+    case 3: launch_edge<C, false, true, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+    case 2: launch_edge<C, false, true, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+    case 1: launch_edge<C, false, false, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+    default: return CM_OK;
+  }
+  int rc = check_launch("cm_mp_spline_backward (edge pass)");
+  if (rc != CM_OK) return rc;
+  if (gX) rc = mp::launch_sender_pass(C, gXe, perm, offsets, nnodes, nedges, gX, st);
+  return rc;
+}
+
+int check_spline(const char *who, const float *r, const float *r_knots, const float *coeffs, int nknots, float r_width,
+                 int64_t nedges) {
+  CM_REQUIRE(nknots >= 2, "%s: need at least two knots, got %d", who, nknots);
+  CM_REQUIRE(r_width > 0.f, "%s: r_width must be positive", who);
+  CM_REQUIRE(nedges == 0 || (r && r_knots && coeffs), "%s: NULL spline operand", who);
+  return CM_OK;
+}
+
+}  // namespace
+}  // namespace cm
+
+extern "C" int cm_mp_spline_forward(const float *X, const float *Y, const float *r, const float *r_knots,
+                                    const float *coeffs, int nknots, float r_width, float r_max, const int32_t *sender,
+                                    const int32_t *first_occ, int64_t nnodes, int64_t nedges, int channels, float *out,
+                                    cm_stream_t stream) {
+  CM_REQUIRE(cm_channels_supported(channels), "cm_mp_spline_forward: channels=%d must be a multiple of 32 in [32, 256]", channels);
+  CM_REQUIRE(nedges >= 0 && nnodes >= 0, "cm_mp_spline_forward: negative size");
+  CM_REQUIRE(nedges < INT32_MAX && nnodes < INT32_MAX / 2, "cm_mp_spline_forward: sizes exceed int32 indexing");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(X && first_occ && out, "cm_mp_spline_forward: NULL pointer");
+  CM_REQUIRE(nedges == 0 || (Y && sender), "cm_mp_spline_forward: NULL edge operand");
+  int rc = cm::check_spline("cm_mp_spline_forward", r, r_knots, coeffs, nknots, r_width, nedges);
+  if (rc != CM_OK) return rc;
+  const cm::Spline sp{r, r_knots, coeffs, nknots, r_width, r_max};
+  rc = CM_EINVAL;
+  CM_DISPATCH_C(channels, rc = cm::launch_forward<C_>(X, Y, sp, sender, first_occ, nnodes, nedges, out, cm::as_stream(stream)));
+  return rc;
+}
+
+extern "C" int cm_mp_spline_backward(const float *X, const float *Y, const float *r, const float *r_knots,
+                                     const float *coeffs, int nknots, float r_width, float r_max, const float *grad_out,
+                                     const int32_t *sender, const int32_t *first_occ, const int32_t *sender_perm,
+                                     const int32_t *sender_offsets, int64_t nnodes, int64_t nedges, int channels,
+                                     float *gX, float *gY, float *grad_r, float *edge_scratch, cm_stream_t stream) {
+  CM_REQUIRE(cm_channels_supported(channels), "cm_mp_spline_backward: channels=%d must be a multiple of 32 in [32, 256]", channels);
+  CM_REQUIRE(nedges >= 0 && nnodes >= 0, "cm_mp_spline_backward: negative size");
+  CM_REQUIRE(nedges < INT32_MAX && nnodes < INT32_MAX / 2, "cm_mp_spline_backward: sizes exceed int32 indexing");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(X && grad_out && first_occ, "cm_mp_spline_backward: NULL pointer");
+  CM_REQUIRE(nedges == 0 || (Y && sender), "cm_mp_spline_backward: NULL edge operand");
+  CM_REQUIRE(!gX || (sender_offsets && (nedges == 0 || (sender_perm && edge_scratch))),
+             "cm_mp_spline_backward: gX wanted but sender_perm / sender_offsets / edge_scratch missing");
+  int rc = cm::check_spline("cm_mp_spline_backward", r, r_knots, coeffs, nknots, r_width, nedges);
+  if (rc != CM_OK) return rc;
+  const cm::Spline sp{r, r_knots, coeffs, nknots, r_width, r_max};
+  rc = CM_EINVAL;
+  CM_DISPATCH_C(channels, rc = cm::launch_backward<C_>(X, Y, sp, grad_out, sender, first_occ, sender_perm, sender_offsets,
+                                                       nnodes, nedges, gX, gY, grad_r, edge_scratch, cm::as_stream(stream)));
+  return rc;
+}

@@ -128,6 +128,15 @@ class _FloatLinearView:
         self.weight = (linear.weight.data.double() / float(divide_by)).float()
 
 
+def _message_passing(tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline):
+    """Tabulated radial weights (edge_feats [E, 4C], the reference's data flow) or, when edge_feats is None, radial
+    weights evaluated inside the message-passing kernels from the spline of the edge lengths."""
+    if edge_feats is not None:
+        return tp.forward(node_feats, edge_attrs, edge_feats.view(edge_feats.shape[0], -1, node_feats.shape[-1]), sender,
+                          receiver, node_feats.shape[0])
+    return tp.forward_spline(node_feats, edge_attrs, edge_lengths, edge_spline, sender, receiver, node_feats.shape[0])
+
+
 class InvariantInteraction(torch.nn.Module):
     """First layer: linear_up, message passing, per-l linear, per-element linear."""
 
@@ -140,12 +149,12 @@ class InvariantInteraction(torch.nn.Module):
         self.skip_tp = element_linear_to_cuda(inter.skip_tp)
         self.avg_num_neighbors = inter.avg_num_neighbors
 
-    def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None):
+    def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,
+                edge_lengths=None, edge_spline=None):
         if sender is None:
             sender, receiver = edge_index[1].int(), edge_index[0].int()
         node_feats = self.linear_up(node_feats)
-        message = self.tp.forward(node_feats, edge_attrs, edge_feats.view(edge_feats.shape[0], -1, node_feats.shape[-1]),
-                                  sender, receiver, node_feats.shape[0])
+        message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline)
         message = self.linear(message)  # 1/avg_num_neighbors is folded into its weights
         message = self.skip_tp(message, node_attrs)
         return message, None
@@ -163,20 +172,23 @@ class InvariantResidualInteraction(torch.nn.Module):
         self.skip_tp = deepcopy(inter.skip_tp).float()
         self.avg_num_neighbors = inter.avg_num_neighbors
 
-    def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None):
+    def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,
+                edge_lengths=None, edge_spline=None):
         if sender is None:
             sender, receiver = edge_index[1].int(), edge_index[0].int()
         sc = self.skip_tp(node_feats, node_attrs)
         node_feats = self.linear_up(node_feats)
-        message = self.tp.forward(node_feats, edge_attrs, edge_feats.view(edge_feats.shape[0], -1, node_feats.shape[-1]),
-                                  sender, receiver, node_feats.shape[0])
+        message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline)
         message = self.linear(message)  # 1/avg_num_neighbors is folded into its weights
         return message, sc
 
 
 class OptimizedInvariantMACE(torch.nn.Module):
-    def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256):
+    def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True):
+        """fused_radial=True evaluates the radial spline inside the message-passing kernels (same numbers, no
+        [nedges, 4C] tensors in memory); False keeps the reference's separate CubicSpline -> message passing steps."""
         super().__init__()
+        self.fused_radial = bool(fused_radial)
         assert int(mace_model.num_interactions) == 2, "exactly two interaction layers are supported"
         self.register_buffer("atomic_numbers", deepcopy(mace_model.atomic_numbers))
         self.register_buffer("r_max", deepcopy(mace_model.r_max))
@@ -259,10 +271,10 @@ class OptimizedInvariantMACE(torch.nn.Module):
 
         node_es_list, node_feats_list = [], []
         for interaction, product, readout, edge_spline in zip(self.interactions, self.products, self.readouts, self.edge_splines):
-            edge_feats = edge_spline.forward(lengths32)
+            edge_feats = None if self.fused_radial else edge_spline.forward(lengths32)
             node_feats, sc = interaction(node_attrs=node_attrs32, node_feats=node_feats.float(), edge_attrs=edge_attrs,
                                          edge_feats=edge_feats, edge_index=data["edge_index"], sender=sender,
-                                         receiver=receiver)
+                                         receiver=receiver, edge_lengths=lengths32, edge_spline=edge_spline)
             node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types).double()
             node_feats_list.append(node_feats)
             node_es_list.append(readout(node_feats, node_heads)[num_atoms_arange, node_heads])

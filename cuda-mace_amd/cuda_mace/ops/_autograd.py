@@ -95,6 +95,41 @@ class InvariantMessagePassingTPAutograd(torch.autograd.Function):
 
 
 # ------------------------------------------------------------------------------------------------
+class InvariantMessagePassingSplineTPAutograd(torch.autograd.Function):
+    """Message passing whose radial weights are evaluated in-kernel from the spline table: equivalent to
+    CubicSplineAutograd followed by InvariantMessagePassingTPAutograd, without R / grad_R in memory.
+    Differentiable in X, Y and the edge lengths r."""
+
+    @staticmethod
+    def forward(ctx, X, Y, r, r_knots, coeffs, r_width, r_max, sender_list, receiver_list, nnodes):
+        _require(X.dtype == F32 and Y.dtype == F32 and r.dtype == F32 and coeffs.dtype == F32 and r_knots.dtype == F32,
+                 "fused message passing: fp32 tensors expected")
+        _require(sender_list.dtype == I32 and receiver_list.dtype == I32, "fused message passing: int32 edge lists expected")
+        _require(Y.dim() == 2 and Y.shape[0] == 16, "fused message passing: Y must be [16, nedges]")
+        _require(X.dim() == 2 and X.shape[1] % 32 == 0, "fused message passing: X must be [nnodes, C] with C % 32 == 0")
+        nnodes = int(nnodes)
+        first_occ = csr_of(receiver_list, nnodes)
+        Xc, Yc, rc = X.contiguous(), Y.contiguous(), r.contiguous().view(-1)
+        out = cabi.mp_spline_forward(Xc, Yc, rc, r_knots, coeffs, r_width, r_max, sender_list, first_occ, nnodes)
+        ctx.save_for_backward(Xc, Yc, rc, r_knots, coeffs, sender_list, first_occ)
+        ctx.nnodes, ctx.r_width, ctx.r_max, ctx.r_shape = nnodes, float(r_width), float(r_max), r.shape
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        X, Y, r, r_knots, coeffs, sender, first_occ = ctx.saved_tensors
+        need_x, need_y, need_r = ctx.needs_input_grad[:3]
+        perm = off = None
+        if need_x:
+            perm, off = sender_view_of(sender, ctx.nnodes)
+        gX, gY, gr = cabi.mp_spline_backward(X, Y, r, r_knots, coeffs, ctx.r_width, ctx.r_max, grad_out.contiguous(), sender,
+                                             first_occ, perm, off, ctx.nnodes, need_gX=need_x, need_gY=need_y, need_gr=need_r)
+        if gr is not None:
+            gr = gr.view(ctx.r_shape)
+        return gX, gY, gr, None, None, None, None, None, None, None
+
+
+# ------------------------------------------------------------------------------------------------
 class EdgeGeometryAutograd(torch.autograd.Function):
     """(positions [N,3], shifts [E,3], row_a int32 [E] non-decreasing, row_b int32 [E]) -> (vectors fp32 [E,3],
     lengths fp32 [E]) with vectors = positions[row_b] - positions[row_a] + shifts evaluated in fp64.

@@ -18,3 +18,13 @@ class InvariantMessagePassingTP(torch.nn.Module):
 
     def forward(self, node_feats, edge_attrs, tp_weights, sender_list, receiver_list, nnodes):
         return self.cuda_obj.forward(node_feats, edge_attrs, tp_weights, sender_list, receiver_list, int(nnodes))
+
+    def forward_spline(self, node_feats, edge_attrs, edge_lengths, spline, sender_list, receiver_list, nnodes):
+        """Same result as forward(node_feats, edge_attrs, spline(edge_lengths).view(E, 4, C), ...) with the radial
+        weights evaluated inside the kernels from `spline` (a cuda_mace.ops.CubicSpline): the [nedges, 4, C] weights
+        and their gradient are never materialised.  Not part of the reference's interface."""
+        from ._autograd import InvariantMessagePassingSplineTPAutograd
+
+        return InvariantMessagePassingSplineTPAutograd.apply(
+            node_feats, edge_attrs, edge_lengths, spline.r_knots, spline.coefficients, spline._h, spline._rmax,
+            sender_list, receiver_list, int(nnodes))

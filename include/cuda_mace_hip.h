@@ -95,6 +95,27 @@ int cm_mp_backward(const float *X, const float *Y, const float *R, const float *
                    float *gX, float *gY, float *gR, float *edge_scratch, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Message passing with the radial weights evaluated in-kernel from the cubic-spline table:
+ *   out[n, m, c] = sum_{e -> n} X[sender[e], c] * Y[m, e] * R(r[e])[l(m) * channels + c]
+ * with R(r) exactly what cm_spline_forward computes (coeffs [nknots - 1, 4, 4 * channels], zero beyond
+ * r_max).  It fuses the reference's CubicSpline call and its InvariantMessagePassingTP call
+ * (models/InvariantMACE.py:320 and :105-112; kernels cuda/src/cubic_spline_impl.cu:5-107 and
+ * cuda/src/invariant_message_passing_impl.cu:74-399) so that R[nedges, 4, channels], dR/dr and grad_R are
+ * never written to or read from HBM.  The backward returns grad_r[e] = sum_j grad_R[e, j] * dR/dr[e, j]
+ * directly (may be NULL), next to gY and gX as in cm_mp_backward.
+ */
+int cm_mp_spline_forward(const float *X, const float *Y, const float *r, const float *r_knots,
+                         const float *coeffs, int nknots, float r_width, float r_max,
+                         const int32_t *sender, const int32_t *first_occ, int64_t nnodes,
+                         int64_t nedges, int channels, float *out, cm_stream_t stream);
+int cm_mp_spline_backward(const float *X, const float *Y, const float *r, const float *r_knots,
+                          const float *coeffs, int nknots, float r_width, float r_max,
+                          const float *grad_out, const int32_t *sender, const int32_t *first_occ,
+                          const int32_t *sender_perm, const int32_t *sender_offsets, int64_t nnodes,
+                          int64_t nedges, int channels, float *gX, float *gY, float *grad_r,
+                          float *edge_scratch, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Real spherical harmonics l <= 3 of normalised edge vectors, sqrt(4 pi) ("component")
  * normalisation, input axes permuted as (x, y, z) = (in[2], in[0], in[1]).
  * Replaces jit_spherical_harmonics / jit_spherical_harmonics_backward

@@ -20,12 +20,12 @@ def _say(*a):
     print(*a, flush=True)
 
 
-def _build(channels, numbers, data, seed):
+def _build(channels, numbers, data, seed, fused=True):
     from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
 
     avg = data["edge_index"].shape[1] / data["positions"].shape[0]
     up = SyntheticInvariantMACE(channels=channels, atomic_numbers=numbers, avg_num_neighbors=avg, seed=seed)
-    return up.export_params(), OptimizedInvariantMACE(up, device="cuda")
+    return up.export_params(), OptimizedInvariantMACE(up, device="cuda", fused_radial=fused)
 
 
 def _compare(params, model, data):
@@ -48,17 +48,21 @@ def test_cluster_config1(cabi):
     data = make_system(21, 4, seed=0, density=None, cluster_box=8.0)
     params, model = _build(64, (1, 6, 7, 8), data, seed=0)
     out, ref = _compare(params, model, data)
+    _, unfused = _build(64, (1, 6, 7, 8), data, seed=0, fused=False)
+    _compare(params, unfused, data)
     assert out["energy"].shape == (1,) and out["forces"].shape == (21, 3)
     assert set(out) == {"energy", "node_energy", "interaction_energy", "forces", "virials", "stress", "hessian",
                         "displacement", "node_feats", "edge_forces"}
 
 
+@pytest.mark.parametrize("fused", [True, False], ids=["fused_radial", "tabulated_radial"])
 @pytest.mark.parametrize("natoms,channels,seed", [(300, 96, 1), (400, 128, 2), (250, 192, 3)])
-def test_periodic_box(cabi, natoms, channels, seed):
-    """Periodic boxes at the benchmark density (0.1 atoms/A^3, about 52 neighbours), 10 elements."""
-    _say("model periodic: N=%d C=%d seed=%d" % (natoms, channels, seed))
+def test_periodic_box(cabi, natoms, channels, seed, fused):
+    """Periodic boxes at the benchmark density (0.1 atoms/A^3, about 52 neighbours), 10 elements; with the radial
+    spline evaluated inside the message-passing kernels and with the reference's separate spline step."""
+    _say("model periodic: N=%d C=%d seed=%d fused=%s" % (natoms, channels, seed, fused))
     data = make_system(natoms, 10, seed=seed, density=0.1)
-    params, model = _build(channels, tuple(range(1, 11)), data, seed=seed)
+    params, model = _build(channels, tuple(range(1, 11)), data, seed=seed, fused=fused)
     _compare(params, model, data)
 
 
