@@ -328,14 +328,18 @@ def symcon_builtin_structure():
     return m3, m2
 
 
-def symcon_forward(X, node_perm, group_offsets, mono3, mono2, T3, T2, T1, want_grad: bool = True, builtin: bool = False):
-    """builtin=True: the monomial lists are the ones compiled into the library; the unrolled kernel is used."""
+def symcon_forward(X, node_perm, group_offsets, mono3, mono2, T3, T2, T1, want_grad: bool = True, builtin: bool = False,
+                   zero_init: bool = True):
+    """builtin=True: the monomial lists are the ones compiled into the library; the unrolled kernel is used.
+    zero_init=False skips clearing the outputs: rows of nodes that are in no group are then undefined (every node is in
+    a group when all element indices are in range)."""
     N, sixteen, C = X.shape
     if sixteen != 16:
         raise CudaMaceError("symmetric contraction: X must be [N,16,C]")
     ne = T1.shape[0]
-    out = torch.zeros(N, C, dtype=F32, device=X.device)
-    grad = torch.zeros(N, 16, C, dtype=F32, device=X.device) if want_grad else None
+    alloc = torch.zeros if zero_init else torch.empty
+    out = alloc(N, C, dtype=F32, device=X.device)
+    grad = alloc(N, 16, C, dtype=F32, device=X.device) if want_grad else None
     _check(
         lib.cm_symcon_forward(
             _dev(X, F32, "X"), _dev(node_perm, I32, "node_perm"), _dev(group_offsets, I32, "group_offsets"),

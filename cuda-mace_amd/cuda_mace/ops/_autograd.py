@@ -279,6 +279,8 @@ class SymmetricContractionAutograd(torch.autograd.Function):
         _require(X.dim() == 3 and X.shape[1] == 16 and X.shape[2] % 32 == 0,
                  "symmetric contraction: X must be [nnodes, 16, C] with C % 32 == 0")
         _require(atom_types.dtype == I32, "symmetric contraction: int32 atom_types expected")
+        # element indices must lie in [0, nelements), as in the reference (which would read weights out of bounds
+        # otherwise); rows of nodes with an index outside that range are left unwritten here
         dev = X.device
 
         def build_structure():
@@ -301,7 +303,7 @@ class SymmetricContractionAutograd(torch.autograd.Function):
 
         perm, off = groups_of(atom_types, ne)
         want_grad = X.requires_grad
-        out, grad = cabi.symcon_forward(X.contiguous(), perm, off, m3, m2, T3, T2, T1, want_grad=want_grad, builtin=builtin)
+        out, grad = cabi.symcon_forward(X.contiguous(), perm, off, m3, m2, T3, T2, T1, want_grad=want_grad, builtin=builtin, zero_init=False)
         if want_grad:
             ctx.save_for_backward(grad)
         return out.view(X.shape[0], 1, X.shape[2])
