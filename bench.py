@@ -24,6 +24,16 @@ sys.path.insert(0, os.path.join(ROOT, "cuda-mace_amd"))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per launch at the default workload (25 000 atoms, 128 channels) from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for a 1 GiB copy (factors 2.000 and 1.000); the counter
+# summary with the commands is kept with the other profile summaries.  Null for any other workload.
+MEASURED_TRAFFIC = {
+    "mp_forward_kernel<128>": 3563800000,
+    "mp_backward_edge_kernel<128,true,true,false>": 6331300000,
+    "mp_spline_forward_kernel<128>": 939900000,
+    "mp_spline_backward_edge_kernel<128,true,true,false>": 1026000000,
+}
+
 
 def mp_algorithmic_bytes(N, E, C):
     """Each operand touched once.  Tabulated radial weights R[E,4,C] (the reference's op): forward reads X, Y, R,
@@ -35,6 +45,54 @@ def mp_algorithmic_bytes(N, E, C):
     fwd_fused = 4 * (17 * E + 17 * N * C) + 4 * E + 8 * N + table
     bwd_fused = 4 * (34 * E + 17 * N * C) + 4 * E + 8 * N + table
     return fwd, bwd_edge, fwd_fused, bwd_fused
+
+
+def isolated_ops(args, torch, cabi, make_system, reps=3):
+    """A reference copy (reads and writes `copy_bytes` each) followed by the four message-passing kernels on random
+    operands at the benchmark shape; prints one line per kernel with its average duration."""
+    import numpy as np
+
+    N, C = args.atoms, args.channels
+    data = make_system(N, args.elements, seed=0, density=0.1)
+    rcv = data["edge_index"][0].int().cuda().contiguous()
+    snd = data["edge_index"][1].int().cuda().contiguous()
+    E = rcv.numel()
+    g = torch.Generator(device="cuda").manual_seed(0)
+    X = torch.randn(N, C, device="cuda", generator=g)
+    Y = torch.randn(16, E, device="cuda", generator=g)
+    R = torch.randn(E, 4, C, device="cuda", generator=g)
+    G = torch.randn(N, 16, C, device="cuda", generator=g)
+    r = torch.rand(E, device="cuda", generator=g) * 4.0 + 0.9
+    kn, h = np.linspace(1e-12, 6.0, 256, retstep=True)
+    knots = torch.tensor(kn, dtype=torch.float32, device="cuda")
+    coeffs = torch.randn(255, 4, 4 * C, device="cuda", generator=g)
+    fo = cabi.first_occurences(rcv, N)
+    copy_bytes = 1 << 30
+    src = torch.empty(copy_bytes // 4, dtype=torch.float32, device="cuda").normal_(generator=g)
+    dst = torch.empty_like(src)
+    fwd_b, bwd_b, fwd_fb, bwd_fb = mp_algorithmic_bytes(N, E, C)
+    cases = [
+        ("copy (reads %d B, writes %d B)" % (copy_bytes, copy_bytes), 2 * copy_bytes, lambda: dst.copy_(src)),
+        ("mp_forward_kernel<%d>" % C, fwd_b, lambda: cabi.mp_forward(X, Y, R, snd, fo, N)),
+        ("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b,
+         lambda: cabi.mp_backward(X, Y, R, G, snd, fo, None, None, N, need_gX=False)),
+        ("mp_spline_forward_kernel<%d>" % C, fwd_fb,
+         lambda: cabi.mp_spline_forward(X, Y, r, knots, coeffs, float(h), 5.0, snd, fo, N)),
+        ("mp_spline_backward_edge_kernel<%d,true,true,false>" % C, bwd_fb,
+         lambda: cabi.mp_spline_backward(X, Y, r, knots, coeffs, float(h), 5.0, G, snd, fo, None, None, N, need_gX=False)),
+    ]
+    print("# isolated ops at N=%d E=%d C=%d" % (N, E, C), flush=True)
+    for name, nbytes, fn in cases:
+        fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / reps
+        print("%-60s %9.1f us  algorithmic %12d B  %8.1f GB/s" % (name, ms * 1e3, nbytes, nbytes / ms / 1e6), flush=True)
 
 
 def main():
@@ -49,6 +107,9 @@ def main():
     ap.add_argument("--tabulated-radial", action="store_true",
                     help="keep the reference's separate spline step (R[E,4,C] in HBM) instead of the fused kernels")
     ap.add_argument("--cpu-atoms", type=int, default=1500, help="size of the box the CPU baseline is timed on")
+    ap.add_argument("--isolated-ops", action="store_true",
+                    help="instead of the model step, launch a plain copy of known size and each message-passing kernel a few "
+                         "times at the benchmark shape (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -67,6 +128,9 @@ def main():
     from cuda_mace.utils.synthetic import make_system, to_device
 
     N, C, ne = args.atoms, args.channels, args.elements
+    if args.isolated_ops:
+        isolated_ops(args, torch, cabi, make_system)
+        return
     t0 = time.time()
     data_cpu = make_system(N, ne, seed=0, density=0.1)
     E = int(data_cpu["edge_index"].shape[1])
@@ -122,27 +186,30 @@ def main():
         ts = [s.elapsed_time(e) for s, e in events[name]]
         return sum(ts) / len(ts) if ts else None
 
-    def entry(nbytes, ms, **extra):
+    default_workload = (N, C, ne) == (25000, 128, 10)
+
+    def entry(kernel, nbytes, ms, **extra):
         gbps = nbytes / (ms * 1e-3) / 1e9
-        d = {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes_per_launch": nbytes,
-             "avg_launch_ms": round(ms, 4)}
+        d = {"kernel": kernel, "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+             "frac": round(gbps / HBM_PEAK_GBPS, 4),
+             "traffic": MEASURED_TRAFFIC.get(kernel) if default_workload else None,
+             "algorithmic_bytes_per_launch": nbytes, "avg_launch_ms": round(ms, 4)}
         d.update(extra)
         return d
 
     fwd_b, bwd_b, fwd_fb, bwd_fb = mp_algorithmic_bytes(N, E, C)
     t_bwd, t_fwd = avg_ms(bwd_name), avg_ms(fwd_name)
     if fused:
-        roofline = entry(bwd_fb, t_bwd, kernel="mp_spline_backward_edge_kernel<%d,true,true,false>" % C,
+        roofline = entry("mp_spline_backward_edge_kernel<%d,true,true,false>" % C, bwd_fb, t_bwd,
                          launches_timed=len(events[bwd_name]),
                          note="radial weights come from the 2 MB spline table in L2 (16 coefficient loads of 16 B per lane and "
                               "edge), so this kernel is bounded by L2 bandwidth, not HBM; see roofline_other_kernels for the "
                               "HBM-bound message passing with tabulated R[E,4,C]")
-        others = {"mp_spline_forward_kernel<%d>" % C: entry(fwd_fb, t_fwd)}
+        others = [entry("mp_spline_forward_kernel<%d>" % C, fwd_fb, t_fwd)]
     else:
-        roofline = entry(bwd_b, t_bwd, kernel="mp_backward_edge_kernel<%d,true,true,false>" % C,
+        roofline = entry("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b, t_bwd,
                          launches_timed=len(events[bwd_name]))
-        others = {"mp_forward_kernel<%d>" % C: entry(fwd_b, t_fwd)}
+        others = [entry("mp_forward_kernel<%d>" % C, fwd_b, t_fwd)]
 
     # the message-passing op with the reference's signature (tabulated R[E,4,C]) at the same shape, timed on its own
     def isolated_mp():
@@ -172,8 +239,9 @@ def main():
 
     if fused:
         tf, tb = isolated_mp()
-        others["mp_forward_kernel<%d> (isolated op, tabulated R)" % C] = entry(fwd_b, tf)
-        others["mp_backward_edge_kernel<%d,true,true,false> (isolated op, tabulated R)" % C] = entry(bwd_b, tb)
+        others.append(entry("mp_forward_kernel<%d>" % C, fwd_b, tf, context="isolated op with tabulated R[E,4,C]"))
+        others.append(entry("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b, tb,
+                            context="isolated op with tabulated R[E,4,C]"))
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
