@@ -63,6 +63,8 @@ __device__ __forceinline__ void st4_stream(float *p, f4 v) {
   __builtin_nontemporal_store(v, reinterpret_cast<f4 *>(p));
 }
 __device__ __forceinline__ float hsum4(f4 a) { return (a.x + a.y) + (a.z + a.w); }
+// a . b as one multiply and three fused multiply-adds
+__device__ __forceinline__ float dot4(f4 a, f4 b) { return fmaf(a.w, b.w, fmaf(a.z, b.z, fmaf(a.y, b.y, a.x * b.x))); }
 __device__ __forceinline__ f4 shfl_down4(f4 v, int delta) {
   f4 r;
   r.x = __shfl_down(v.x, delta);

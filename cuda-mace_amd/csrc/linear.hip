@@ -2,6 +2,9 @@
 //
 //   OUT[n, m, :] = scale * X[n, m, :] . W[g(n)][l(m)]      (scale = 1/sqrt(K) in the model)
 //
+// for features with 16 components per node (l(m) = floor(sqrt(m)), four weight blocks per group) or with a
+// single scalar component per node (one weight block per group).
+//
 // A workgroup of four wavefronts owns a tile of 128 nodes x one component m x all Nout columns, so
 // every row of the tile uses the same K x Nout weight block W[g][l(m)].  K is walked in chunks of 32:
 // the X rows of the tile (each chunk of a row is one 128-byte line) and the matching columns of the
@@ -30,8 +33,8 @@ template <int NT>  // Nout = 32 * NT
 __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__restrict__ X, const float *__restrict__ WT,
                                                                const int32_t *__restrict__ node_perm,
                                                                const int32_t *__restrict__ group_offsets, int nnodes,
-                                                               int ngroups, int K, float scale,
-                                                               float *__restrict__ OUT) {
+                                                               int ngroups, int zero_last_group, int ncomp, int K,
+                                                               float scale, float *__restrict__ OUT) {
   constexpr int NOUT = 32 * NT;
   __shared__ __attribute__((aligned(16))) float sA[kTileNodes * kLd];
   __shared__ __attribute__((aligned(16))) float sB[NOUT * kLd];
@@ -40,8 +43,9 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
   const int wave = tid / kWave;
-  const int m = blockIdx.y;  // component 0..15
-  const int l = l_of_m(m);
+  const int m = blockIdx.y;  // component 0..ncomp-1
+  const int l = ncomp == 1 ? 0 : l_of_m(m);
+  const int nblocks = ncomp == 1 ? 1 : 4;  // weight blocks per group
 
   // locate (group, first position in the grouped node order) of this tile
   int tile = blockIdx.x;
@@ -76,7 +80,15 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
   }
   __syncthreads();
 
-  const float *Wg = WT + (static_cast<int64_t>(g) * 4 + l) * NOUT * K;  // [NOUT, K]
+  if (zero_last_group && g == ngroups - 1) {
+    // rows that belong to no weight group: defined as zero
+    for (int i = tid; i < kTileNodes * NOUT; i += kWaves * kWave) {
+      const int node = sNode[i / NOUT];
+      if (node >= 0) OUT[(static_cast<int64_t>(node) * ncomp + m) * NOUT + i % NOUT] = 0.f;
+    }
+    return;
+  }
+  const float *Wg = WT + (static_cast<int64_t>(g) * nblocks + l) * NOUT * K;  // [NOUT, K]
 
   v16f acc[NT];
 #pragma unroll
@@ -100,7 +112,7 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
     for (int i = 0; i < A_PASSES; ++i) {
       const int node = sNode[32 * i + srow];
       pa[i] = zero4();
-      if (node >= 0) pa[i] = ld4_stream(X + (static_cast<int64_t>(node) * 16 + m) * K + kc + scol);
+      if (node >= 0) pa[i] = ld4_stream(X + (static_cast<int64_t>(node) * ncomp + m) * K + kc + scol);
     }
 #pragma unroll
     for (int i = 0; i < B_PASSES; ++i) pb[i] = ld4(Wg + static_cast<int64_t>(32 * i + srow) * K + kc + scol);
@@ -135,7 +147,7 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
     const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
     const int node = sNode[row];
     if (node >= 0) {
-      float *op = OUT + (static_cast<int64_t>(node) * 16 + m) * NOUT + mrow;
+      float *op = OUT + (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
 #pragma unroll
       for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
     }
@@ -144,10 +156,10 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
 
 template <int NT>
 int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
-           int K, float scale, float *OUT, hipStream_t st) {
+           int zero_last_group, int ncomp, int K, float scale, float *OUT, hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
-  hipLaunchKernelGGL(linear_kernel<NT>, dim3(static_cast<unsigned>(tiles), 16), dim3(kWaves * kWave), 0, st, X, WT, perm,
-                     offs, static_cast<int>(nnodes), ngroups, K, scale, OUT);
+  hipLaunchKernelGGL(linear_kernel<NT>, dim3(static_cast<unsigned>(tiles), ncomp), dim3(kWaves * kWave), 0, st, X, WT, perm,
+                     offs, static_cast<int>(nnodes), ngroups, zero_last_group, ncomp, K, scale, OUT);
   return check_launch("cm_linear");
 }
 
@@ -155,7 +167,11 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
 }  // namespace cm
 
 extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_perm, const int32_t *group_offsets,
-                         int64_t nnodes, int ngroups, int K, int Nout, float scale, float *OUT, cm_stream_t stream) {
+                         int64_t nnodes, int ngroups, int zero_last_group, int ncomp, int K, int Nout, float scale,
+                         float *OUT, cm_stream_t stream) {
+  CM_REQUIRE(ncomp == 1 || ncomp == 16, "cm_linear: ncomp=%d must be 1 or 16", ncomp);
+  CM_REQUIRE(!zero_last_group || (group_offsets != nullptr && ngroups >= 2),
+             "cm_linear: a zero group needs node_perm / group_offsets and at least one weight group before it");
   CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 16, "cm_linear: nnodes out of range");
   CM_REQUIRE(K >= 32 && K <= 256 && K % 32 == 0, "cm_linear: K=%d must be a multiple of 32 in [32, 256]", K);
   CM_REQUIRE(Nout >= 32 && Nout <= 256 && Nout % 32 == 0, "cm_linear: Nout=%d must be a multiple of 32 in [32, 256]", Nout);
@@ -166,14 +182,14 @@ extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_p
   CM_REQUIRE(X && W_T && OUT, "cm_linear: NULL pointer");
   hipStream_t st = cm::as_stream(stream);
   switch (Nout / 32) {
-    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
-    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
-    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
-    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
-    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
-    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
-    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
-    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, K, scale, OUT, st);
+    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
+    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
+    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
+    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
+    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
+    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
+    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
+    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
   }
   return CM_EINVAL;
 }

@@ -206,22 +206,22 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
       if constexpr (WANT_GY) {
         const f4 t0 = x * r0, t1 = x * r1, t2 = x * r2, t3 = x * r3;
         float p[16];
-        p[0] = hsum4(g[0] * t0);
-        p[1] = hsum4(g[1] * t1);
-        p[2] = hsum4(g[2] * t1);
-        p[3] = hsum4(g[3] * t1);
-        p[4] = hsum4(g[4] * t2);
-        p[5] = hsum4(g[5] * t2);
-        p[6] = hsum4(g[6] * t2);
-        p[7] = hsum4(g[7] * t2);
-        p[8] = hsum4(g[8] * t2);
-        p[9] = hsum4(g[9] * t3);
-        p[10] = hsum4(g[10] * t3);
-        p[11] = hsum4(g[11] * t3);
-        p[12] = hsum4(g[12] * t3);
-        p[13] = hsum4(g[13] * t3);
-        p[14] = hsum4(g[14] * t3);
-        p[15] = hsum4(g[15] * t3);
+        p[0] = dot4(g[0], t0);
+        p[1] = dot4(g[1], t1);
+        p[2] = dot4(g[2], t1);
+        p[3] = dot4(g[3], t1);
+        p[4] = dot4(g[4], t2);
+        p[5] = dot4(g[5], t2);
+        p[6] = dot4(g[6], t2);
+        p[7] = dot4(g[7], t2);
+        p[8] = dot4(g[8], t2);
+        p[9] = dot4(g[9], t3);
+        p[10] = dot4(g[10], t3);
+        p[11] = dot4(g[11], t3);
+        p[12] = dot4(g[12], t3);
+        p[13] = dot4(g[13], t3);
+        p[14] = dot4(g[14], t3);
+        p[15] = dot4(g[15], t3);
         slot_reduce16<K::SW>(p, cl);
         if constexpr (K::SW >= 16) {
           if (cl < 16) sGY[myrev * kChunk + j] = p[0];

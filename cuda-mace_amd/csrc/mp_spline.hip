@@ -15,6 +15,14 @@
 
 #include "mp_common.hpp"
 
+// waves per SIMD the register allocator must leave room for (forward, backward edge pass)
+#ifndef CM_FUSED_FWD_WAVES
+#define CM_FUSED_FWD_WAVES 3
+#endif
+#ifndef CM_FUSED_BWD_WAVES
+#define CM_FUSED_BWD_WAVES 3
+#endif
+
 namespace cm {
 namespace {
 
@@ -55,7 +63,7 @@ struct MRange {
 // forward
 // -----------------------------------------------------------------------------------------------
 template <int C>
-__global__ __launch_bounds__(kWave) void mp_spline_forward_kernel(const float *__restrict__ X,
+__global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_kernel(const float *__restrict__ X,
                                                                  const float *__restrict__ Y, Spline sp,
                                                                  const int32_t *__restrict__ sender,
                                                                  const int32_t *__restrict__ first_occ, int nnodes,
@@ -132,7 +140,7 @@ __global__ __launch_bounds__(kWave) void mp_spline_forward_kernel(const float *_
 // backward, edge pass: gY, g_r and the per-edge contribution to gX
 // -----------------------------------------------------------------------------------------------
 template <int C, bool WANT_GY, bool WANT_GR, bool WANT_GX>
-__global__ __launch_bounds__(kWave) void mp_spline_backward_edge_kernel(
+__global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_edge_kernel(
     const float *__restrict__ X, const float *__restrict__ Y, Spline sp, const float *__restrict__ G,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges,
     float *__restrict__ gY, float *__restrict__ g_r, float *__restrict__ gXe) {
@@ -202,7 +210,7 @@ __global__ __launch_bounds__(kWave) void mp_spline_backward_edge_kernel(
         if constexpr (WANT_GY) {
           const f4 t = x * rl;
 #pragma unroll
-          for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) p[m] = hsum4(g[m] * t);
+          for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) p[m] = dot4(g[m], t);
         }
         if constexpr (WANT_GX) gxe += rl * q;
         if constexpr (WANT_GR) gr4 += (x * q) * drl;

@@ -18,7 +18,7 @@ import torch
 
 from cuda_mace.ops.cubic_spline import CubicSpline
 from cuda_mace.ops.invariant_message_passing import InvariantMessagePassingTP
-from cuda_mace.ops.linear import ElementalLinear, Linear
+from cuda_mace.ops.linear import ElementalLinear, Linear, ScalarElementalLinear
 from cuda_mace.ops.spherical_harmonics import SphericalHarmonics
 from cuda_mace.ops.symmetric_contraction import SymmetricContraction as CUDAContraction
 from cuda_mace.ops._autograd import EdgeGeometryAutograd, _cached
@@ -128,6 +128,16 @@ def element_linear_to_cuda(skip_tp):
     return ElementalLinear(skip_tp.__dict__["irreps_in1"], skip_tp.__dict__["irreps_out"], instructions, ws, num_elements)
 
 
+def scalar_skip_to_cuda(skip_tp):
+    """The residual skip connection of the second layer (a fully connected tensor product of scalar features with the
+    one-hot species, weight [C, ne, C], normalised by 1/sqrt(C * ne)) as a per-element linear on the MFMA kernel."""
+    num_elements = skip_tp.__dict__["irreps_in2"].dim
+    n_in = skip_tp.__dict__["irreps_in1"].num_irreps
+    n_out = skip_tp.__dict__["irreps_out"].num_irreps
+    ws = skip_tp.weight.data.double().reshape(n_in, num_elements, n_out).permute(1, 0, 2) / sqrt(num_elements)
+    return ScalarElementalLinear(ws)
+
+
 class _FloatLinearView:
     """Presents an e3nn-Linear-like module with fp32 weights without converting the module in place; `divide_by`
     folds the reference's `linear(message) / avg_num_neighbors` (models/InvariantMACE.py:114) into the weights."""
@@ -190,7 +200,7 @@ class InvariantResidualInteraction(torch.nn.Module):
         self.linear_up = linear_matmul(inter.linear_up)
         self.linear = Linear(_FloatLinearView(inter.linear, divide_by=inter.avg_num_neighbors))
         self.tp = InvariantMessagePassingTP()
-        self.skip_tp = deepcopy(inter.skip_tp).float()
+        self.skip_tp = scalar_skip_to_cuda(inter.skip_tp)
         self.avg_num_neighbors = inter.avg_num_neighbors
 
     def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,

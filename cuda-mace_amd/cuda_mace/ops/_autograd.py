@@ -57,8 +57,7 @@ def groups_of_one_hot(one_hot: torch.Tensor):
         mask = one_hot == 1
         elem = mask.to(torch.int8).argmax(dim=1).to(I32)
         elem = torch.where(mask.any(dim=1), elem, torch.full_like(elem, ne))
-        perm, off = cabi.stable_key_sort(elem.contiguous(), ne + 1)
-        return perm, off[: ne + 1].contiguous()
+        return cabi.stable_key_sort(elem.contiguous(), ne + 1)  # group ne collects the rows without an element
 
     return _cached(one_hot, "_cm_groups", None, build)
 
@@ -220,18 +219,18 @@ class ElementalLinearAutograd(torch.autograd.Function):
     @staticmethod
     def forward(ctx, X, W, W_T, one_hot_encoding):
         _require(X.dtype == F32 and W.dtype == F32 and W_T.dtype == F32, "elemental linear: fp32 tensors expected")
-        _require(X.dim() == 3 and X.shape[1] == 16, "elemental linear: X must be [nnodes, 16, K]")
+        _require((X.dim() == 3 and X.shape[1] == 16) or X.dim() == 2, "elemental linear: X must be [nnodes, 16, K] or [nnodes, K]")
         _require(one_hot_encoding.dim() == 2 and one_hot_encoding.shape[1] == W.shape[0],
                  "elemental linear: one_hot must be [nnodes, nelements]")
         perm, off = groups_of_one_hot(one_hot_encoding)
         ctx.save_for_backward(W, perm, off)
-        ctx.scale = 1.0 / float(X.shape[2]) ** 0.5
-        return cabi.linear(X.contiguous(), W_T, perm, off, scale=ctx.scale)
+        ctx.scale = 1.0 / float(X.shape[-1]) ** 0.5
+        return cabi.linear(X.contiguous(), W_T, perm, off, scale=ctx.scale, zero_last_group=True)
 
     @staticmethod
     def backward(ctx, grad_out):
         W, perm, off = ctx.saved_tensors
-        return cabi.linear(grad_out.contiguous(), W, perm, off, scale=ctx.scale), None, None, None
+        return cabi.linear(grad_out.contiguous(), W, perm, off, scale=ctx.scale, zero_last_group=True), None, None, None
 
 
 # ------------------------------------------------------------------------------------------------

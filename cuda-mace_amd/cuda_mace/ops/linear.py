@@ -65,3 +65,20 @@ class ElementalLinear(torch.nn.Module):
 
     def forward(self, x, y):
         return self.cuda_obj.forward(x, self.weights, self.weights_transposed, y)
+
+
+class ScalarElementalLinear(torch.nn.Module):
+    """Per-element channel mixing of scalar features: out[n, :] = x[n, :] @ W[element(n)] / sqrt(K) for x [nnodes, K],
+    y the one-hot species matrix.  Same kernels as ElementalLinear with a single component per node.  The reference
+    leaves this case (the residual skip connection of the second layer) to the upstream e3nn tensor product
+    (models/InvariantMACE.py:133, 149)."""
+
+    def __init__(self, weights: torch.Tensor):
+        super().__init__()
+        self.cuda_obj = classes.linear_wmma.ElementalLinear()
+        w = weights.detach().float().contiguous()  # [ne, K, N']
+        self.register_buffer("weights", w)
+        self.register_buffer("weights_transposed", w.transpose(-1, -2).contiguous())
+
+    def forward(self, x, y):
+        return self.cuda_obj.forward(x, self.weights, self.weights_transposed, y)

@@ -174,19 +174,23 @@ int cm_spline_backward(const float *r, const float *r_knots, const float *coeffs
  * that is the true gradient only for square layers; here the caller passes the factor.
  * Replaces jit_linear and jit_elemental_linear (jit_wrappers/src/linear_wrapper.cpp:23-95, 97-191) and
  * linear_kernel_ptr / elemental_linear_kernel_ptr (cuda/src/linear_impl.cu:16-133, 134-255).
- *   X [nnodes, 16, K]; OUT [nnodes, 16, Nout];
- *   W_T [ngroups, 4, Nout, K]: the TRANSPOSED weight blocks, W_T[g][l][j][k] = W[g][l][k][j].  The
+ *   X [nnodes, ncomp, K]; OUT [nnodes, ncomp, Nout]; ncomp = 16 (l(m) = floor(sqrt(m)), four weight blocks per
+ *   group) or ncomp = 1 (scalar features, one weight block per group: the reference leaves that case to
+ *   torch.matmul / the upstream e3nn tensor product, models/InvariantMACE.py:41-53, 133, 149).
+ *   W_T [ngroups, 4 or 1, Nout, K]: the TRANSPOSED weight blocks, W_T[g][l][j][k] = W[g][l][k][j].  The
  *   reference keeps both W and W_T as module buffers (ops/linear.py:47-51); the forward passes its
  *   weights_transposed buffer here and the backward with respect to X passes its weights buffer.
  *   Plain linear: ngroups = 1, node_perm = group_offsets = NULL.
  *   Per-element linear: node_perm int32 [nnodes] lists nodes grouped by element and
  *   group_offsets int32 [ngroups + 1] delimits the groups (cm_stable_key_sort on the element
- *   index); rows of nodes that are in no group are not written.
+ *   index); rows of nodes that are in no group are not written.  With zero_last_group != 0 the last of the
+ *   ngroups groups has no weights (W_T holds ngroups - 1 groups) and its rows are written as zeros: that is
+ *   where nodes whose one-hot row names no element go.
  *   K and Nout: multiples of 32 in [32, 256].
  */
 int cm_linear(const float *X, const float *W_T, const int32_t *node_perm,
-              const int32_t *group_offsets, int64_t nnodes, int ngroups, int K, int Nout,
-              float scale, float *OUT, cm_stream_t stream);
+              const int32_t *group_offsets, int64_t nnodes, int ngroups, int zero_last_group,
+              int ncomp, int K, int Nout, float scale, float *OUT, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Symmetric contraction, correlation 3, scalar (L = 0) output, with its analytic gradient.

@@ -231,6 +231,29 @@ def test_elemental_linear(cabi, N, C, ne, seed):
     close(out, ref, 1e-5, 2e-6)
 
 
+@pytest.mark.parametrize("N,K,Nout,ne,seed", [(1, 32, 32, 1, 0), (700, 128, 128, 10, 1), (130, 96, 64, 3, 2)])
+def test_scalar_elemental_linear_and_zero_group(cabi, N, K, Nout, ne, seed):
+    """Single-component features (the layer-2 skip connection) and rows whose one-hot names no element."""
+    _say("scalar_elemental_linear", N, K, Nout, ne, seed)
+    g = torch.Generator().manual_seed(seed)
+    X = torch.randn(N, K, generator=g, dtype=torch.float64)
+    W = torch.randn(ne, K, Nout, generator=g, dtype=torch.float64)
+    elem = torch.randint(0, ne + 1, (N,), generator=g)  # value ne = "no element"
+    ref = torch.einsum("nk,nkj->nj", X, torch.cat([W, torch.zeros(1, K, Nout, dtype=torch.float64)])[elem]) / math.sqrt(K)
+    perm, off = cabi.stable_key_sort(elem.int().to(DEV), ne + 1)
+    WT = W.transpose(-1, -2).contiguous().float().to(DEV)
+    out = cabi.linear(X.float().to(DEV), WT, perm, off, zero_last_group=True)
+    close(out, ref, 1e-5, 2e-6)
+    assert float(out[(elem == ne).to(DEV)].abs().sum()) == 0.0
+    # the same through the 16-component path
+    X16 = torch.randn(N, 16, K, generator=g, dtype=torch.float64)
+    W16 = torch.randn(ne, 4, K, Nout, generator=g, dtype=torch.float64)
+    one_hot = torch.nn.functional.one_hot(elem, ne + 1)[:, :ne].double()
+    ref16 = O.elemental_linear(X16, W16, one_hot)
+    out16 = cabi.linear(X16.float().to(DEV), W16.transpose(-1, -2).contiguous().float().to(DEV), perm, off, zero_last_group=True)
+    close(out16, ref16, 1e-5, 2e-6)
+
+
 # ------------------------------------------------------------------------------------------------
 # symmetric contraction with synthetic sparse tables
 # ------------------------------------------------------------------------------------------------
