@@ -30,26 +30,28 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 MEASURED_TRAFFIC = {
     "mp_forward_kernel<128>": 3563800000,
     "mp_backward_edge_kernel<128,true,true,false>": 6331300000,
-    "mp_spline_forward_kernel<128>": 939900000,
-    "mp_spline_backward_edge_kernel<128,true,true,false>": 1026000000,
+    "mp_spline_forward_kernel<128,true>": 776800000,
+    "mp_spline_backward_edge_kernel<128,true,true,true,false>": 818300000,
 }
 
 
 def mp_algorithmic_bytes(N, E, C):
     """Each operand touched once.  Tabulated radial weights R[E,4,C] (the reference's op): forward reads X, Y, R,
     sender, CSR and writes out; the backward edge pass without gX (first layer) reads X, Y, R, grad_out, sender, CSR and
-    writes gY, gR.  Fused radial spline: R, gR are replaced by the edge lengths / their gradient and the spline table."""
+    writes gY, gR.  Fused kernels: Y, R, gY, gR are replaced by the edge vectors / their gradient and the spline table."""
     fwd = 4 * (4 * E * C + 16 * E + 17 * N * C) + 4 * E + 8 * N
     bwd_edge = 4 * (8 * E * C + 32 * E + 17 * N * C) + 4 * E + 8 * N
     table = 255 * 16 * C * 4
-    fwd_fused = 4 * (17 * E + 17 * N * C) + 4 * E + 8 * N + table
-    bwd_fused = 4 * (34 * E + 17 * N * C) + 4 * E + 8 * N + table
+    # fully fused kernels: edge vectors in (3E), out / grad_out (16NC), X (NC); the backward also writes the [E,3] gradient
+    fwd_fused = 4 * (3 * E + 17 * N * C) + 4 * E + 8 * N + table
+    bwd_fused = 4 * (6 * E + 17 * N * C) + 4 * E + 8 * N + table
     return fwd, bwd_edge, fwd_fused, bwd_fused
 
 
 def isolated_ops(args, torch, cabi, make_system, reps=3):
-    """A reference copy (reads and writes `copy_bytes` each) followed by the four message-passing kernels on random
-    operands at the benchmark shape; prints one line per kernel with its average duration."""
+    """A reference copy (reads and writes `copy_bytes` each) followed by the message-passing kernels (tabulated radial
+    weights, and fully fused from the edge vectors) on random operands at the benchmark shape; prints one line per
+    kernel with its average duration."""
     import numpy as np
 
     N, C = args.atoms, args.channels
@@ -62,7 +64,8 @@ def isolated_ops(args, torch, cabi, make_system, reps=3):
     Y = torch.randn(16, E, device="cuda", generator=g)
     R = torch.randn(E, 4, C, device="cuda", generator=g)
     G = torch.randn(N, 16, C, device="cuda", generator=g)
-    r = torch.rand(E, device="cuda", generator=g) * 4.0 + 0.9
+    vec = torch.randn(E, 3, device="cuda", generator=g)
+    vec = vec / vec.norm(dim=1, keepdim=True) * (torch.rand(E, 1, device="cuda", generator=g) * 4.0 + 0.9)
     kn, h = np.linspace(1e-12, 6.0, 256, retstep=True)
     knots = torch.tensor(kn, dtype=torch.float32, device="cuda")
     coeffs = torch.randn(255, 4, 4 * C, device="cuda", generator=g)
@@ -76,10 +79,10 @@ def isolated_ops(args, torch, cabi, make_system, reps=3):
         ("mp_forward_kernel<%d>" % C, fwd_b, lambda: cabi.mp_forward(X, Y, R, snd, fo, N)),
         ("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b,
          lambda: cabi.mp_backward(X, Y, R, G, snd, fo, None, None, N, need_gX=False)),
-        ("mp_spline_forward_kernel<%d>" % C, fwd_fb,
-         lambda: cabi.mp_spline_forward(X, Y, r, knots, coeffs, float(h), 5.0, snd, fo, N)),
-        ("mp_spline_backward_edge_kernel<%d,true,true,false>" % C, bwd_fb,
-         lambda: cabi.mp_spline_backward(X, Y, r, knots, coeffs, float(h), 5.0, G, snd, fo, None, None, N, need_gX=False)),
+        ("mp_spline_forward_kernel<%d,true>" % C, fwd_fb,
+         lambda: cabi.mp_edge_forward(X, vec, knots, coeffs, float(h), 5.0, snd, fo, N)),
+        ("mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb,
+         lambda: cabi.mp_edge_backward(X, vec, knots, coeffs, float(h), 5.0, G, snd, fo, None, None, N, need_gX=False)),
     ]
     print("# isolated ops at N=%d E=%d C=%d" % (N, E, C), flush=True)
     for name, nbytes, fn in cases:
@@ -150,7 +153,7 @@ def main():
 
     # live timing of the message-passing kernels: events on the launch stream around every forward launch and around
     # every backward edge pass that runs without the sender pass (first layer: one kernel per call)
-    fwd_name, bwd_name = ("mp_spline_forward", "mp_spline_backward") if fused else ("mp_forward", "mp_backward")
+    fwd_name, bwd_name = ("mp_edge_forward", "mp_edge_backward") if fused else ("mp_forward", "mp_backward")
     events = {fwd_name: [], bwd_name: []}
     originals = {fwd_name: getattr(cabi, fwd_name), bwd_name: getattr(cabi, bwd_name)}
 
@@ -200,12 +203,13 @@ def main():
     fwd_b, bwd_b, fwd_fb, bwd_fb = mp_algorithmic_bytes(N, E, C)
     t_bwd, t_fwd = avg_ms(bwd_name), avg_ms(fwd_name)
     if fused:
-        roofline = entry("mp_spline_backward_edge_kernel<%d,true,true,false>" % C, bwd_fb, t_bwd,
+        roofline = entry("mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb, t_bwd,
                          launches_timed=len(events[bwd_name]),
-                         note="radial weights come from the 2 MB spline table in L2 (16 coefficient loads of 16 B per lane and "
-                              "edge), so this kernel is bounded by L2 bandwidth, not HBM; see roofline_other_kernels for the "
-                              "HBM-bound message passing with tabulated R[E,4,C]")
-        others = [entry("mp_spline_forward_kernel<%d>" % C, fwd_fb, t_fwd)]
+                         note="harmonics and radial weights are evaluated in-kernel; the radial coefficients come from the 2 MB "
+                              "spline table in L2 (16 loads of 16 B per lane and edge) and the backward issues ~10k VALU "
+                              "instructions per wave, so this kernel is bounded by VALU issue and L2 bandwidth, not HBM; see "
+                              "roofline_other_kernels for the HBM-bound message passing with tabulated R[E,4,C]")
+        others = [entry("mp_spline_forward_kernel<%d,true>" % C, fwd_fb, t_fwd)]
     else:
         roofline = entry("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b, t_bwd,
                          launches_timed=len(events[bwd_name]))

@@ -11,9 +11,15 @@
 // backward) and drops them, so only 16 registers of radial data are live at a time.  The backward
 // returns the gradient with respect to the edge length directly:
 //   g_r[e] = sum_{l, c} X[s, c] * q_l[c] * dR_l/dr[c],   q_l = sum_{m in l} Y[m, e] * grad_out[n, m, c].
+//
+// The FROM_VEC variants go one step further and take the fp32 edge vectors instead of Y and r: the 16 harmonics and the
+// length are computed per edge while the chunk is staged, and the backward turns the reduced gY and g_r of an edge
+// straight into the gradient with respect to its vector (harmonics Jacobian + radial part), so Y[16, E], grad_Y and
+// grad_r never exist either.
 #include <type_traits>
 
 #include "mp_common.hpp"
+#include "sh_device.hpp"
 
 // waves per SIMD the register allocator must leave room for (forward, backward edge pass)
 #ifndef CM_FUSED_FWD_WAVES
@@ -29,6 +35,7 @@ namespace {
 using namespace mp;
 
 struct Spline {
+  const float *vec;     // [E, 3] edge vectors (FROM_VEC variants; then r is unused)
   const float *r;       // [E]
   const float *knots;   // [nknots]
   const float *coeffs;  // [nknots - 1, 4, 4C]
@@ -37,19 +44,49 @@ struct Spline {
   float r_max;
 };
 
-// Stages the knot interval (or -1 beyond the cutoff) and the offset inside it for the chunk's edges.
-__device__ __forceinline__ void stage_radial(const Spline &sp, int base, int cnt, int lane, int *sIdx, float *sXr) {
-  if (lane < cnt) {
-    const float re = sp.r[base + lane];
-    int idx = -1;
-    float x = 0.f;
-    if (re <= sp.r_max) {
-      idx = static_cast<int>(re / sp.r_width);
-      idx = idx < 0 ? 0 : (idx > sp.nknots - 2 ? sp.nknots - 2 : idx);
-      x = re - sp.knots[idx];
+// Knot interval (or -1 beyond the cutoff) and offset inside it for one edge length.
+__device__ __forceinline__ void locate(const Spline &sp, float re, int &idx, float &x) {
+  idx = -1;
+  x = 0.f;
+  if (re <= sp.r_max) {
+    idx = static_cast<int>(re / sp.r_width);
+    idx = idx < 0 ? 0 : (idx > sp.nknots - 2 ? sp.nknots - 2 : idx);
+    x = re - sp.knots[idx];
+  }
+}
+
+// Stages, for the chunk's edges, sender, Y (transposed to [edge][16]), knot interval and offset.  FROM_VEC: Y and the
+// length come from the edge vector; otherwise from the Y and r arrays.
+template <bool FROM_VEC>
+__device__ __forceinline__ void stage_edges(const float *__restrict__ Y, const int32_t *__restrict__ sender, const Spline &sp,
+                                            int64_t nedges, int base, int cnt, int lane, float *sY, int *sS, int *sIdx,
+                                            float *sXr) {
+  if constexpr (!FROM_VEC) {
+    stage_chunk(Y, sender, nedges, base, cnt, lane, sY, sS);
+    if (lane < cnt) {
+      int idx;
+      float x;
+      locate(sp, sp.r[base + lane], idx, x);
+      sIdx[lane] = idx;
+      sXr[lane] = x;
     }
-    sIdx[lane] = idx;
-    sXr[lane] = x;
+  } else {
+    if (lane < cnt) {
+      const int64_t e = base + lane;
+      sS[lane] = sender[e];
+      const float v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
+      const float re = sqrtf(v0 * v0 + v1 * v1 + v2 * v2);
+      int idx;
+      float x;
+      locate(sp, re, idx, x);
+      sIdx[lane] = idx;
+      sXr[lane] = x;
+      float y[16];
+      sh::eval(sh::direction(v0, v1, v2), y);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<f4 *>(sY + lane * 16 + 4 * q) = f4{y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]};
+    }
   }
 }
 
@@ -62,7 +99,7 @@ struct MRange {
 // -----------------------------------------------------------------------------------------------
 // forward
 // -----------------------------------------------------------------------------------------------
-template <int C>
+template <int C, bool FROM_VEC>
 __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_kernel(const float *__restrict__ X,
                                                                  const float *__restrict__ Y, Spline sp,
                                                                  const int32_t *__restrict__ sender,
@@ -89,8 +126,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
   for (int base = e0; base < e1; base += kChunk) {
     const int cnt = min(kChunk, e1 - base);
     __syncthreads();
-    stage_chunk(Y, sender, nedges, base, cnt, lane, sY, sS);
-    stage_radial(sp, base, cnt, lane, sIdx, sXr);
+    stage_edges<FROM_VEC>(Y, sender, sp, nedges, base, cnt, lane, sY, sS, sIdx, sXr);
     __syncthreads();
     if (active) {
       for (int j = slot; j < cnt; j += K::EPW) {
@@ -139,7 +175,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
 // -----------------------------------------------------------------------------------------------
 // backward, edge pass: gY, g_r and the per-edge contribution to gX
 // -----------------------------------------------------------------------------------------------
-template <int C, bool WANT_GY, bool WANT_GR, bool WANT_GX>
+template <int C, bool FROM_VEC, bool WANT_GY, bool WANT_GR, bool WANT_GX>
 __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_edge_kernel(
     const float *__restrict__ X, const float *__restrict__ Y, Spline sp, const float *__restrict__ G,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges,
@@ -171,8 +207,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   for (int base = e0; base < e1; base += kChunk) {
     const int cnt = min(kChunk, e1 - base);
     __syncthreads();
-    stage_chunk(Y, sender, nedges, base, cnt, lane, sY, sS);
-    stage_radial(sp, base, cnt, lane, sIdx, sXr);
+    stage_edges<FROM_VEC>(Y, sender, sp, nedges, base, cnt, lane, sY, sS, sIdx, sXr);
     __syncthreads();
     // every lane of a slot takes part in the reductions, so the loop bound is slot-uniform
     for (int j = slot; j < cnt; j += K::EPW) {
@@ -236,58 +271,81 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
       __syncthreads();
       if (lane < cnt) {
         const int64_t e = base + lane;
-        if constexpr (WANT_GY) {
+        if constexpr (FROM_VEC) {
+          // gradient with respect to the edge vector: harmonics Jacobian applied to gY, plus g_r along the direction
+          // (gY doubles as the output pointer of the [E, 3] vector gradient in this variant)
+          const float v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
+          const sh::Direction d = sh::direction(v0, v1, v2);
+          float gy[16], gin[3];
 #pragma unroll
-          for (int m = 0; m < 16; ++m) gY[m * nedges + e] = sGY[m * kChunk + lane];
+          for (int m = 0; m < 16; ++m) gy[m] = sGY[m * kChunk + lane];
+          sh::vjp(d, gy, gin);
+          const float gr = sGr[lane];
+          gY[3 * e + 0] = gin[0] + gr * d.y;
+          gY[3 * e + 1] = gin[1] + gr * d.z;
+          gY[3 * e + 2] = gin[2] + gr * d.x;
+        } else {
+          if constexpr (WANT_GY) {
+#pragma unroll
+            for (int m = 0; m < 16; ++m) gY[m * nedges + e] = sGY[m * kChunk + lane];
+          }
+          if constexpr (WANT_GR) g_r[e] = sGr[lane];
         }
-        if constexpr (WANT_GR) g_r[e] = sGr[lane];
       }
     }
   }
 }
 
-template <int C>
+template <int C, bool FROM_VEC>
 int launch_forward(const float *X, const float *Y, const Spline &sp, const int32_t *sender, const int32_t *first_occ,
                    int64_t nnodes, int64_t nedges, float *out, hipStream_t st) {
-  hipLaunchKernelGGL(mp_spline_forward_kernel<C>, dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st, X, Y, sp, sender,
-                     first_occ, static_cast<int>(nnodes), nedges, out);
-  return check_launch("cm_mp_spline_forward");
+  hipLaunchKernelGGL((mp_spline_forward_kernel<C, FROM_VEC>), dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st, X, Y, sp,
+                     sender, first_occ, static_cast<int>(nnodes), nedges, out);
+  return check_launch(FROM_VEC ? "cm_mp_edge_forward" : "cm_mp_spline_forward");
 }
 
-template <int C, bool GY, bool GR, bool GX>
+template <int C, bool FROM_VEC, bool GY, bool GR, bool GX>
 void launch_edge(const float *X, const float *Y, const Spline &sp, const float *G, const int32_t *sender,
                  const int32_t *first_occ, int64_t nnodes, int64_t nedges, float *gY, float *g_r, float *gXe,
                  hipStream_t st) {
-  hipLaunchKernelGGL((mp_spline_backward_edge_kernel<C, GY, GR, GX>), dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st,
-                     X, Y, sp, G, sender, first_occ, static_cast<int>(nnodes), nedges, gY, g_r, gXe);
+  hipLaunchKernelGGL((mp_spline_backward_edge_kernel<C, FROM_VEC, GY, GR, GX>), dim3(static_cast<unsigned>(nnodes)),
+                     dim3(kWave), 0, st, X, Y, sp, G, sender, first_occ, static_cast<int>(nnodes), nedges, gY, g_r, gXe);
 }
 
-template <int C>
+// gY / g_r: outputs of the Y-and-r variant; in the FROM_VEC variant gY is the [E, 3] vector gradient and g_r is unused.
+template <int C, bool FROM_VEC>
 int launch_backward(const float *X, const float *Y, const Spline &sp, const float *G, const int32_t *sender,
                     const int32_t *first_occ, const int32_t *perm, const int32_t *offsets, int64_t nnodes, int64_t nedges,
                     float *gX, float *gY, float *g_r, float *gXe, hipStream_t st) {
-  const int key = (gY ? 4 : 0) | (g_r ? 2 : 0) | (gX ? 1 : 0);
-  switch (key) {
-    case 7: launch_edge<C, true, true, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
-    case 6: launch_edge<C, true, true, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
-    case 5: launch_edge<C, true, false, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
-    case 4: launch_edge<C, true, false, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
-    case 3: launch_edge<C, false, true, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
-    case 2: launch_edge<C, false, true, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
-    case 1: launch_edge<C, false, false, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
-    default: return CM_OK;
+  if constexpr (FROM_VEC) {
+    if (gY && gX) launch_edge<C, true, true, true, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st);
+    else if (gY) launch_edge<C, true, true, true, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st);
+    else if (gX) launch_edge<C, true, false, false, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st);
+    else return CM_OK;
+  } else {
+    const int key = (gY ? 4 : 0) | (g_r ? 2 : 0) | (gX ? 1 : 0);
+    switch (key) {
+      case 7: launch_edge<C, false, true, true, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+      case 6: launch_edge<C, false, true, true, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+      case 5: launch_edge<C, false, true, false, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+      case 4: launch_edge<C, false, true, false, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+      case 3: launch_edge<C, false, false, true, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+      case 2: launch_edge<C, false, false, true, false>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+      case 1: launch_edge<C, false, false, false, true>(X, Y, sp, G, sender, first_occ, nnodes, nedges, gY, g_r, gXe, st); break;
+      default: return CM_OK;
+    }
   }
-  int rc = check_launch("cm_mp_spline_backward (edge pass)");
+  int rc = check_launch(FROM_VEC ? "cm_mp_edge_backward (edge pass)" : "cm_mp_spline_backward (edge pass)");
   if (rc != CM_OK) return rc;
   if (gX) rc = mp::launch_sender_pass(C, gXe, perm, offsets, nnodes, nedges, gX, st);
   return rc;
 }
 
-int check_spline(const char *who, const float *r, const float *r_knots, const float *coeffs, int nknots, float r_width,
-                 int64_t nedges) {
+int check_spline(const char *who, const float *r_or_vec, const float *r_knots, const float *coeffs, int nknots,
+                 float r_width, int64_t nedges) {
   CM_REQUIRE(nknots >= 2, "%s: need at least two knots, got %d", who, nknots);
   CM_REQUIRE(r_width > 0.f, "%s: r_width must be positive", who);
-  CM_REQUIRE(nedges == 0 || (r && r_knots && coeffs), "%s: NULL spline operand", who);
+  CM_REQUIRE(nedges == 0 || (r_or_vec && r_knots && coeffs), "%s: NULL spline operand", who);
   return CM_OK;
 }
 
@@ -306,9 +364,9 @@ extern "C" int cm_mp_spline_forward(const float *X, const float *Y, const float 
   CM_REQUIRE(nedges == 0 || (Y && sender), "cm_mp_spline_forward: NULL edge operand");
   int rc = cm::check_spline("cm_mp_spline_forward", r, r_knots, coeffs, nknots, r_width, nedges);
   if (rc != CM_OK) return rc;
-  const cm::Spline sp{r, r_knots, coeffs, nknots, r_width, r_max};
+  const cm::Spline sp{nullptr, r, r_knots, coeffs, nknots, r_width, r_max};
   rc = CM_EINVAL;
-  CM_DISPATCH_C(channels, rc = cm::launch_forward<C_>(X, Y, sp, sender, first_occ, nnodes, nedges, out, cm::as_stream(stream)));
+  CM_DISPATCH_C(channels, rc = (cm::launch_forward<C_, false>(X, Y, sp, sender, first_occ, nnodes, nedges, out, cm::as_stream(stream))));
   return rc;
 }
 
@@ -327,9 +385,49 @@ extern "C" int cm_mp_spline_backward(const float *X, const float *Y, const float
              "cm_mp_spline_backward: gX wanted but sender_perm / sender_offsets / edge_scratch missing");
   int rc = cm::check_spline("cm_mp_spline_backward", r, r_knots, coeffs, nknots, r_width, nedges);
   if (rc != CM_OK) return rc;
-  const cm::Spline sp{r, r_knots, coeffs, nknots, r_width, r_max};
+  const cm::Spline sp{nullptr, r, r_knots, coeffs, nknots, r_width, r_max};
   rc = CM_EINVAL;
-  CM_DISPATCH_C(channels, rc = cm::launch_backward<C_>(X, Y, sp, grad_out, sender, first_occ, sender_perm, sender_offsets,
-                                                       nnodes, nedges, gX, gY, grad_r, edge_scratch, cm::as_stream(stream)));
+  CM_DISPATCH_C(channels, rc = (cm::launch_backward<C_, false>(X, Y, sp, grad_out, sender, first_occ, sender_perm, sender_offsets,
+                                                               nnodes, nedges, gX, gY, grad_r, edge_scratch, cm::as_stream(stream))));
+  return rc;
+}
+
+extern "C" int cm_mp_edge_forward(const float *X, const float *vectors, const float *r_knots, const float *coeffs, int nknots,
+                                  float r_width, float r_max, const int32_t *sender, const int32_t *first_occ,
+                                  int64_t nnodes, int64_t nedges, int channels, float *out, cm_stream_t stream) {
+  CM_REQUIRE(cm_channels_supported(channels), "cm_mp_edge_forward: channels=%d must be a multiple of 32 in [32, 256]", channels);
+  CM_REQUIRE(nedges >= 0 && nnodes >= 0, "cm_mp_edge_forward: negative size");
+  CM_REQUIRE(nedges < INT32_MAX / 3 && nnodes < INT32_MAX / 2, "cm_mp_edge_forward: sizes exceed int32 indexing");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(X && first_occ && out, "cm_mp_edge_forward: NULL pointer");
+  CM_REQUIRE(nedges == 0 || sender, "cm_mp_edge_forward: NULL edge operand");
+  int rc = cm::check_spline("cm_mp_edge_forward", vectors, r_knots, coeffs, nknots, r_width, nedges);
+  if (rc != CM_OK) return rc;
+  const cm::Spline sp{vectors, nullptr, r_knots, coeffs, nknots, r_width, r_max};
+  rc = CM_EINVAL;
+  CM_DISPATCH_C(channels, rc = (cm::launch_forward<C_, true>(X, nullptr, sp, sender, first_occ, nnodes, nedges, out, cm::as_stream(stream))));
+  return rc;
+}
+
+extern "C" int cm_mp_edge_backward(const float *X, const float *vectors, const float *r_knots, const float *coeffs, int nknots,
+                                   float r_width, float r_max, const float *grad_out, const int32_t *sender,
+                                   const int32_t *first_occ, const int32_t *sender_perm, const int32_t *sender_offsets,
+                                   int64_t nnodes, int64_t nedges, int channels, float *gX, float *grad_vectors,
+                                   float *edge_scratch, cm_stream_t stream) {
+  CM_REQUIRE(cm_channels_supported(channels), "cm_mp_edge_backward: channels=%d must be a multiple of 32 in [32, 256]", channels);
+  CM_REQUIRE(nedges >= 0 && nnodes >= 0, "cm_mp_edge_backward: negative size");
+  CM_REQUIRE(nedges < INT32_MAX / 3 && nnodes < INT32_MAX / 2, "cm_mp_edge_backward: sizes exceed int32 indexing");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(X && grad_out && first_occ, "cm_mp_edge_backward: NULL pointer");
+  CM_REQUIRE(nedges == 0 || sender, "cm_mp_edge_backward: NULL edge operand");
+  CM_REQUIRE(!gX || (sender_offsets && (nedges == 0 || (sender_perm && edge_scratch))),
+             "cm_mp_edge_backward: gX wanted but sender_perm / sender_offsets / edge_scratch missing");
+  int rc = cm::check_spline("cm_mp_edge_backward", vectors, r_knots, coeffs, nknots, r_width, nedges);
+  if (rc != CM_OK) return rc;
+  const cm::Spline sp{vectors, nullptr, r_knots, coeffs, nknots, r_width, r_max};
+  rc = CM_EINVAL;
+  CM_DISPATCH_C(channels, rc = (cm::launch_backward<C_, true>(X, nullptr, sp, grad_out, sender, first_occ, sender_perm,
+                                                              sender_offsets, nnodes, nedges, gX, grad_vectors, nullptr,
+                                                              edge_scratch, cm::as_stream(stream))));
   return rc;
 }

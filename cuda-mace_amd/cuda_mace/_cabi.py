@@ -40,6 +40,8 @@ SIGNATURES = {
     "cm_mp_backward": (_i32, [_p] * 8 + [_i64, _i64, _i32] + [_p] * 5),
     "cm_mp_spline_forward": (_i32, [_p] * 5 + [_i32, _f32, _f32, _p, _p, _i64, _i64, _i32, _p, _p]),
     "cm_mp_spline_backward": (_i32, [_p] * 5 + [_i32, _f32, _f32] + [_p] * 5 + [_i64, _i64, _i32] + [_p] * 5),
+    "cm_mp_edge_forward": (_i32, [_p] * 4 + [_i32, _f32, _f32, _p, _p, _i64, _i64, _i32, _p, _p]),
+    "cm_mp_edge_backward": (_i32, [_p] * 4 + [_i32, _f32, _f32] + [_p] * 5 + [_i64, _i64, _i32] + [_p] * 4),
     "cm_edge_geometry_forward": (_i32, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p]),
     "cm_edge_geometry_backward": (_i32, [_p] * 9 + [_i64, _i64, _p, _p, _p]),
     "cm_sh_forward": (_i32, [_p, _i64, _p, _p]),
@@ -188,6 +190,44 @@ def mp_spline_backward(X, Y, r, r_knots, coeffs, r_width: float, r_max: float, g
         )
     )
     return gX, gY, gr
+
+
+def mp_edge_forward(X, vectors, r_knots, coeffs, r_width: float, r_max: float, sender, first_occ, nnodes: int) -> torch.Tensor:
+    C = X.shape[-1]
+    E = sender.numel()
+    if vectors.shape != (E, 3):
+        raise CudaMaceError("vectors must be [nedges, 3] with nedges = %d" % E)
+    if coeffs.shape != (r_knots.numel() - 1, 4, 4 * C):
+        raise CudaMaceError("coeffs must be [nknots-1, 4, 4*channels] = %s, got %s" % ((r_knots.numel() - 1, 4, 4 * C), tuple(coeffs.shape)))
+    out = torch.empty(nnodes, 16, C, dtype=F32, device=X.device)
+    _check(
+        lib.cm_mp_edge_forward(
+            _dev(X, F32, "X"), _dev(vectors, F32, "vectors"), _dev(r_knots, F32, "r_knots"), _dev(coeffs, F32, "coeffs"),
+            r_knots.numel(), float(r_width), float(r_max), _dev(sender, I32, "sender_list"),
+            _dev(first_occ, I32, "first_occurences"), nnodes, E, C, _dev(out, F32, "out"), _stream(),
+        )
+    )
+    return out
+
+
+def mp_edge_backward(X, vectors, r_knots, coeffs, r_width: float, r_max: float, grad_out, sender, first_occ, sender_perm,
+                     sender_offsets, nnodes: int, need_gX: bool = True, need_gvec: bool = True):
+    C = X.shape[-1]
+    E = sender.numel()
+    dev = X.device
+    gX = torch.empty(nnodes, C, dtype=F32, device=dev) if need_gX else None
+    gvec = torch.empty(E, 3, dtype=F32, device=dev) if need_gvec else None
+    scratch = torch.empty(E, C, dtype=F32, device=dev) if need_gX else None
+    _check(
+        lib.cm_mp_edge_backward(
+            _dev(X, F32, "X"), _dev(vectors, F32, "vectors"), _dev(r_knots, F32, "r_knots"), _dev(coeffs, F32, "coeffs"),
+            r_knots.numel(), float(r_width), float(r_max), _dev(grad_out, F32, "grad_out"), _dev(sender, I32, "sender_list"),
+            _dev(first_occ, I32, "first_occurences"), _dev(sender_perm, I32, "sender_perm") if need_gX else None,
+            _dev(sender_offsets, I32, "sender_offsets") if need_gX else None, nnodes, E, C,
+            _dev(gX, F32, "gX"), _dev(gvec, F32, "grad_vectors"), _dev(scratch, F32, "scratch"), _stream(),
+        )
+    )
+    return gX, gvec
 
 
 # ---- spherical harmonics ------------------------------------------------------------------------

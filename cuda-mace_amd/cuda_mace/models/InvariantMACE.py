@@ -148,12 +148,15 @@ class _FloatLinearView:
         self.weight = (linear.weight.data.double() / float(divide_by)).float()
 
 
-def _message_passing(tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline):
-    """Tabulated radial weights (edge_feats [E, 4C], the reference's data flow) or, when edge_feats is None, radial
-    weights evaluated inside the message-passing kernels from the spline of the edge lengths."""
+def _message_passing(tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline, edge_vectors):
+    """Tabulated radial weights (edge_feats [E, 4C], the reference's data flow); or, when edge_feats is None, radial
+    weights evaluated inside the message-passing kernels from the spline of the edge lengths; or, when edge_attrs is
+    None too, harmonics and radial weights both evaluated inside the kernels from the fp32 edge vectors."""
     if edge_feats is not None:
         return tp.forward(node_feats, edge_attrs, edge_feats.view(edge_feats.shape[0], -1, node_feats.shape[-1]), sender,
                           receiver, node_feats.shape[0])
+    if edge_attrs is None:
+        return tp.forward_edges(node_feats, edge_vectors, edge_spline, sender, receiver, node_feats.shape[0])
     return tp.forward_spline(node_feats, edge_attrs, edge_lengths, edge_spline, sender, receiver, node_feats.shape[0])
 
 
@@ -178,11 +181,12 @@ class InvariantInteraction(torch.nn.Module):
         self.compose_linears = True
 
     def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,
-                edge_lengths=None, edge_spline=None):
+                edge_lengths=None, edge_spline=None, edge_vectors=None):
         if sender is None:
             sender, receiver = edge_index[1].int(), edge_index[0].int()
         node_feats = self.linear_up(node_feats)
-        message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline)
+        message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline,
+                                   edge_vectors)
         if self.compose_linears:
             message = self.skip_tp.cuda_obj.forward(message, self.composed_weights, self.composed_weights_transposed, node_attrs)
         else:
@@ -204,20 +208,22 @@ class InvariantResidualInteraction(torch.nn.Module):
         self.avg_num_neighbors = inter.avg_num_neighbors
 
     def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,
-                edge_lengths=None, edge_spline=None):
+                edge_lengths=None, edge_spline=None, edge_vectors=None):
         if sender is None:
             sender, receiver = edge_index[1].int(), edge_index[0].int()
         sc = self.skip_tp(node_feats, node_attrs)
         node_feats = self.linear_up(node_feats)
-        message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline)
+        message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline,
+                                   edge_vectors)
         message = self.linear(message)  # 1/avg_num_neighbors is folded into its weights
         return message, sc
 
 
 class OptimizedInvariantMACE(torch.nn.Module):
     def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True):
-        """fused_radial=True evaluates the radial spline inside the message-passing kernels (same numbers, no
-        [nedges, 4C] tensors in memory); False keeps the reference's separate CubicSpline -> message passing steps."""
+        """fused_radial=True evaluates the spherical harmonics and the radial spline inside the message-passing kernels
+        (same numbers; no [16, nedges] or [nedges, 4C] tensors in memory); False keeps the reference's separate
+        SphericalHarmonics -> CubicSpline -> message passing steps."""
         super().__init__()
         self.fused_radial = bool(fused_radial)
         assert int(mace_model.num_interactions) == 2, "exactly two interaction layers are supported"
@@ -298,14 +304,16 @@ class OptimizedInvariantMACE(torch.nn.Module):
 
         # vectors = positions[edge_index[1]] - positions[edge_index[0]] + shifts in fp64, rounded once to fp32
         vectors32, lengths32 = EdgeGeometryAutograd.apply(positions, shifts, receiver, sender)
-        edge_attrs = self.spherical_harmonics.forward(vectors32)
+        # fused mode: the message-passing kernels take the vectors themselves and evaluate the harmonics per edge
+        edge_attrs = None if self.fused_radial else self.spherical_harmonics.forward(vectors32)
 
         node_es_list, node_feats_list = [], []
         for interaction, product, readout, edge_spline in zip(self.interactions, self.products, self.readouts, self.edge_splines):
             edge_feats = None if self.fused_radial else edge_spline.forward(lengths32)
             node_feats, sc = interaction(node_attrs=node_attrs32, node_feats=node_feats.float(), edge_attrs=edge_attrs,
                                          edge_feats=edge_feats, edge_index=data["edge_index"], sender=sender,
-                                         receiver=receiver, edge_lengths=lengths32, edge_spline=edge_spline)
+                                         receiver=receiver, edge_lengths=lengths32, edge_spline=edge_spline,
+                                         edge_vectors=vectors32)
             node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types).double()
             node_feats_list.append(node_feats)
             node_es_list.append(_select_head(readout(node_feats, node_heads), node_heads))

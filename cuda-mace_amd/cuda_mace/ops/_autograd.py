@@ -129,6 +129,39 @@ class InvariantMessagePassingSplineTPAutograd(torch.autograd.Function):
 
 
 # ------------------------------------------------------------------------------------------------
+class InvariantMessagePassingEdgeTPAutograd(torch.autograd.Function):
+    """Message passing straight from the edge vectors: harmonics, length and radial spline are evaluated in-kernel.
+    Equivalent to SphericalHarmonicsAutograd + CubicSplineAutograd + InvariantMessagePassingTPAutograd on
+    (vectors, |vectors|); differentiable in X and the vectors."""
+
+    @staticmethod
+    def forward(ctx, X, vectors, r_knots, coeffs, r_width, r_max, sender_list, receiver_list, nnodes):
+        _require(X.dtype == F32 and vectors.dtype == F32 and coeffs.dtype == F32 and r_knots.dtype == F32,
+                 "edge message passing: fp32 tensors expected")
+        _require(sender_list.dtype == I32 and receiver_list.dtype == I32, "edge message passing: int32 edge lists expected")
+        _require(vectors.dim() == 2 and vectors.shape[1] == 3, "edge message passing: vectors must be [nedges, 3]")
+        _require(X.dim() == 2 and X.shape[1] % 32 == 0, "edge message passing: X must be [nnodes, C] with C % 32 == 0")
+        nnodes = int(nnodes)
+        first_occ = csr_of(receiver_list, nnodes)
+        Xc, vc = X.contiguous(), vectors.contiguous()
+        out = cabi.mp_edge_forward(Xc, vc, r_knots, coeffs, r_width, r_max, sender_list, first_occ, nnodes)
+        ctx.save_for_backward(Xc, vc, r_knots, coeffs, sender_list, first_occ)
+        ctx.nnodes, ctx.r_width, ctx.r_max = nnodes, float(r_width), float(r_max)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        X, vectors, r_knots, coeffs, sender, first_occ = ctx.saved_tensors
+        need_x, need_v = ctx.needs_input_grad[:2]
+        perm = off = None
+        if need_x:
+            perm, off = sender_view_of(sender, ctx.nnodes)
+        gX, gvec = cabi.mp_edge_backward(X, vectors, r_knots, coeffs, ctx.r_width, ctx.r_max, grad_out.contiguous(), sender,
+                                         first_occ, perm, off, ctx.nnodes, need_gX=need_x, need_gvec=need_v)
+        return gX, gvec, None, None, None, None, None, None, None
+
+
+# ------------------------------------------------------------------------------------------------
 class EdgeGeometryAutograd(torch.autograd.Function):
     """(positions [N,3], shifts [E,3], row_a int32 [E] non-decreasing, row_b int32 [E]) -> (vectors fp32 [E,3],
     lengths fp32 [E]) with vectors = positions[row_b] - positions[row_a] + shifts evaluated in fp64.

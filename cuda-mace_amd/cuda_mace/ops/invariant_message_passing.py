@@ -28,3 +28,13 @@ class InvariantMessagePassingTP(torch.nn.Module):
         return InvariantMessagePassingSplineTPAutograd.apply(
             node_feats, edge_attrs, edge_lengths, spline.r_knots, spline.coefficients, spline._h, spline._rmax,
             sender_list, receiver_list, int(nnodes))
+
+    def forward_edges(self, node_feats, edge_vectors, spline, sender_list, receiver_list, nnodes):
+        """Same result as forward_spline with edge_attrs = spherical harmonics of edge_vectors and edge_lengths =
+        their norms, all evaluated inside the kernels: neither the harmonics nor the radial weights are ever stored.
+        Not part of the reference's interface."""
+        from ._autograd import InvariantMessagePassingEdgeTPAutograd
+
+        return InvariantMessagePassingEdgeTPAutograd.apply(
+            node_feats, edge_vectors, spline.r_knots, spline.coefficients, spline._h, spline._rmax, sender_list,
+            receiver_list, int(nnodes))

@@ -116,6 +116,24 @@ int cm_mp_spline_backward(const float *X, const float *Y, const float *r, const 
                           float *edge_scratch, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Message passing straight from the edge vectors: the 16 harmonics (cm_sh_forward's) and the length are computed per
+ * edge inside the kernels next to the radial spline, i.e. cm_mp_spline_forward with Y = SH(vectors), r = |vectors|.
+ * Fuses the reference's SphericalHarmonics, CubicSpline and InvariantMessagePassingTP calls
+ * (models/InvariantMACE.py:306, 320, 105-112); Y[16, nedges], grad_Y and grad_r never exist.
+ *   vectors fp32 [nedges, 3].  Backward: grad_vectors fp32 [nedges, 3] (may be NULL) is the full gradient with respect
+ *   to the edge vector, harmonics Jacobian and radial part included; gX as in cm_mp_backward.
+ */
+int cm_mp_edge_forward(const float *X, const float *vectors, const float *r_knots, const float *coeffs,
+                       int nknots, float r_width, float r_max, const int32_t *sender,
+                       const int32_t *first_occ, int64_t nnodes, int64_t nedges, int channels,
+                       float *out, cm_stream_t stream);
+int cm_mp_edge_backward(const float *X, const float *vectors, const float *r_knots, const float *coeffs,
+                        int nknots, float r_width, float r_max, const float *grad_out,
+                        const int32_t *sender, const int32_t *first_occ, const int32_t *sender_perm,
+                        const int32_t *sender_offsets, int64_t nnodes, int64_t nedges, int channels,
+                        float *gX, float *grad_vectors, float *edge_scratch, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Real spherical harmonics l <= 3 of normalised edge vectors, sqrt(4 pi) ("component")
  * normalisation, input axes permuted as (x, y, z) = (in[2], in[0], in[1]).
  * Replaces jit_spherical_harmonics / jit_spherical_harmonics_backward

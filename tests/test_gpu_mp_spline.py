@@ -70,6 +70,27 @@ def test_mp_spline_forward_backward(cabi, case):
     bound = 4e-6 * (gR2.view(E, -1).abs().double().cpu() * O.spline_eval(r, knots, coeffs, h, 5.0, deriv=True)[1].abs()).sum(-1) + 1e-30
     assert bool(((gr.double().cpu() - gr2.double().cpu()).abs() <= bound).all())
 
+    # edge-vector variant: harmonics and length computed in-kernel; oracle = SH + spline + MP, gradient by autograd
+    g2 = torch.Generator().manual_seed(case[4] + 7)
+    vec = torch.randn(E, 3, generator=g2, dtype=torch.float64)
+    vec = (vec / vec.norm(dim=1, keepdim=True) * r[:, None]).float().double()  # lengths spread like r, fp32-representable
+    va = vec.clone().requires_grad_(True)
+    Xb = X.clone().requires_grad_(True)
+    Rv = O.spline_eval(va.norm(dim=1), knots, coeffs, h, 5.0).view(E, 4, C)
+    ref_e = O.mp_forward(Xb, O.spherical_harmonics(va), Rv, snd, rcv, nnodes)
+    (ref_e * G).sum().backward()
+    out_e = cabi.mp_edge_forward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, snd.cuda(), fo, nnodes)
+    gX_e, gvec = cabi.mp_edge_backward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, d(G), snd.cuda(), fo, perm, off, nnodes)
+    close(out_e, ref_e.detach(), 2e-5, 2e-6)
+    close(gX_e, Xb.grad, 2e-5, 2e-6)
+    close(gvec, va.grad, 5e-5, 5e-6)
+    gX_only, none = cabi.mp_edge_backward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, d(G), snd.cuda(), fo, perm, off, nnodes,
+                                          need_gvec=False)
+    assert none is None and torch.equal(gX_only, gX_e)
+    none, gvec_only = cabi.mp_edge_backward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, d(G), snd.cuda(), fo, perm, off, nnodes,
+                                            need_gX=False)
+    assert none is None and torch.equal(gvec_only, gvec)
+
     # subsets of gradients
     only_r = cabi.mp_spline_backward(d(X), d(Y), d(r), d(knots), d(coeffs), h, 5.0, d(G), snd.cuda(), fo, perm, off, nnodes,
                                      need_gX=False, need_gY=False)
