@@ -29,11 +29,18 @@ __global__ void edge_geometry_forward_kernel(const double *__restrict__ pos, con
   len[e] = static_cast<float>(sqrt(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]));
 }
 
-// total gradient with respect to the edge vector: g_vec + g_len * vec / |vec| (vec recomputed in fp64)
+// total gradient with respect to the edge vector: g_vec + g_len * vec / |vec| (vec recomputed in fp64).  Without a
+// length gradient nothing but g_vec is touched.
+template <bool HAS_GLEN>
 __device__ __forceinline__ void edge_grad(const double *__restrict__ pos, const double *__restrict__ shifts,
                                           const int32_t *__restrict__ a, const int32_t *__restrict__ b,
                                           const float *__restrict__ gvec, const float *__restrict__ glen, int64_t e,
                                           int nnodes, double (&g)[3]) {
+  if constexpr (!HAS_GLEN) {
+#pragma unroll
+    for (int k = 0; k < 3; ++k) g[k] = gvec ? static_cast<double>(gvec[3 * e + k]) : 0.0;
+    return;
+  }
   const int ia = a[e], ib = b[e];
   g[0] = g[1] = g[2] = 0.0;
   if (static_cast<unsigned>(ia) >= static_cast<unsigned>(nnodes) || static_cast<unsigned>(ib) >= static_cast<unsigned>(nnodes)) return;
@@ -41,11 +48,12 @@ __device__ __forceinline__ void edge_grad(const double *__restrict__ pos, const 
 #pragma unroll
   for (int k = 0; k < 3; ++k) v[k] = pos[3 * ib + k] - pos[3 * ia + k] + shifts[3 * e + k];
   const double r = sqrt(v[0] * v[0] + v[1] * v[1] + v[2] * v[2]);
-  const double s = (glen != nullptr && r > 0.0) ? static_cast<double>(glen[e]) / r : 0.0;
+  const double s = r > 0.0 ? static_cast<double>(glen[e]) / r : 0.0;
 #pragma unroll
   for (int k = 0; k < 3; ++k) g[k] = (gvec ? static_cast<double>(gvec[3 * e + k]) : 0.0) + s * v[k];
 }
 
+template <bool HAS_GLEN>
 __global__ void edge_grad_kernel(const double *__restrict__ pos, const double *__restrict__ shifts,
                                  const int32_t *__restrict__ a, const int32_t *__restrict__ b,
                                  const float *__restrict__ gvec, const float *__restrict__ glen, int64_t nedges,
@@ -53,12 +61,13 @@ __global__ void edge_grad_kernel(const double *__restrict__ pos, const double *_
   const int64_t e = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
   if (e >= nedges) return;
   double g[3];
-  edge_grad(pos, shifts, a, b, gvec, glen, e, nnodes, g);
+  edge_grad<HAS_GLEN>(pos, shifts, a, b, gvec, glen, e, nnodes, g);
   gshift[3 * e + 0] = g[0];
   gshift[3 * e + 1] = g[1];
   gshift[3 * e + 2] = g[2];
 }
 
+template <bool HAS_GLEN>
 __global__ __launch_bounds__(256) void edge_geometry_backward_kernel(
     const double *__restrict__ pos, const double *__restrict__ shifts, const int32_t *__restrict__ a,
     const int32_t *__restrict__ b, const int32_t *__restrict__ a_first_occ, const int32_t *__restrict__ b_perm,
@@ -73,14 +82,14 @@ __global__ __launch_bounds__(256) void edge_geometry_backward_kernel(
   for (int k = b_offsets[node] + lane; k < b_offsets[node + 1]; k += kWave) {
     const int e = b_perm[k];
     if (static_cast<unsigned>(e) >= static_cast<uint64_t>(nedges)) continue;
-    edge_grad(pos, shifts, a, b, gvec, glen, e, nnodes, g);
+    edge_grad<HAS_GLEN>(pos, shifts, a, b, gvec, glen, e, nnodes, g);
     acc[0] += g[0];
     acc[1] += g[1];
     acc[2] += g[2];
   }
   // edges that start at this atom (row a, contiguous): - gradient
   for (int e = a_first_occ[node] + lane; e < a_first_occ[nnodes + node]; e += kWave) {
-    edge_grad(pos, shifts, a, b, gvec, glen, e, nnodes, g);
+    edge_grad<HAS_GLEN>(pos, shifts, a, b, gvec, glen, e, nnodes, g);
     acc[0] -= g[0];
     acc[1] -= g[1];
     acc[2] -= g[2];
@@ -125,14 +134,23 @@ extern "C" int cm_edge_geometry_backward(const double *positions, const int32_t 
   hipStream_t st = cm::as_stream(stream);
   if (grad_positions) {
     const int block = 256, per = block / cm::kWave;
-    hipLaunchKernelGGL(cm::edge_geometry_backward_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nnodes, per))), dim3(block), 0,
-                       st, positions, shifts, row_a, row_b, a_first_occ, b_perm, b_offsets, grad_vectors, grad_lengths, nedges,
-                       static_cast<int>(nnodes), grad_positions);
+    const dim3 grid(static_cast<unsigned>(cm::ceil_div(nnodes, per)));
+    if (grad_lengths)
+      hipLaunchKernelGGL(cm::edge_geometry_backward_kernel<true>, grid, dim3(block), 0, st, positions, shifts, row_a, row_b,
+                         a_first_occ, b_perm, b_offsets, grad_vectors, grad_lengths, nedges, static_cast<int>(nnodes), grad_positions);
+    else
+      hipLaunchKernelGGL(cm::edge_geometry_backward_kernel<false>, grid, dim3(block), 0, st, positions, shifts, row_a, row_b,
+                         a_first_occ, b_perm, b_offsets, grad_vectors, grad_lengths, nedges, static_cast<int>(nnodes), grad_positions);
   }
   if (grad_shifts && nedges > 0) {
     const int block = 256;
-    hipLaunchKernelGGL(cm::edge_grad_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nedges, block))), dim3(block), 0, st,
-                       positions, shifts, row_a, row_b, grad_vectors, grad_lengths, nedges, static_cast<int>(nnodes), grad_shifts);
+    const dim3 grid(static_cast<unsigned>(cm::ceil_div(nedges, block)));
+    if (grad_lengths)
+      hipLaunchKernelGGL(cm::edge_grad_kernel<true>, grid, dim3(block), 0, st, positions, shifts, row_a, row_b, grad_vectors,
+                         grad_lengths, nedges, static_cast<int>(nnodes), grad_shifts);
+    else
+      hipLaunchKernelGGL(cm::edge_grad_kernel<false>, grid, dim3(block), 0, st, positions, shifts, row_a, row_b, grad_vectors,
+                         grad_lengths, nedges, static_cast<int>(nnodes), grad_shifts);
   }
   return cm::check_launch("cm_edge_geometry_backward");
 }

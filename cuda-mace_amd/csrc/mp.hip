@@ -260,7 +260,17 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
   const int k1 = offsets[node + 1];
   f4 acc = zero4();
   if (active) {
-    for (int k = k0 + slot; k < k1; k += K::EPW) {
+    // four independent row gathers in flight per slot; the summation order stays fixed
+    int k = k0 + slot;
+    for (; k + 3 * K::EPW < k1; k += 4 * K::EPW) {
+      const int ea = perm[k], eb = perm[k + K::EPW], ec = perm[k + 2 * K::EPW], ed = perm[k + 3 * K::EPW];
+      const f4 va = static_cast<unsigned>(ea) < static_cast<uint64_t>(nedges) ? ld4(gXe + static_cast<int64_t>(ea) * C + 4 * cl) : zero4();
+      const f4 vb = static_cast<unsigned>(eb) < static_cast<uint64_t>(nedges) ? ld4(gXe + static_cast<int64_t>(eb) * C + 4 * cl) : zero4();
+      const f4 vc = static_cast<unsigned>(ec) < static_cast<uint64_t>(nedges) ? ld4(gXe + static_cast<int64_t>(ec) * C + 4 * cl) : zero4();
+      const f4 vd = static_cast<unsigned>(ed) < static_cast<uint64_t>(nedges) ? ld4(gXe + static_cast<int64_t>(ed) * C + 4 * cl) : zero4();
+      acc += (va + vb) + (vc + vd);
+    }
+    for (; k < k1; k += K::EPW) {
       const int e = perm[k];
       if (static_cast<unsigned>(e) < static_cast<uint64_t>(nedges)) acc += ld4(gXe + static_cast<int64_t>(e) * C + 4 * cl);
     }

@@ -134,7 +134,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
         const int idx = sIdx[j];
         if (idx < 0 || static_cast<unsigned>(s) >= static_cast<unsigned>(nnodes)) continue;
         const float xr = sXr[j];
-        const f4 x = ld4(X + static_cast<int64_t>(s) * C + 4 * cl);
+        const f4 x = ld4(X + (static_cast<unsigned>(s) * C + 4u * cl));
         float y[16];
         {
           const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
@@ -144,10 +144,12 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
             y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
           }
         }
-        const float *cp = sp.coeffs + static_cast<int64_t>(idx) * (16 * C) + 4 * cl;
+        const unsigned co = static_cast<unsigned>(idx) * (16u * C) + 4u * cl;  // 32-bit offset from the uniform table base
+        const float *__restrict__ tab = sp.coeffs;
         auto per_l = [&](auto lc) {
           constexpr int L = decltype(lc)::value;
-          const f4 a = ld4(cp + L * C), b = ld4(cp + 4 * C + L * C), c = ld4(cp + 8 * C + L * C), d = ld4(cp + 12 * C + L * C);
+          const f4 a = ld4(tab + (co + L * C)), b = ld4(tab + (co + (4 * C + L * C))), c = ld4(tab + (co + (8 * C + L * C))),
+                   d = ld4(tab + (co + (12 * C + L * C)));
           const f4 t = x * (a + xr * (b + xr * (c + xr * d)));
 #pragma unroll
           for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) acc[m] += y[m] * t;
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
       const bool live = active && idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
       const float xr = sXr[j];
       f4 x = zero4();
-      if (live) x = ld4(X + static_cast<int64_t>(s) * C + 4 * cl);
+      if (live) x = ld4(X + (static_cast<unsigned>(s) * C + 4u * cl));
       float y[16];
       {
         const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
@@ -227,7 +229,8 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
           y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
         }
       }
-      const float *cp = sp.coeffs + static_cast<int64_t>(idx < 0 ? 0 : idx) * (16 * C) + 4 * cl;
+      const unsigned co = static_cast<unsigned>(idx < 0 ? 0 : idx) * (16u * C) + 4u * cl;
+      const float *__restrict__ tab = sp.coeffs;
       float p[16];
       f4 gxe = zero4();
       f4 gr4 = zero4();
@@ -235,7 +238,8 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
         constexpr int L = decltype(lc)::value;
         f4 rl = zero4(), drl = zero4();
         if (live) {
-          const f4 a = ld4(cp + L * C), b = ld4(cp + 4 * C + L * C), c = ld4(cp + 8 * C + L * C), d = ld4(cp + 12 * C + L * C);
+          const f4 a = ld4(tab + (co + L * C)), b = ld4(tab + (co + (4 * C + L * C))), c = ld4(tab + (co + (8 * C + L * C))),
+                   d = ld4(tab + (co + (12 * C + L * C)));
           rl = a + xr * (b + xr * (c + xr * d));
           drl = b + xr * (2.f * c + (3.f * xr) * d);
         }
@@ -342,7 +346,10 @@ int launch_backward(const float *X, const float *Y, const Spline &sp, const floa
 }
 
 int check_spline(const char *who, const float *r_or_vec, const float *r_knots, const float *coeffs, int nknots,
-                 float r_width, int64_t nedges) {
+                 float r_width, int64_t nedges, int64_t nnodes, int channels) {
+  // the kernels address X rows and table rows with 32-bit element offsets
+  CM_REQUIRE(nnodes * channels < (int64_t{1} << 31) && static_cast<int64_t>(nknots) * 16 * channels < (int64_t{1} << 31),
+             "%s: nnodes * channels or the spline table exceeds 32-bit element offsets", who);
   CM_REQUIRE(nknots >= 2, "%s: need at least two knots, got %d", who, nknots);
   CM_REQUIRE(r_width > 0.f, "%s: r_width must be positive", who);
   CM_REQUIRE(nedges == 0 || (r_or_vec && r_knots && coeffs), "%s: NULL spline operand", who);
@@ -362,7 +369,7 @@ extern "C" int cm_mp_spline_forward(const float *X, const float *Y, const float 
   if (nnodes == 0) return CM_OK;
   CM_REQUIRE(X && first_occ && out, "cm_mp_spline_forward: NULL pointer");
   CM_REQUIRE(nedges == 0 || (Y && sender), "cm_mp_spline_forward: NULL edge operand");
-  int rc = cm::check_spline("cm_mp_spline_forward", r, r_knots, coeffs, nknots, r_width, nedges);
+  int rc = cm::check_spline("cm_mp_spline_forward", r, r_knots, coeffs, nknots, r_width, nedges, nnodes, channels);
   if (rc != CM_OK) return rc;
   const cm::Spline sp{nullptr, r, r_knots, coeffs, nknots, r_width, r_max};
   rc = CM_EINVAL;
@@ -383,7 +390,7 @@ extern "C" int cm_mp_spline_backward(const float *X, const float *Y, const float
   CM_REQUIRE(nedges == 0 || (Y && sender), "cm_mp_spline_backward: NULL edge operand");
   CM_REQUIRE(!gX || (sender_offsets && (nedges == 0 || (sender_perm && edge_scratch))),
              "cm_mp_spline_backward: gX wanted but sender_perm / sender_offsets / edge_scratch missing");
-  int rc = cm::check_spline("cm_mp_spline_backward", r, r_knots, coeffs, nknots, r_width, nedges);
+  int rc = cm::check_spline("cm_mp_spline_backward", r, r_knots, coeffs, nknots, r_width, nedges, nnodes, channels);
   if (rc != CM_OK) return rc;
   const cm::Spline sp{nullptr, r, r_knots, coeffs, nknots, r_width, r_max};
   rc = CM_EINVAL;
@@ -401,7 +408,7 @@ extern "C" int cm_mp_edge_forward(const float *X, const float *vectors, const fl
   if (nnodes == 0) return CM_OK;
   CM_REQUIRE(X && first_occ && out, "cm_mp_edge_forward: NULL pointer");
   CM_REQUIRE(nedges == 0 || sender, "cm_mp_edge_forward: NULL edge operand");
-  int rc = cm::check_spline("cm_mp_edge_forward", vectors, r_knots, coeffs, nknots, r_width, nedges);
+  int rc = cm::check_spline("cm_mp_edge_forward", vectors, r_knots, coeffs, nknots, r_width, nedges, nnodes, channels);
   if (rc != CM_OK) return rc;
   const cm::Spline sp{vectors, nullptr, r_knots, coeffs, nknots, r_width, r_max};
   rc = CM_EINVAL;
@@ -422,7 +429,7 @@ extern "C" int cm_mp_edge_backward(const float *X, const float *vectors, const f
   CM_REQUIRE(nedges == 0 || sender, "cm_mp_edge_backward: NULL edge operand");
   CM_REQUIRE(!gX || (sender_offsets && (nedges == 0 || (sender_perm && edge_scratch))),
              "cm_mp_edge_backward: gX wanted but sender_perm / sender_offsets / edge_scratch missing");
-  int rc = cm::check_spline("cm_mp_edge_backward", vectors, r_knots, coeffs, nknots, r_width, nedges);
+  int rc = cm::check_spline("cm_mp_edge_backward", vectors, r_knots, coeffs, nknots, r_width, nedges, nnodes, channels);
   if (rc != CM_OK) return rc;
   const cm::Spline sp{vectors, nullptr, r_knots, coeffs, nknots, r_width, r_max};
   rc = CM_EINVAL;

@@ -145,11 +145,13 @@ class EdgeGeometryAutograd(torch.autograd.Function):
         vec, length = cabi.edge_geometry_forward(pos64, row_a, row_b, sh64)
         ctx.save_for_backward(pos64, sh64, row_a, row_b)
         ctx.dtypes = (positions.dtype, shifts.dtype)
-        ctx.mark_non_differentiable()
+        ctx.set_materialize_grads(False)  # an unused output arrives as None in backward, not as zeros
         return vec, length
 
     @staticmethod
     def backward(ctx, grad_vec, grad_len):
+        if grad_vec is None and grad_len is None:
+            return None, None, None, None
         pos64, sh64, row_a, row_b = ctx.saved_tensors
         need_pos, need_shift = ctx.needs_input_grad[:2]
         nnodes = pos64.shape[0]
