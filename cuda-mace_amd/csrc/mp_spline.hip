@@ -195,6 +195,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   const int slot = lane / K::SW;
   const int cl = lane % K::SW;
   const bool active = cl < K::LPE;
+  const unsigned cla = active ? cl : 0;  // lanes beyond the channel count read lane 0's addresses; their g is zero
   const int e0 = first_occ[node];
   const int e1 = first_occ[nnodes + node];
   if (e0 >= e1) return;
@@ -211,15 +212,16 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
     __syncthreads();
     stage_edges<FROM_VEC>(Y, sender, sp, nedges, base, cnt, lane, sY, sS, sIdx, sXr);
     __syncthreads();
-    // every lane of a slot takes part in the reductions, so the loop bound is slot-uniform
+    // Every lane of a slot takes part in the reductions, so the loop bound is slot-uniform.  The body is free of
+    // branches: edges beyond the cutoff or with an invalid sender read clamped addresses and are zeroed where their
+    // results are stored, which lets the table loads of all four l be in flight together.
     for (int j = slot; j < cnt; j += K::EPW) {
       const int64_t e = base + j;
       const int s = sS[j];
       const int idx = sIdx[j];
-      const bool live = active && idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
+      const bool live = idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
       const float xr = sXr[j];
-      f4 x = zero4();
-      if (live) x = ld4(X + (static_cast<unsigned>(s) * C + 4u * cl));
+      const f4 x = ld4(X + ((live ? static_cast<unsigned>(s) : 0u) * C + 4u * cla));
       float y[16];
       {
         const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
@@ -229,20 +231,17 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
           y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
         }
       }
-      const unsigned co = static_cast<unsigned>(idx < 0 ? 0 : idx) * (16u * C) + 4u * cl;
+      const unsigned co = static_cast<unsigned>(idx < 0 ? 0 : idx) * (16u * C) + 4u * cla;
       const float *__restrict__ tab = sp.coeffs;
+      const float xr2 = 2.f * xr, xr3 = 3.f * xr * xr;
       float p[16];
       f4 gxe = zero4();
-      f4 gr4 = zero4();
+      f4 grq = zero4();
       auto per_l = [&](auto lc) {
         constexpr int L = decltype(lc)::value;
-        f4 rl = zero4(), drl = zero4();
-        if (live) {
-          const f4 a = ld4(tab + (co + L * C)), b = ld4(tab + (co + (4 * C + L * C))), c = ld4(tab + (co + (8 * C + L * C))),
-                   d = ld4(tab + (co + (12 * C + L * C)));
-          rl = a + xr * (b + xr * (c + xr * d));
-          drl = b + xr * (2.f * c + (3.f * xr) * d);
-        }
+        const f4 a = ld4(tab + (co + L * C)), b = ld4(tab + (co + (4 * C + L * C))), c = ld4(tab + (co + (8 * C + L * C))),
+                 d = ld4(tab + (co + (12 * C + L * C)));
+        const f4 rl = a + xr * (b + xr * (c + xr * d));
         f4 q = zero4();
 #pragma unroll
         for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) q += y[m] * g[m];
@@ -252,18 +251,19 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
           for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) p[m] = dot4(g[m], t);
         }
         if constexpr (WANT_GX) gxe += rl * q;
-        if constexpr (WANT_GR) gr4 += (x * q) * drl;
+        if constexpr (WANT_GR) grq += q * (b + xr2 * c + xr3 * d);  // q_l * dR_l/dr
       };
       per_l(std::integral_constant<int, 0>{});
       per_l(std::integral_constant<int, 1>{});
       per_l(std::integral_constant<int, 2>{});
       per_l(std::integral_constant<int, 3>{});
+      if constexpr (WANT_GX) gxe = live ? gxe : zero4();
 
       if constexpr (WANT_GX) {
         if (active) st4(gXe + e * C + 4 * cl, gxe);
       }
       if constexpr (WANT_GR) {
-        const float tot = slot_sum<K::SW>(hsum4(gr4));
+        const float tot = slot_sum<K::SW>(hsum4(x * grq));
         if (cl == 0) sGr[j] = tot;
       }
       if constexpr (WANT_GY) {
@@ -275,6 +275,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
       __syncthreads();
       if (lane < cnt) {
         const int64_t e = base + lane;
+        const bool dead = sIdx[lane] < 0 || static_cast<unsigned>(sS[lane]) >= static_cast<unsigned>(nnodes);
         if constexpr (FROM_VEC) {
           // gradient with respect to the edge vector: harmonics Jacobian applied to gY, plus g_r along the direction
           // (gY doubles as the output pointer of the [E, 3] vector gradient in this variant)
@@ -285,15 +286,15 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
           for (int m = 0; m < 16; ++m) gy[m] = sGY[m * kChunk + lane];
           sh::vjp(d, gy, gin);
           const float gr = sGr[lane];
-          gY[3 * e + 0] = gin[0] + gr * d.y;
-          gY[3 * e + 1] = gin[1] + gr * d.z;
-          gY[3 * e + 2] = gin[2] + gr * d.x;
+          gY[3 * e + 0] = dead ? 0.f : gin[0] + gr * d.y;
+          gY[3 * e + 1] = dead ? 0.f : gin[1] + gr * d.z;
+          gY[3 * e + 2] = dead ? 0.f : gin[2] + gr * d.x;
         } else {
           if constexpr (WANT_GY) {
 #pragma unroll
-            for (int m = 0; m < 16; ++m) gY[m * nedges + e] = sGY[m * kChunk + lane];
+            for (int m = 0; m < 16; ++m) gY[m * nedges + e] = dead ? 0.f : sGY[m * kChunk + lane];
           }
-          if constexpr (WANT_GR) g_r[e] = sGr[lane];
+          if constexpr (WANT_GR) g_r[e] = dead ? 0.f : sGr[lane];
         }
       }
     }
