@@ -26,7 +26,13 @@
 #define CM_FUSED_FWD_WAVES 3
 #endif
 #ifndef CM_FUSED_BWD_WAVES
-#define CM_FUSED_BWD_WAVES 3
+#define CM_FUSED_BWD_WAVES 2
+#endif
+// The backward edge pass without the per-edge gX output runs with a rotated edge loop (next edge's loads requested
+// before the current edge's reductions), which needs the registers of two waves per SIMD.  The variant with gX is as
+// fast at two waves per SIMD as at three and, unlike at three, never spills (measured at 96, 128 and 192 channels).
+#ifndef CM_FUSED_BWD_ROTATED_WAVES
+#define CM_FUSED_BWD_ROTATED_WAVES 2
 #endif
 
 namespace cm {
@@ -178,11 +184,12 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
 // backward, edge pass: gY, g_r and the per-edge contribution to gX
 // -----------------------------------------------------------------------------------------------
 template <int C, bool FROM_VEC, bool WANT_GY, bool WANT_GR, bool WANT_GX>
-__global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_edge_kernel(
+__global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_ROTATED_WAVES) void mp_spline_backward_edge_kernel(
     const float *__restrict__ X, const float *__restrict__ Y, Spline sp, const float *__restrict__ G,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges,
     float *__restrict__ gY, float *__restrict__ g_r, float *__restrict__ gXe) {
   using K = Cfg<C>;
+  constexpr bool kRotate = !WANT_GX;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
   __shared__ int sIdx[kChunk];
@@ -212,16 +219,36 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
     __syncthreads();
     stage_edges<FROM_VEC>(Y, sender, sp, nedges, base, cnt, lane, sY, sS, sIdx, sXr);
     __syncthreads();
-    // Every lane of a slot takes part in the reductions, so the loop bound is slot-uniform.  The body is free of
-    // branches: edges beyond the cutoff or with an invalid sender read clamped addresses and are zeroed where their
-    // results are stored, which lets the table loads of all four l be in flight together.
-    for (int j = slot; j < cnt; j += K::EPW) {
-      const int64_t e = base + j;
+    // Every lane of a slot takes part in the reductions, so the loop bound is slot-uniform.  Edges beyond the cutoff
+    // or with an invalid sender read clamped addresses and are zeroed where their results are stored.  In the
+    // rotated form the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
+    // arithmetic of the current one, so they travel while the cross-lane reductions (a chain of dependent lane
+    // exchanges) run.
+    f4 x, ca[4], cb[4], cc[4], cd[4];
+    float xr;
+    bool live;
+    auto fetch = [&](int j) {
       const int s = sS[j];
       const int idx = sIdx[j];
-      const bool live = idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
-      const float xr = sXr[j];
-      const f4 x = ld4(X + ((live ? static_cast<unsigned>(s) : 0u) * C + 4u * cla));
+      live = idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
+      xr = sXr[j];
+      x = ld4(X + ((live ? static_cast<unsigned>(s) : 0u) * C + 4u * cla));
+      const unsigned co = static_cast<unsigned>(idx < 0 ? 0 : idx) * (16u * C) + 4u * cla;
+      const float *__restrict__ tab = sp.coeffs;
+#pragma unroll
+      for (int L = 0; L < 4; ++L) {
+        ca[L] = ld4(tab + (co + L * C));
+        cb[L] = ld4(tab + (co + (4 * C + L * C)));
+        cc[L] = ld4(tab + (co + (8 * C + L * C)));
+        cd[L] = ld4(tab + (co + (12 * C + L * C)));
+      }
+    };
+    if constexpr (kRotate) {
+      if (slot < cnt) fetch(slot);
+    }
+    for (int j = slot; j < cnt; j += K::EPW) {
+      const int64_t e = base + j;
+      if constexpr (!kRotate) fetch(j);
       float y[16];
       {
         const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
@@ -231,16 +258,13 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
           y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
         }
       }
-      const unsigned co = static_cast<unsigned>(idx < 0 ? 0 : idx) * (16u * C) + 4u * cla;
-      const float *__restrict__ tab = sp.coeffs;
       const float xr2 = 2.f * xr, xr3 = 3.f * xr * xr;
       float p[16];
       f4 gxe = zero4();
       f4 grq = zero4();
       auto per_l = [&](auto lc) {
         constexpr int L = decltype(lc)::value;
-        const f4 a = ld4(tab + (co + L * C)), b = ld4(tab + (co + (4 * C + L * C))), c = ld4(tab + (co + (8 * C + L * C))),
-                 d = ld4(tab + (co + (12 * C + L * C)));
+        const f4 a = ca[L], b = cb[L], c = cc[L], d = cd[L];
         const f4 rl = a + xr * (b + xr * (c + xr * d));
         f4 q = zero4();
 #pragma unroll
@@ -258,12 +282,18 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
       per_l(std::integral_constant<int, 2>{});
       per_l(std::integral_constant<int, 3>{});
       if constexpr (WANT_GX) gxe = live ? gxe : zero4();
+      float grv = 0.f;
+      if constexpr (WANT_GR) grv = hsum4(x * grq);
+
+      if constexpr (kRotate) {
+        if (j + K::EPW < cnt) fetch(j + K::EPW);
+      }
 
       if constexpr (WANT_GX) {
         if (active) st4(gXe + e * C + 4 * cl, gxe);
       }
       if constexpr (WANT_GR) {
-        const float tot = slot_sum<K::SW>(hsum4(x * grq));
+        const float tot = slot_sum<K::SW>(grv);
         if (cl == 0) sGr[j] = tot;
       }
       if constexpr (WANT_GY) {
