@@ -181,10 +181,12 @@ class InvariantInteraction(torch.nn.Module):
         self.compose_linears = True
 
     def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,
-                edge_lengths=None, edge_spline=None, edge_vectors=None):
+                edge_lengths=None, edge_spline=None, edge_vectors=None, node_feats_are_up: bool = False):
+        """node_feats_are_up: node_feats is already linear_up(embedding) (the model caches it per species tensor)."""
         if sender is None:
             sender, receiver = edge_index[1].int(), edge_index[0].int()
-        node_feats = self.linear_up(node_feats)
+        if not node_feats_are_up:
+            node_feats = self.linear_up(node_feats)
         message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline,
                                    edge_vectors)
         if self.compose_linears:
@@ -208,7 +210,7 @@ class InvariantResidualInteraction(torch.nn.Module):
         self.avg_num_neighbors = inter.avg_num_neighbors
 
     def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,
-                edge_lengths=None, edge_spline=None, edge_vectors=None):
+                edge_lengths=None, edge_spline=None, edge_vectors=None, node_feats_are_up: bool = False):
         if sender is None:
             sender, receiver = edge_index[1].int(), edge_index[0].int()
         sc = self.skip_tp(node_feats, node_attrs)
@@ -289,9 +291,19 @@ class OptimizedInvariantMACE(torch.nn.Module):
                 positions=positions, unit_shifts=data["unit_shifts"], cell=cell, edge_index=data["edge_index"],
                 num_graphs=num_graphs, batch=batch)
 
-        node_e0 = _select_head(self.atomic_energies_fn(node_attrs.double()), node_heads)
+        # What depends on the species alone -- the atomic reference energies, the node embedding and the first layer's
+        # linear_up of it (weights are frozen) -- is evaluated once per node_attrs tensor and reused while that tensor
+        # is unchanged, like the index structures below.
+        def species_only():
+            with torch.no_grad():
+                attrs64 = node_attrs.double()
+                return (self.atomic_energies_fn(attrs64),
+                        self.interactions[0].linear_up(self.node_embedding(attrs64).float()))
+
+        e0_per_head, node_feats_up = _cached(node_attrs, "_cm_species_only", id(self), species_only)
+        node_e0 = _select_head(e0_per_head, node_heads)
         e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs)
-        node_feats = self.node_embedding(node_attrs.double())
+        node_feats = None
 
         # index structures shared by both layers, cached on the caller's tensors so that they are rebuilt only when
         # the neighbour list / the species change: int32 edge lists (their CSR offsets and sender-sorted view are in
@@ -310,10 +322,11 @@ class OptimizedInvariantMACE(torch.nn.Module):
         node_es_list, node_feats_list = [], []
         for interaction, product, readout, edge_spline in zip(self.interactions, self.products, self.readouts, self.edge_splines):
             edge_feats = None if self.fused_radial else edge_spline.forward(lengths32)
-            node_feats, sc = interaction(node_attrs=node_attrs32, node_feats=node_feats.float(), edge_attrs=edge_attrs,
-                                         edge_feats=edge_feats, edge_index=data["edge_index"], sender=sender,
-                                         receiver=receiver, edge_lengths=lengths32, edge_spline=edge_spline,
-                                         edge_vectors=vectors32)
+            node_feats, sc = interaction(node_attrs=node_attrs32,
+                                         node_feats=node_feats_up if node_feats is None else node_feats.float(),
+                                         edge_attrs=edge_attrs, edge_feats=edge_feats, edge_index=data["edge_index"],
+                                         sender=sender, receiver=receiver, edge_lengths=lengths32, edge_spline=edge_spline,
+                                         edge_vectors=vectors32, node_feats_are_up=node_feats is None)
             node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types).double()
             node_feats_list.append(node_feats)
             node_es_list.append(_select_head(readout(node_feats, node_heads), node_heads))
