@@ -27,6 +27,7 @@ _i64 = ctypes.c_int64
 _i32 = ctypes.c_int
 _f32 = ctypes.c_float
 _sz = ctypes.c_size_t
+_f64 = ctypes.c_double
 
 # name -> (restype, argtypes); mirrors include/cuda_mace_hip.h one to one
 SIGNATURES = {
@@ -53,6 +54,9 @@ SIGNATURES = {
     "cm_symcon_forward": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
     "cm_symcon_builtin_structure": (_i32, [_p, _i32, _p, _i32, _p, _p]),
     "cm_symcon_backward": (_i32, [_p, _p, _i64, _i32, _p, _p]),
+    "cm_neighbour_list_workspace": (_sz, [_i64, _i64]),
+    "cm_neighbour_list_count": (_i32, [_p, _p, _i32, _i32, _i32, _f64, _i64, _i64, _p, _sz, _p, _p, _p]),
+    "cm_neighbour_list_fill": (_i32, [_p, _f64, _i64, _i64, _p, _p, _i64, _p, _p, _p, _p, _p]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():
@@ -408,3 +412,41 @@ def symcon_backward(grad, grad_out) -> torch.Tensor:
     gX = torch.empty_like(grad)
     _check(lib.cm_symcon_backward(_dev(grad, F32, "grad"), _dev(grad_out, F32, "grad_out"), N, C, _dev(gX, F32, "gX"), _stream()))
     return gX
+
+
+# ---- neighbour list -------------------------------------------------------------------------------
+def neighbour_list(positions, cell, pbc, cutoff: float, max_cells: int = 0):
+    """(row_i int32 [E], row_j int32 [E], unit_shifts int32 [E, 3]) sorted by (i, j, S); positions fp64 [N, 3] and
+    cell fp64 [3, 3] (or None) on the device, pbc three booleans.  One host synchronisation (the number of pairs)."""
+    N = positions.shape[0]
+    dev = positions.device
+    max_cells = int(max_cells) if max_cells else max(1, min(N, 1 << 22))
+    ws_bytes = lib.cm_neighbour_list_workspace(N, max_cells)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    head = torch.empty(N + 2, dtype=I32, device=dev)  # offsets [N + 1] followed by the status word
+    px, py, pz = (int(bool(b)) for b in pbc)
+    _check(
+        lib.cm_neighbour_list_count(
+            _dev(positions, F64, "positions"), _dev(cell, F64, "cell"), px, py, pz, float(cutoff), N, max_cells,
+            ws.data_ptr(), ws_bytes, head.data_ptr(), head.data_ptr() + 4 * (N + 1), _stream(),
+        )
+    )
+    E, status = (int(v) for v in head[N:].tolist())
+    if status == 1:
+        raise CudaMaceError("neighbour list: a periodic axis needs a non-singular cell")
+    if status != 0:
+        raise CudaMaceError("neighbour list: the cell is thinner than cutoff / 32 along a periodic axis")
+    if E >= 2**31 // 4 - 1:
+        raise CudaMaceError("neighbour list: more pairs than int32 indexing holds")
+    row_i = torch.empty(E, dtype=I32, device=dev)
+    row_j = torch.empty(E, dtype=I32, device=dev)
+    S = torch.empty(E, 3, dtype=I32, device=dev)
+    if E > 0:
+        scratch = torch.empty(4 * E, dtype=I32, device=dev)
+        _check(
+            lib.cm_neighbour_list_fill(
+                _dev(positions, F64, "positions"), float(cutoff), N, max_cells, ws.data_ptr(), head.data_ptr(), E,
+                scratch.data_ptr(), row_i.data_ptr(), row_j.data_ptr(), S.data_ptr(), _stream(),
+            )
+        )
+    return row_i, row_j, S

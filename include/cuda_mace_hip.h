@@ -252,6 +252,34 @@ int cm_symcon_builtin_structure(int32_t *mono3_ijk_host, int capacity3, int32_t 
 int cm_symcon_backward(const float *grad, const float *grad_out, int64_t nnodes, int channels,
                        float *gX, cm_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Neighbour list on the device: all ordered pairs (i, j, S) with |r_j - r_i + S . cell| < cutoff, (j, S) != (i, 0),
+ * sorted lexicographically by (i, j, Sx, Sy, Sz) -- the step before the path.  The reference leaves it to the
+ * host: its model consumes data["edge_index"] / ["shifts"] built upstream (models/InvariantMACE.py:297-301) and its
+ * tests obtain them from a CPU neighbour search through the upstream data loader (tests/test_utils.py:62-105).
+ * Row i of the result is non-decreasing, which is what cm_first_occurences and the message-passing kernels need.
+ *   positions fp64 [nnodes, 3] (atoms may lie outside the cell); cell fp64 [3, 3] row vectors (device pointer;
+ *   may be NULL without periodic axes); pbc_x/y/z: periodicity along the cell vectors; cutoff > 0.
+ * The accept test is v = (r_j - r_i) + (Sx c0 + Sy c1 + Sz c2), v0 v0 + v1 v1 + v2 v2 < cutoff^2, evaluated in fp64
+ * left to right without fused multiply-adds.
+ * Two calls, because the number of pairs is known only after the first:
+ *   cm_neighbour_list_count: builds the cell list in `workspace` (cm_neighbour_list_workspace(nnodes, max_cells)
+ *     bytes; max_cells bounds the number of bins, nnodes is a good value) and writes offsets int32 [nnodes + 1]
+ *     (offsets[i] = first pair of atom i, offsets[nnodes] = number of pairs) and status int32 [1] (0 = ok,
+ *     1 = periodic axis with a singular cell, 2 = a periodic axis thinner than cutoff / 32; offsets are then
+ *     all zero).
+ *   cm_neighbour_list_fill: after the caller has read offsets[nnodes] = nedges and provided edge_scratch int32
+ *     [4 * nedges], writes row_i, row_j int32 [nedges] and unit_shifts int32 [nedges, 3].  `workspace` must be
+ *     the one the count call filled, untouched, with the same positions, cutoff, nnodes and max_cells.
+ */
+size_t cm_neighbour_list_workspace(int64_t nnodes, int64_t max_cells);
+int cm_neighbour_list_count(const double *positions, const double *cell, int pbc_x, int pbc_y, int pbc_z,
+                            double cutoff, int64_t nnodes, int64_t max_cells, void *workspace,
+                            size_t workspace_bytes, int32_t *offsets, int32_t *status, cm_stream_t stream);
+int cm_neighbour_list_fill(const double *positions, double cutoff, int64_t nnodes, int64_t max_cells,
+                           const void *workspace, const int32_t *offsets, int64_t nedges, int32_t *edge_scratch,
+                           int32_t *row_i, int32_t *row_j, int32_t *unit_shifts, cm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,10 @@ Pin status of each function (what fixes it besides its own formula):
                           U_matrix_real is PARITY UNPINNED (upstream package
                           is not available offline; only matters for trained
                           checkpoints, not for random-init weights)
+  neighbour_list          scipy cKDTree (periodic, box > 2 cutoff), explicit
+                          replication of the cell into a non-periodic cluster
+                          searched by a non-periodic cKDTree (small cells,
+                          several images of a pair), (i,j,S) <-> (j,i,-S)
   reference model         rotation / translation / permutation invariance,
                           F = -dE/dx by central differences, sum F = 0;
                           equality with upstream mace on a real checkpoint is

@@ -246,3 +246,50 @@ def edge_geometry(positions, row_a, row_b, shifts):
     model calls at models/InvariantMACE.py:297-301.  Gradients by torch.autograd on this expression."""
     vec = positions[row_b.long()] - positions[row_a.long()] + shifts
     return vec, vec.norm(dim=-1)
+
+
+# -----------------------------------------------------------------------------------------------
+def neighbour_list(positions: np.ndarray, cell, pbc, cutoff: float):
+    """All ordered pairs (i, j, S) with |r_j - r_i + S . cell| < cutoff and (j, S) != (i, 0), sorted by
+    (i, j, Sx, Sy, Sz): what the upstream host-side neighbour search hands the reference's model
+    (models/InvariantMACE.py:297-301 consumes edge_index / shifts; tests/test_utils.py:62-105 builds them through the
+    upstream data loader).  Brute force over all atom pairs and all images that can reach; the accept test is
+    evaluated term by term in fp64,
+        v = (r_j - r_i) + ((Sx c0 + Sy c1) + Sz c2),   (v0 v0 + v1 v1) + v2 v2 < cutoff^2.
+    Returns (edge_index int64 [2, E], unit_shifts int64 [E, 3])."""
+    pos = np.asarray(positions, dtype=np.float64).reshape(-1, 3)
+    n = pos.shape[0]
+    pbc = np.array([bool(b) for b in pbc])
+    c = np.zeros((3, 3)) if cell is None else np.asarray(cell, dtype=np.float64).reshape(3, 3)
+    if pbc.any():
+        inv = np.linalg.inv(c)
+        heights = 1.0 / np.linalg.norm(inv, axis=0)
+        reach = np.where(pbc, np.ceil(cutoff / heights).astype(np.int64) + 1, 0)
+    else:
+        inv = np.zeros((3, 3))
+        reach = np.zeros(3, dtype=np.int64)
+    rows = []
+    rc2 = cutoff * cutoff
+    offsets = np.array([(a, b, d) for a in range(-reach[0], reach[0] + 1) for b in range(-reach[1], reach[1] + 1)
+                        for d in range(-reach[2], reach[2] + 1)], dtype=np.int64)
+    for i in range(n):
+        d = pos - pos[i]                                     # r_j - r_i, [n, 3]
+        # image that brings the pair closest in fractional terms, then every image within reach of it
+        S0 = np.where(pbc, -np.round(d @ inv), 0).astype(np.int64)          # [n, 3]
+        S = S0[:, None, :] + offsets[None, :, :]                              # [n, n_img, 3]
+        Sf = S.astype(np.float64)
+        d2 = 0.0
+        for k in range(3):
+            shift = (Sf[..., 0] * c[0, k] + Sf[..., 1] * c[1, k]) + Sf[..., 2] * c[2, k]
+            v = d[:, None, k] + shift
+            d2 = v * v if k == 0 else d2 + v * v
+        hit = d2 < rc2
+        hit[i] &= ~np.all(S[i] == 0, axis=-1)
+        j, img = np.nonzero(hit)
+        for jj, im in zip(j, img):
+            rows.append((i, jj, S[jj, im, 0], S[jj, im, 1], S[jj, im, 2]))
+    if not rows:
+        return np.zeros((2, 0), dtype=np.int64), np.zeros((0, 3), dtype=np.int64)
+    arr = np.array(sorted(set(rows)), dtype=np.int64)
+    assert arr.shape[0] == len(rows), "an image was visited twice"
+    return arr[:, :2].T.copy(), arr[:, 2:].copy()

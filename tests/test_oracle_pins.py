@@ -202,3 +202,59 @@ def test_symmetric_contraction_brute_force():
                 s += U2[i, j, p] * W2[e, p, c] * X[n, i, c] * X[n, j, c]
             ref[n, c] = s
     torch.testing.assert_close(out, ref)
+
+
+# ---- neighbour list ---------------------------------------------------------------------------------------
+def test_neighbour_list_oracle_vs_kdtree_periodic():
+    """Cubic box wider than two cutoffs: scipy's periodic cKDTree finds the same pairs; the image follows from the
+    minimum-image convention."""
+    from scipy.spatial import cKDTree
+
+    rng = np.random.default_rng(0)
+    box, rc = 12.0, 5.0
+    pos = rng.uniform(-5.0, 20.0, (150, 3))  # atoms outside the cell too
+    ei, S = O.neighbour_list(pos, np.eye(3) * box, (1, 1, 1), rc)
+    pairs = cKDTree(np.mod(pos, box), boxsize=box).query_pairs(rc, output_type="ndarray")
+    i = np.concatenate([pairs[:, 0], pairs[:, 1]])
+    j = np.concatenate([pairs[:, 1], pairs[:, 0]])
+    Sk = -np.round((pos[j] - pos[i]) / box).astype(np.int64)
+    order = np.lexsort((Sk[:, 2], Sk[:, 1], Sk[:, 0], j, i))
+    assert np.array_equal(ei, np.stack([i[order], j[order]]))
+    assert np.array_equal(S, Sk[order])
+
+
+def test_neighbour_list_oracle_vs_replicated_cluster():
+    """Triclinic cell smaller than the cutoff, two periodic axes: replicate the atoms explicitly and search the
+    resulting cluster without periodicity."""
+    from scipy.spatial import cKDTree
+
+    rng = np.random.default_rng(1)
+    cell = np.array([[4.0, 0, 0], [1.0, 3.5, 0], [0.5, 0.7, 4.2]])
+    pos = rng.uniform(-3, 8, (7, 3))
+    rc, R = 5.0, 4
+    ei, S = O.neighbour_list(pos, cell, (1, 1, 0), rc)
+    imgs = [(a, b, 0) for a in range(-R, R + 1) for b in range(-R, R + 1)]
+    allpos = np.concatenate([pos + np.array(im) @ cell for im in imgs])
+    tree = cKDTree(allpos)
+    rows = []
+    for i in range(7):
+        for k in tree.query_ball_point(pos[i], rc):
+            im, j = imgs[k // 7], k % 7
+            if (j == i and im == (0, 0, 0)) or not np.linalg.norm(allpos[k] - pos[i]) < rc:
+                continue
+            rows.append((i, j) + im)
+    rows = np.array(sorted(rows))
+    assert rows.shape[0] > 100
+    assert np.array_equal(rows[:, :2].T, ei) and np.array_equal(rows[:, 2:], S)
+    # reverse pairs carry the negated image
+    fwd = {tuple(r) for r in np.concatenate([ei.T, S], axis=1)}
+    assert fwd == {(j, i, -a, -b, -c) for (i, j, a, b, c) in fwd}
+
+
+def test_neighbour_list_oracle_cluster_and_self_images():
+    pos = np.array([[0.0, 0, 0], [1.0, 0, 0], [0, 4.0, 0], [10.0, 10, 10]])
+    ei, S = O.neighbour_list(pos, None, (0, 0, 0), 4.5)
+    assert ei.T.tolist() == [[0, 1], [0, 2], [1, 0], [1, 2], [2, 0], [2, 1]] and not S.any()
+    # a single atom in a 3 A cubic cell with a 3.5 A cutoff sees its 6 nearest images only (next shell at 4.24 A)
+    ei, S = O.neighbour_list(np.array([[0.3, 0.2, 0.1]]), np.eye(3) * 3.0, (1, 1, 1), 3.5)
+    assert ei.shape[1] == 6 and sorted(map(tuple, S)) == sorted([(1, 0, 0), (-1, 0, 0), (0, 1, 0), (0, -1, 0), (0, 0, 1), (0, 0, -1)])
