@@ -203,12 +203,20 @@ def main():
     fwd_b, bwd_b, fwd_fb, bwd_fb = mp_algorithmic_bytes(N, E, C)
     t_bwd, t_fwd = avg_ms(bwd_name), avg_ms(fwd_name)
     if fused:
+        sh_b, spline_b = 88 * E, 4 * (8 * E * C + E)  # harmonics backward, spline backward (each operand once)
         roofline = entry("mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb, t_bwd,
                          launches_timed=len(events[bwd_name]),
-                         note="harmonics and radial weights are evaluated in-kernel; the radial coefficients come from the 2 MB "
-                              "spline table in L2 (16 loads of 16 B per lane and edge) and the backward issues ~10k VALU "
-                              "instructions per wave, so this kernel is bounded by VALU issue and L2 bandwidth, not HBM; see "
-                              "roofline_other_kernels for the HBM-bound message passing with tabulated R[E,4,C]")
+                         note="harmonics and radial weights are evaluated in-kernel, so the kernel's own HBM operands are "
+                              "small; the radial coefficients come from the 2 MB spline table in L2 (16 loads of 16 B per "
+                              "lane and edge) and the backward occupies ~80% of all VALU issue slots: bounded by VALU issue "
+                              "and L1 delivery, not HBM; see roofline_other_kernels for the HBM-bound message passing with "
+                              "tabulated R[E,4,C]",
+                         unfused_equivalent={
+                             "bytes": bwd_b + sh_b + spline_b,
+                             "GB/s": round((bwd_b + sh_b + spline_b) / (t_bwd * 1e-3) / 1e9, 1),
+                             "meaning": "algorithmic HBM bytes of the three separate kernels this launch replaces (message-"
+                                        "passing backward with tabulated R, spline backward, harmonics backward) divided by "
+                                        "this launch's duration"})
         others = [entry("mp_spline_forward_kernel<%d,true>" % C, fwd_fb, t_fwd)]
     else:
         roofline = entry("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b, t_bwd,
@@ -247,6 +255,22 @@ def main():
         others.append(entry("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b, tb,
                             context="isolated op with tabulated R[E,4,C]"))
 
+    # the step before the path: neighbour list rebuilt on the device (excluded from the timed steps, as the reference's
+    # own timing excludes it); checked against the host-built list of the generator
+    from cuda_mace.utils.neighbour_list import get_neighborhood
+
+    def build_list():
+        return get_neighborhood(data["positions"].detach(), 5.0, (True, True, True), data["cell"])
+
+    ei_dev = build_list()[0]
+    torch.cuda.synchronize()
+    t_nl = time.perf_counter()
+    for _ in range(5):
+        build_list()
+    torch.cuda.synchronize()
+    neighbour_list = {"ms_per_build": round(1e3 * (time.perf_counter() - t_nl) / 5, 3), "pairs": int(ei_dev.shape[1]),
+                      "identical_to_host_list": bool(torch.equal(ei_dev, data["edge_index"]))}
+
     cpu_baseline = None
     if not args.no_cpu_baseline:
         from oracle import mace_model as oracle_model  # the checker, timed as the reported CPU baseline
@@ -277,6 +301,7 @@ def main():
                                "l_max 3, correlation 3, %d elements, random-init weights (seed 0)" % (N, E, C, ne),
                    "atoms": N, "edges": E, "channels": C, "radial": "fused spline" if fused else "tabulated"},
         "roofline": roofline, "roofline_other_kernels": others, "cpu_baseline": cpu_baseline,
+        "neighbour_list": neighbour_list,
     }
     if cpu_baseline:
         line["speedup_vs_cpu_baseline"] = round(value / cpu_baseline["value"], 1)
