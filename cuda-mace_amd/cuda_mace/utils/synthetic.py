@@ -97,5 +97,17 @@ def make_system(n_atoms: int, num_elements: int, seed: int = 0, density: Optiona
     }
 
 
+def collate(systems) -> Dict[str, torch.Tensor]:
+    """Several single-graph `data` dictionaries as one batch: nodes concatenated, edge indices offset, `batch` / `ptr`
+    naming the graph of every node, one 3x3 cell per graph stacked row-wise ([3 * graphs, 3], as upstream batches it)."""
+    counts = [int(d["positions"].shape[0]) for d in systems]
+    starts = np.concatenate([[0], np.cumsum(counts)])
+    out = {k: torch.cat([d[k] for d in systems], dim=0) for k in ("positions", "node_attrs", "unit_shifts", "shifts", "cell")}
+    out["edge_index"] = torch.cat([d["edge_index"] + int(o) for d, o in zip(systems, starts[:-1])], dim=1)
+    out["batch"] = torch.cat([torch.full((c,), g, dtype=torch.int64) for g, c in enumerate(counts)])
+    out["ptr"] = torch.tensor(starts, dtype=torch.int64)
+    return out
+
+
 def to_device(data: Dict[str, torch.Tensor], device) -> Dict[str, torch.Tensor]:
     return {k: v.to(device) for k, v in data.items()}

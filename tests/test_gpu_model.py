@@ -99,3 +99,31 @@ def test_virials_match_strain_derivative(cabi):
         assert abs(fd - float(vir[a, b])) < 2e-3 * max(1.0, float(vir.abs().max()))
     vol = float(torch.det(data["cell"]))
     torch.testing.assert_close(out["stress"].double().cpu()[0], -vir / vol, rtol=1e-5, atol=1e-8)
+
+
+def test_batch_of_graphs(cabi):
+    """Three different periodic boxes as one batch: per-graph energies, forces, virials and stress equal those of the
+    graphs evaluated one by one (GPU) and the fp64 reference."""
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.utils.synthetic import collate
+
+    systems = [make_system(n, 4, seed=20 + k, density=0.1) for k, n in enumerate((150, 230, 120))]
+    deg = sum(int(d["edge_index"].shape[1]) for d in systems) / sum(int(d["positions"].shape[0]) for d in systems)
+    upstream = SyntheticInvariantMACE(channels=64, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=deg, seed=9)
+    params = upstream.export_params()
+    model = OptimizedInvariantMACE(upstream, device="cuda")
+    batch = model(to_device(collate(systems), "cuda"), compute_virials=True, compute_stress=True)
+    assert batch["energy"].shape == (3,) and batch["virials"].shape == (3, 3, 3) and batch["stress"].shape == (3, 3, 3)
+    start = 0
+    for g, d in enumerate(systems):
+        n = d["positions"].shape[0]
+        single = model(to_device(d, "cuda"), compute_virials=True, compute_stress=True)
+        ref = M.energy_and_forces(params, d)
+        scale = float(ref["forces"].abs().max())
+        assert abs(float(batch["energy"][g].detach()) - float(ref["energy"])) <= 1e-5 * abs(float(ref["energy"])) + 1e-6
+        assert float((batch["forces"][start:start + n].double().cpu() - ref["forces"]).abs().max()) <= 1e-4
+        torch.testing.assert_close(batch["energy"][g].detach(), single["energy"][0].detach(), rtol=1e-6, atol=1e-7)
+        torch.testing.assert_close(batch["forces"][start:start + n], single["forces"], rtol=0, atol=1e-6 * scale + 1e-7)
+        torch.testing.assert_close(batch["virials"][g], single["virials"][0], rtol=1e-5, atol=1e-5 * float(single["virials"].abs().max()))
+        torch.testing.assert_close(batch["stress"][g], single["stress"][0], rtol=1e-5, atol=1e-5 * float(single["stress"].abs().max()))
+        start += n
