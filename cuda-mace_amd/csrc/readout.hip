@@ -1,0 +1,120 @@
+// Readouts of the two-layer invariant model and their derivative, one pass.
+//
+// The reference keeps upstream's readout modules in fp64 and feeds them the fp32 node features cast to double
+// (models/InvariantMACE.py:196, 330-337, 343): a linear readout of the first layer's features, a one-hidden-layer
+// readout (normalised silu gate) of the second layer's, then scale and shift.  Per step that is a dozen small fp64
+// GEMM and element-wise launches forward and as many backward.  Here one kernel does all of it per node in fp64:
+//
+//   e[n]   = scale * ( h1[n] . w1  +  sum_j w2b[j] * act(z_j) ) + shift,      z = h2[n] . W2a,   act(z) = cst * z * sigmoid(z)
+//   d2[n,c] = scale * sum_j W2a[c, j] * w2b[j] * act'(z_j)                     (= d e[n] / d h2[n, c], stored in fp32)
+//   d e[n] / d h1[n, c] = scale * w1[c]                                        (constant, not stored)
+//
+// and, on request, the [N, 2C] fp64 concatenation of the features that the model returns as "node_feats".  The
+// backward is then a scaling of those derivatives by the incoming gradient of e[n].
+//
+// Work split: a workgroup of 256 threads takes 16 nodes; their h2 rows are staged in LDS with coalesced loads and
+// W2a sits in LDS; thread (node, j) accumulates z_j over the channels, 16-lane shuffles reduce over j.
+#include <cmath>
+
+#include "common.hpp"
+
+namespace cm {
+namespace {
+
+constexpr int kNodes = 16;    // nodes per workgroup
+constexpr int kHidden = 16;   // threads per node = largest hidden width handled
+constexpr int kMaxC = 256;
+constexpr int kLdW = kHidden + 1;  // padded row stride of the weight tile in LDS (doubles)
+
+__global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
+    const float *__restrict__ h1, const float *__restrict__ h2, const double *__restrict__ w1, const double *__restrict__ W2a,
+    const double *__restrict__ w2b, double act_cst, double scale, double shift, int nnodes, int C, int H,
+    double *__restrict__ node_es, float *__restrict__ d2, double *__restrict__ feats64) {
+  __shared__ double sW[kMaxC * kLdW];      // W2a [C, H], H padded to 16 columns with zeros
+  __shared__ float s2[kNodes * kMaxC];
+  __shared__ double sD[kNodes * kHidden];  // w2b[j] * act'(z_j) per node
+  const int t = threadIdx.x;
+  const int node0 = blockIdx.x * kNodes;
+  const int rows = min(kNodes, nnodes - node0);
+  for (int i = t; i < C * kHidden; i += blockDim.x) {
+    const int c = i / kHidden, j = i % kHidden;
+    sW[c * kLdW + j] = j < H ? W2a[c * H + j] : 0.0;
+  }
+  for (int i = t; i < rows * C; i += blockDim.x) {
+    const int r = i / C, c = i % C;
+    const float b = h2[static_cast<int64_t>(node0 + r) * C + c];
+    const float a = feats64 ? h1[static_cast<int64_t>(node0 + r) * C + c] : 0.f;
+    s2[r * kMaxC + c] = b;
+    if (feats64) {
+      feats64[static_cast<int64_t>(node0 + r) * (2 * C) + c] = a;
+      feats64[static_cast<int64_t>(node0 + r) * (2 * C) + C + c] = b;
+    }
+  }
+  __syncthreads();
+  const int r = t / kHidden, j = t % kHidden;
+  const bool live = r < rows;
+  // first readout: each of the node's 16 threads takes every 16th channel
+  double e1 = 0.0, z = 0.0;
+  if (live) {
+    const float *row1 = h1 + static_cast<int64_t>(node0 + r) * C;
+    for (int c = j; c < C; c += kHidden) e1 += static_cast<double>(row1[c]) * w1[c];
+    for (int c = 0; c < C; ++c) z += static_cast<double>(s2[r * kMaxC + c]) * sW[c * kLdW + j];
+  }
+  double e2 = 0.0, dj = 0.0;
+  if (live && j < H) {
+    const double sig = 1.0 / (1.0 + exp(-z));
+    e2 = w2b[j] * act_cst * z * sig;
+    dj = w2b[j] * act_cst * (sig + z * sig * (1.0 - sig));
+  }
+  sD[t] = dj;
+  double e = e1 + e2;
+#pragma unroll
+  for (int off = kHidden / 2; off > 0; off >>= 1) e += __shfl_xor(e, off);
+  if (live && j == 0) node_es[node0 + r] = scale * e + shift;
+  __syncthreads();
+  for (int i = t; i < rows * C; i += blockDim.x) {
+    const int rr = i / C, c = i % C;
+    double acc = 0.0;
+#pragma unroll
+    for (int q = 0; q < kHidden; ++q) acc += sW[c * kLdW + q] * sD[rr * kHidden + q];
+    d2[static_cast<int64_t>(node0 + rr) * C + c] = static_cast<float>(scale * acc);
+  }
+}
+
+__global__ void readout_backward_kernel(const double *__restrict__ g, const double *__restrict__ w1, const float *__restrict__ d2,
+                                        double scale, int64_t total, int C, float *__restrict__ g1, float *__restrict__ g2) {
+  const int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (i >= total) return;
+  const double gn = g[i / C];
+  if (g1) g1[i] = static_cast<float>(gn * scale * w1[i % C]);
+  if (g2) g2[i] = static_cast<float>(gn * static_cast<double>(d2[i]));
+}
+
+}  // namespace
+}  // namespace cm
+
+extern "C" int cm_readout_forward(const float *h1, const float *h2, const double *w1, const double *W2a, const double *w2b,
+                                  double act_cst, double scale, double shift, int64_t nnodes, int channels, int hidden,
+                                  double *node_energies, float *d_h2, double *node_feats64, cm_stream_t stream) {
+  CM_REQUIRE(channels >= 1 && channels <= cm::kMaxC, "cm_readout_forward: channels=%d must be in [1, %d]", channels, cm::kMaxC);
+  CM_REQUIRE(hidden >= 1 && hidden <= cm::kHidden, "cm_readout_forward: hidden=%d must be in [1, %d]", hidden, cm::kHidden);
+  CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 2, "cm_readout_forward: nnodes out of range");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(h1 && h2 && w1 && W2a && w2b && node_energies && d_h2, "cm_readout_forward: NULL pointer");
+  hipLaunchKernelGGL(cm::readout_forward_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nnodes, cm::kNodes))),
+                     dim3(cm::kNodes * cm::kHidden), 0, cm::as_stream(stream), h1, h2, w1, W2a, w2b, act_cst, scale, shift,
+                     static_cast<int>(nnodes), channels, hidden, node_energies, d_h2, node_feats64);
+  return cm::check_launch("cm_readout_forward");
+}
+
+extern "C" int cm_readout_backward(const double *grad_node_energies, const double *w1, const float *d_h2, double scale,
+                                   int64_t nnodes, int channels, float *grad_h1, float *grad_h2, cm_stream_t stream) {
+  CM_REQUIRE(channels >= 1 && channels <= cm::kMaxC, "cm_readout_backward: channels=%d must be in [1, %d]", channels, cm::kMaxC);
+  CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 2, "cm_readout_backward: nnodes out of range");
+  if (nnodes == 0 || (!grad_h1 && !grad_h2)) return CM_OK;
+  CM_REQUIRE(grad_node_energies && w1 && d_h2, "cm_readout_backward: NULL pointer");
+  const int64_t total = nnodes * channels;
+  hipLaunchKernelGGL(cm::readout_backward_kernel, dim3(static_cast<unsigned>(cm::ceil_div(total, 256))), dim3(256), 0,
+                     cm::as_stream(stream), grad_node_energies, w1, d_h2, scale, total, channels, grad_h1, grad_h2);
+  return cm::check_launch("cm_readout_backward");
+}

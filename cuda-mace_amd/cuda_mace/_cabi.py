@@ -54,6 +54,8 @@ SIGNATURES = {
     "cm_symcon_forward": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
     "cm_symcon_builtin_structure": (_i32, [_p, _i32, _p, _i32, _p, _p]),
     "cm_symcon_backward": (_i32, [_p, _p, _i64, _i32, _p, _p]),
+    "cm_readout_forward": (_i32, [_p] * 5 + [_f64, _f64, _f64, _i64, _i32, _i32, _p, _p, _p, _p]),
+    "cm_readout_backward": (_i32, [_p, _p, _p, _f64, _i64, _i32, _p, _p, _p]),
     "cm_neighbour_list_workspace": (_sz, [_i64, _i64]),
     "cm_neighbour_list_count": (_i32, [_p, _p, _i32, _i32, _i32, _f64, _i64, _i64, _p, _sz, _p, _p, _p]),
     "cm_neighbour_list_fill": (_i32, [_p, _f64, _i64, _i64, _p, _p, _i64, _p, _p, _p, _p, _p]),
@@ -450,3 +452,35 @@ def neighbour_list(positions, cell, pbc, cutoff: float, max_cells: int = 0):
             )
         )
     return row_i, row_j, S
+
+
+# ---- readouts -------------------------------------------------------------------------------------
+def readout_forward(h1, h2, w1, W2a, w2b, act_cst: float, scale: float, shift: float, want_feats: bool = True):
+    """(node_energies fp64 [N], d_h2 fp32 [N, C], node_feats fp64 [N, 2C] or None)."""
+    N, C = h1.shape
+    H = W2a.shape[1]
+    dev = h1.device
+    es = torch.empty(N, dtype=F64, device=dev)
+    d2 = torch.empty(N, C, dtype=F32, device=dev)
+    feats = torch.empty(N, 2 * C, dtype=F64, device=dev) if want_feats else None
+    _check(
+        lib.cm_readout_forward(
+            _dev(h1, F32, "h1"), _dev(h2, F32, "h2"), _dev(w1, F64, "w1"), _dev(W2a, F64, "W2a"), _dev(w2b, F64, "w2b"),
+            float(act_cst), float(scale), float(shift), N, C, H, _dev(es, F64, "node_energies"), _dev(d2, F32, "d_h2"),
+            _dev(feats, F64, "node_feats"), _stream(),
+        )
+    )
+    return es, d2, feats
+
+
+def readout_backward(g, w1, d2, scale: float, need_h1: bool = True, need_h2: bool = True):
+    N, C = d2.shape
+    g1 = torch.empty_like(d2) if need_h1 else None
+    g2 = torch.empty_like(d2) if need_h2 else None
+    _check(
+        lib.cm_readout_backward(
+            _dev(g, F64, "grad_node_energies"), _dev(w1, F64, "w1"), _dev(d2, F32, "d_h2"), float(scale), N, C,
+            _dev(g1, F32, "grad_h1"), _dev(g2, F32, "grad_h2"), _stream(),
+        )
+    )
+    return g1, g2

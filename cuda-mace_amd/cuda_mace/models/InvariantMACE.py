@@ -21,7 +21,7 @@ from cuda_mace.ops.invariant_message_passing import InvariantMessagePassingTP
 from cuda_mace.ops.linear import ElementalLinear, Linear, ScalarElementalLinear
 from cuda_mace.ops.spherical_harmonics import SphericalHarmonics
 from cuda_mace.ops.symmetric_contraction import SymmetricContraction as CUDAContraction
-from cuda_mace.ops._autograd import EdgeGeometryAutograd, _cached
+from cuda_mace.ops._autograd import EdgeGeometryAutograd, ReadoutEnergyAutograd, _cached
 from cuda_mace.utils.irreps import Instruction
 
 
@@ -89,6 +89,33 @@ def _select_head(per_head: torch.Tensor, node_heads: torch.Tensor) -> torch.Tens
     if per_head.shape[1] == 1:
         return per_head[:, 0]
     return torch.gather(per_head, 1, node_heads.view(-1, 1)).squeeze(1)
+
+
+def fused_readout_parameters(readouts, scale_shift):
+    """Weights of the readout pair in the form the fused readout kernel takes, or None when the modules are not the
+    standard pair of a two-layer invariant model (a linear readout to one scalar, then linear -> normalised silu gate ->
+    linear to one scalar, single head, scalar scale and shift).  Attribute names follow upstream's readout blocks
+    (`linear`; `linear_1`, `non_linearity`, `linear_2`), whose modules the reference keeps as they are
+    (models/InvariantMACE.py:196)."""
+    try:
+        r0, r1 = readouts
+        lin0, lin1, lin2 = r0.linear, r1.linear_1, r1.linear_2
+        gate = r1.non_linearity.acts[0]
+        dims = [(l.__dict__["irreps_in"].num_irreps, l.__dict__["irreps_out"].num_irreps) for l in (lin0, lin1, lin2)]
+        (c0, o0), (c1, hidden), (h2, o2) = dims
+        if not (o0 == 1 and o2 == 1 and c0 == c1 and h2 == hidden and 1 <= hidden <= 16 and c0 <= 256):
+            return None
+        if getattr(gate, "f", None) is not torch.nn.functional.silu or len(r1.non_linearity.acts) != 1:
+            return None
+        if scale_shift.scale.numel() != 1 or scale_shift.shift.numel() != 1:
+            return None
+        w1 = lin0.weight.data.double().reshape(c0) / sqrt(c0)
+        W2a = lin1.weight.data.double().reshape(c1, hidden) / sqrt(c1)
+        w2b = lin2.weight.data.double().reshape(hidden) / sqrt(hidden)
+        return {"w1": w1.contiguous(), "W2a": W2a.contiguous(), "w2b": w2b.contiguous(), "act_cst": float(gate.cst),
+                "scale": float(scale_shift.scale), "shift": float(scale_shift.shift)}
+    except (AttributeError, KeyError, TypeError, ValueError, IndexError, RuntimeError):
+        return None
 
 
 # ---- model pieces -----------------------------------------------------------------------------------------
@@ -222,10 +249,13 @@ class InvariantResidualInteraction(torch.nn.Module):
 
 
 class OptimizedInvariantMACE(torch.nn.Module):
-    def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True):
+    def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True,
+                 fused_readout: bool = True):
         """fused_radial=True evaluates the spherical harmonics and the radial spline inside the message-passing kernels
         (same numbers; no [16, nedges] or [nedges, 4C] tensors in memory); False keeps the reference's separate
-        SphericalHarmonics -> CubicSpline -> message passing steps."""
+        SphericalHarmonics -> CubicSpline -> message passing steps.  fused_readout=True evaluates both readouts, scale
+        and shift in one fp64 kernel per direction when the readout modules have the standard form; False (or any other
+        form, or several heads) runs the modules themselves in fp64 as the reference does."""
         super().__init__()
         self.fused_radial = bool(fused_radial)
         assert int(mace_model.num_interactions) == 2, "exactly two interaction layers are supported"
@@ -262,6 +292,15 @@ class OptimizedInvariantMACE(torch.nn.Module):
         self.edge_splines = torch.nn.ModuleList(edge_splines)
 
         self.scale_shift = deepcopy(mace_model.scale_shift).double()
+        # both readouts, scale and shift as one fp64 kernel per direction when the modules have the standard form;
+        # otherwise the modules themselves run, as in the reference
+        fused = fused_readout_parameters(mace_model.readouts, mace_model.scale_shift)
+        self.fused_readout = bool(fused_readout) and fused is not None
+        if self.fused_readout:
+            self.register_buffer("readout_w1", fused["w1"])
+            self.register_buffer("readout_W2a", fused["W2a"])
+            self.register_buffer("readout_w2b", fused["w2b"])
+            self.readout_constants = (fused["act_cst"], fused["scale"], fused["shift"])
         self.to(device)
         # inference model: the custom ops differentiate with respect to features and geometry only, so no weight
         # needs a gradient; frozen weights also let autograd skip dX of the first layer, whose input depends on
@@ -279,8 +318,8 @@ class OptimizedInvariantMACE(torch.nn.Module):
         positions = data["positions"]
         node_attrs = data["node_attrs"]
         batch = data["batch"]
-        node_heads = data["head"][batch] if "head" in data else torch.zeros_like(batch)
-        num_atoms_arange = torch.arange(positions.shape[0], device=positions.device)
+        node_heads = data["head"][batch] if "head" in data else None  # None: every node reads head 0
+        zero_heads = None if node_heads is not None else _cached(batch, "_cm_zero_heads", None, lambda: torch.zeros_like(batch))
         num_graphs = data["ptr"].numel() - 1
         shifts = data["shifts"]
         cell = data.get("cell")
@@ -301,7 +340,7 @@ class OptimizedInvariantMACE(torch.nn.Module):
                         self.interactions[0].linear_up(self.node_embedding(attrs64).float()))
 
         e0_per_head, node_feats_up = _cached(node_attrs, "_cm_species_only", id(self), species_only)
-        node_e0 = _select_head(e0_per_head, node_heads)
+        node_e0 = _select_head(e0_per_head, zero_heads if node_heads is None else node_heads)
         e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs)
         node_feats = None
 
@@ -319,21 +358,29 @@ class OptimizedInvariantMACE(torch.nn.Module):
         # fused mode: the message-passing kernels take the vectors themselves and evaluate the harmonics per edge
         edge_attrs = None if self.fused_radial else self.spherical_harmonics.forward(vectors32)
 
+        fused_readout = self.fused_readout and node_heads is None
         node_es_list, node_feats_list = [], []
         for interaction, product, readout, edge_spline in zip(self.interactions, self.products, self.readouts, self.edge_splines):
             edge_feats = None if self.fused_radial else edge_spline.forward(lengths32)
             node_feats, sc = interaction(node_attrs=node_attrs32,
-                                         node_feats=node_feats_up if node_feats is None else node_feats.float(),
+                                         node_feats=node_feats_up if node_feats is None else node_feats,
                                          edge_attrs=edge_attrs, edge_feats=edge_feats, edge_index=data["edge_index"],
                                          sender=sender, receiver=receiver, edge_lengths=lengths32, edge_spline=edge_spline,
                                          edge_vectors=vectors32, node_feats_are_up=node_feats is None)
-            node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types).double()
+            node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types)  # fp32 [N, C]
             node_feats_list.append(node_feats)
-            node_es_list.append(_select_head(readout(node_feats, node_heads), node_heads))
+            if not fused_readout:
+                heads = zero_heads if node_heads is None else node_heads
+                node_es_list.append(_select_head(readout(node_feats.double(), heads), heads))
 
-        node_feats_out = torch.cat(node_feats_list, dim=-1)
-        node_inter_es = torch.sum(torch.stack(node_es_list, dim=0), dim=0)
-        node_inter_es = self.scale_shift(node_inter_es, node_heads)
+        if fused_readout:
+            act_cst, scale, shift = self.readout_constants
+            node_inter_es, node_feats_out = ReadoutEnergyAutograd.apply(
+                node_feats_list[0], node_feats_list[1], self.readout_w1, self.readout_W2a, self.readout_w2b, act_cst, scale, shift)
+        else:
+            node_feats_out = torch.cat([f.double() for f in node_feats_list], dim=-1)
+            node_inter_es = torch.sum(torch.stack(node_es_list, dim=0), dim=0)
+            node_inter_es = self.scale_shift(node_inter_es, zero_heads if node_heads is None else node_heads)
         inter_e = scatter_sum(src=node_inter_es.double(), index=batch, dim=-1, dim_size=num_graphs)
 
         total_energy = e0 + inter_e

@@ -128,14 +128,38 @@ class _LinearReadout(torch.nn.Module):
         return self.linear(x)
 
 
+class _Normalize2Mom(torch.nn.Module):
+    """f scaled to unit second moment under a standard normal input (what e3nn's normalize2mom wraps a gate in)."""
+
+    def __init__(self, f, cst: float):
+        super().__init__()
+        self.f = f
+        self.cst = float(cst)
+
+    def forward(self, x):
+        return self.cst * self.f(x)
+
+
+class _Activation(torch.nn.Module):
+    """Gate on scalar features, holding its functions in `acts` like e3nn's nn.Activation."""
+
+    def __init__(self):
+        super().__init__()
+        self.acts = torch.nn.ModuleList([_Normalize2Mom(torch.nn.functional.silu, SILU_2MOM)])
+
+    def forward(self, x):
+        return self.acts[0](x)
+
+
 class _NonLinearReadout(torch.nn.Module):
     def __init__(self, channels: int, hidden: int, generator: torch.Generator):
         super().__init__()
         self.linear_1 = _Linear0e(channels, hidden, generator)
+        self.non_linearity = _Activation()
         self.linear_2 = _Linear0e(hidden, 1, generator)
 
     def forward(self, x, heads=None):
-        return self.linear_2(SILU_2MOM * torch.nn.functional.silu(self.linear_1(x)))
+        return self.linear_2(self.non_linearity(self.linear_1(x)))
 
 
 class _ScaleShift(torch.nn.Module):

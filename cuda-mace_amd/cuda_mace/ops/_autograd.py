@@ -168,6 +168,25 @@ class EdgeGeometryAutograd(torch.autograd.Function):
         return gpos, gshift, None, None
 
 
+class ReadoutEnergyAutograd(torch.autograd.Function):
+    """(h1, h2 fp32 [N, C]) -> (node energies fp64 [N], node_feats fp64 [N, 2C]): both readouts, scale and shift in one
+    kernel; the derivative with respect to h2 is produced by the same pass and only scaled in the backward."""
+
+    @staticmethod
+    def forward(ctx, h1, h2, w1, W2a, w2b, act_cst, scale, shift):
+        es, d2, feats = cabi.readout_forward(h1.detach().contiguous(), h2.detach().contiguous(), w1, W2a, w2b, act_cst, scale, shift)
+        ctx.save_for_backward(w1, d2)
+        ctx.scale = float(scale)
+        ctx.mark_non_differentiable(feats)
+        return es, feats
+
+    @staticmethod
+    def backward(ctx, grad_es, _grad_feats):
+        w1, d2 = ctx.saved_tensors
+        g1, g2 = cabi.readout_backward(grad_es.contiguous(), w1, d2, ctx.scale, ctx.needs_input_grad[0], ctx.needs_input_grad[1])
+        return g1, g2, None, None, None, None, None, None
+
+
 # ------------------------------------------------------------------------------------------------
 def monomials_from_packed(U3_num, U3_idx, U3_val, U2_num, U2_idx, U2_val):
     """Host pass over the packed sparse coupling tables (format of ops/symmetric_contraction.py:91-187):

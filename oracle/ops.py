@@ -293,3 +293,13 @@ def neighbour_list(positions: np.ndarray, cell, pbc, cutoff: float):
     arr = np.array(sorted(set(rows)), dtype=np.int64)
     assert arr.shape[0] == len(rows), "an image was visited twice"
     return arr[:, :2].T.copy(), arr[:, 2:].copy()
+
+
+# -----------------------------------------------------------------------------------------------
+def readout_energies(h1, h2, w1, W2a, w2b, act_cst: float, scale: float, shift: float):
+    """Node energies of the two readouts the reference's model applies in fp64 to the per-layer node features
+    (models/InvariantMACE.py:330-337: linear readout of layer 1, one-hidden-layer readout with a normalised silu gate
+    of layer 2) followed by scale and shift (:343).  Weights come with their 1/sqrt(fan_in) folded in."""
+    h1, h2 = h1.double(), h2.double()
+    z = h2 @ W2a.double()
+    return scale * (h1 @ w1.double() + (act_cst * torch.nn.functional.silu(z)) @ w2b.double()) + shift

@@ -20,12 +20,14 @@ def _say(*a):
     print(*a, flush=True)
 
 
-def _build(channels, numbers, data, seed, fused=True):
+def _build(channels, numbers, data, seed, fused=True, fused_readout=True):
     from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
 
     avg = data["edge_index"].shape[1] / data["positions"].shape[0]
     up = SyntheticInvariantMACE(channels=channels, atomic_numbers=numbers, avg_num_neighbors=avg, seed=seed)
-    return up.export_params(), OptimizedInvariantMACE(up, device="cuda", fused_radial=fused)
+    model = OptimizedInvariantMACE(up, device="cuda", fused_radial=fused, fused_readout=fused_readout)
+    assert model.fused_readout == fused_readout
+    return up.export_params(), model
 
 
 def _compare(params, model, data):
@@ -50,6 +52,8 @@ def test_cluster_config1(cabi):
     out, ref = _compare(params, model, data)
     _, unfused = _build(64, (1, 6, 7, 8), data, seed=0, fused=False)
     _compare(params, unfused, data)
+    _, module_readouts = _build(64, (1, 6, 7, 8), data, seed=0, fused_readout=False)  # the readout modules themselves
+    _compare(params, module_readouts, data)
     assert out["energy"].shape == (1,) and out["forces"].shape == (21, 3)
     assert set(out) == {"energy", "node_energy", "interaction_energy", "forces", "virials", "stress", "hessian",
                         "displacement", "node_feats", "edge_forces"}

@@ -356,3 +356,28 @@ def test_edge_geometry(cabi, nnodes, avg, iso, seed):
     vec2, _ = O.edge_geometry(pos, row_a, row_b, shifts)
     (vec2 * gv.float().double()).sum().backward()
     close(only_vec, pos.grad, 1e-12, 1e-13)
+
+
+# ---- readouts ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("N,C,H,seed", [(1, 32, 16, 0), (1000, 128, 16, 1), (37, 96, 5, 2), (515, 256, 1, 3), (16, 64, 16, 4)])
+def test_readout_forward_backward(cabi, N, C, H, seed):
+    g = torch.Generator().manual_seed(seed)
+    h1 = torch.randn(N, C, generator=g).double()
+    h2 = torch.randn(N, C, generator=g).double()
+    w1 = torch.randn(C, generator=g, dtype=torch.float64) / C ** 0.5
+    W2a = torch.randn(C, H, generator=g, dtype=torch.float64) / C ** 0.5
+    w2b = torch.randn(H, generator=g, dtype=torch.float64) / H ** 0.5
+    gn = torch.randn(N, generator=g, dtype=torch.float64)
+    cst, scale, shift = 1.6791767923989418, 0.8, -0.3
+    a1, a2 = h1.clone().requires_grad_(True), h2.clone().requires_grad_(True)
+    ref = O.readout_energies(a1, a2, w1, W2a, w2b, cst, scale, shift)
+    (ref * gn).sum().backward()
+    dev = lambda t: t.to(DEV)
+    es, d2, feats = cabi.readout_forward(dev(h1.float()), dev(h2.float()), dev(w1), dev(W2a), dev(w2b), cst, scale, shift)
+    close(es, ref.detach(), 1e-12, 1e-12)  # fp64 arithmetic on identical (fp32-representable) inputs
+    assert torch.equal(feats.cpu(), torch.cat([h1, h2], dim=1))
+    g1, g2 = cabi.readout_backward(dev(gn), dev(w1), d2, scale)
+    close(g1, a1.grad, 1e-6, 1e-7)
+    close(g2, a2.grad, 1e-6, 1e-7)
+    only2 = cabi.readout_backward(dev(gn), dev(w1), d2, scale, need_h1=False)
+    assert only2[0] is None and torch.equal(only2[1], g2)
