@@ -29,12 +29,13 @@ constexpr int kTileNodes = 32 * kWaves;  // rows per workgroup (MFMA M = 32 per 
 constexpr int kKC = 32;                  // K columns staged per step
 constexpr int kLd = kKC + 4;             // padded LDS row stride (floats)
 
-template <int NT>  // Nout = 32 * NT
+template <int NT, bool SCALED>  // Nout = 32 * NT; SCALED: X is multiplied by row_scale on the way in
 __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__restrict__ X, const float *__restrict__ WT,
                                                                const int32_t *__restrict__ node_perm,
                                                                const int32_t *__restrict__ group_offsets, int nnodes,
                                                                int ngroups, int zero_last_group, int ncomp, int K,
-                                                               float scale, float *__restrict__ OUT) {
+                                                               float scale, const float *__restrict__ row_scale,
+                                                               float *__restrict__ OUT) {
   constexpr int NOUT = 32 * NT;
   __shared__ __attribute__((aligned(16))) float sA[kTileNodes * kLd];
   __shared__ __attribute__((aligned(16))) float sB[NOUT * kLd];
@@ -96,48 +97,63 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
 
-  // staging map: 8 threads x 16 bytes cover the 32 staged columns of a row; 32 rows per pass
-  const int srow = tid / 8;
-  const int scol = (tid % 8) * 4;
+  // staging map: kKC / 4 threads x 16 bytes cover the staged columns of a row
+  constexpr int kTPR = kKC / 4;                    // threads per row
+  constexpr int kRPP = kWaves * kWave / kTPR;      // rows per pass
+  const int srow = tid / kTPR;
+  const int scol = (tid % kTPR) * 4;
   // MFMA operand map: row / column within the 32-wide block and which half of the 8-wide k step
   const int mrow = lane % 32;
   const int half = lane / 32;
 
-  constexpr int A_PASSES = kTileNodes / 32;
-  constexpr int B_PASSES = NOUT / 32;
-  f4 pa[A_PASSES], pb[B_PASSES];
+  constexpr int A_PASSES = kTileNodes / kRPP;
+  constexpr int B_PASSES = NOUT / kRPP;
+  f4 pa[A_PASSES], pb[B_PASSES], ps[SCALED ? A_PASSES : 1];
   // global -> register prefetch of one K chunk; the next chunk is in flight while the current one is multiplied
   auto prefetch = [&](int kc) {
 #pragma unroll
     for (int i = 0; i < A_PASSES; ++i) {
-      const int node = sNode[32 * i + srow];
+      const int node = sNode[kRPP * i + srow];
       pa[i] = zero4();
-      if (node >= 0) pa[i] = ld4_stream(X + (static_cast<int64_t>(node) * ncomp + m) * K + kc + scol);
+      if (node >= 0) {
+        pa[i] = ld4_stream(X + (static_cast<int64_t>(node) * ncomp + m) * K + kc + scol);
+        // optional per-node, per-column factor shared by all components (the contraction's upstream gradient); it is
+        // applied when the chunk moves to LDS, so that nothing waits for these loads here
+        if constexpr (SCALED) ps[i] = ld4(row_scale + static_cast<int64_t>(node) * K + kc + scol);
+      }
     }
 #pragma unroll
-    for (int i = 0; i < B_PASSES; ++i) pb[i] = ld4(Wg + static_cast<int64_t>(32 * i + srow) * K + kc + scol);
+    for (int i = 0; i < B_PASSES; ++i) pb[i] = ld4(Wg + static_cast<int64_t>(kRPP * i + srow) * K + kc + scol);
   };
   prefetch(0);
   for (int kc = 0; kc < K; kc += kKC) {
     __syncthreads();  // previous chunk fully consumed
 #pragma unroll
-    for (int i = 0; i < A_PASSES; ++i) *reinterpret_cast<f4 *>(sA + (32 * i + srow) * kLd + scol) = pa[i];
+    for (int i = 0; i < A_PASSES; ++i) {
+      f4 v = pa[i];
+      if constexpr (SCALED) v *= ps[i];
+      *reinterpret_cast<f4 *>(sA + (kRPP * i + srow) * kLd + scol) = v;
+    }
 #pragma unroll
-    for (int i = 0; i < B_PASSES; ++i) *reinterpret_cast<f4 *>(sB + (32 * i + srow) * kLd + scol) = pb[i];
+    for (int i = 0; i < B_PASSES; ++i) *reinterpret_cast<f4 *>(sB + (kRPP * i + srow) * kLd + scol) = pb[i];
     __syncthreads();
     if (kc + kKC < K) prefetch(kc + kKC);
 
 #pragma unroll
     for (int kb = 0; kb < kKC; kb += 8) {
       const f4 a = *reinterpret_cast<const f4 *>(sA + (32 * wave + mrow) * kLd + kb + 4 * half);
+      f4 b[NT];
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        const f4 b = *reinterpret_cast<const f4 *>(sB + (32 * t + mrow) * kLd + kb + 4 * half);
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc[t], 0, 0, 0);
-      }
+      for (int t = 0; t < NT; ++t) b[t] = *reinterpret_cast<const f4 *>(sB + (32 * t + mrow) * kLd + kb + 4 * half);
+      // consecutive MFMAs go to different accumulators, so none waits for the result of the one before it
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b[t].x, acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b[t].y, acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b[t].z, acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b[t].w, acc[t], 0, 0, 0);
     }
   }
 
@@ -156,10 +172,15 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
 
 template <int NT>
 int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
-           int zero_last_group, int ncomp, int K, float scale, float *OUT, hipStream_t st) {
+           int zero_last_group, int ncomp, int K, float scale, const float *row_scale, float *OUT, hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
-  hipLaunchKernelGGL(linear_kernel<NT>, dim3(static_cast<unsigned>(tiles), ncomp), dim3(kWaves * kWave), 0, st, X, WT, perm,
-                     offs, static_cast<int>(nnodes), ngroups, zero_last_group, ncomp, K, scale, OUT);
+  const dim3 grid(static_cast<unsigned>(tiles), ncomp), block(kWaves * kWave);
+  if (row_scale)
+    hipLaunchKernelGGL((linear_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                       zero_last_group, ncomp, K, scale, row_scale, OUT);
+  else
+    hipLaunchKernelGGL((linear_kernel<NT, false>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                       zero_last_group, ncomp, K, scale, row_scale, OUT);
   return check_launch("cm_linear");
 }
 
@@ -168,7 +189,7 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
 
 extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_perm, const int32_t *group_offsets,
                          int64_t nnodes, int ngroups, int zero_last_group, int ncomp, int K, int Nout, float scale,
-                         float *OUT, cm_stream_t stream) {
+                         const float *row_scale, float *OUT, cm_stream_t stream) {
   CM_REQUIRE(ncomp == 1 || ncomp == 16, "cm_linear: ncomp=%d must be 1 or 16", ncomp);
   CM_REQUIRE(!zero_last_group || (group_offsets != nullptr && ngroups >= 2),
              "cm_linear: a zero group needs node_perm / group_offsets and at least one weight group before it");
@@ -182,14 +203,14 @@ extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_p
   CM_REQUIRE(X && W_T && OUT, "cm_linear: NULL pointer");
   hipStream_t st = cm::as_stream(stream);
   switch (Nout / 32) {
-    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
-    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
-    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
-    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
-    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
-    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
-    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
-    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, OUT, st);
+    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
+    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
+    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
+    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
+    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
+    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
+    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
+    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
   }
   return CM_EINVAL;
 }

@@ -21,7 +21,9 @@ from cuda_mace.ops.invariant_message_passing import InvariantMessagePassingTP
 from cuda_mace.ops.linear import ElementalLinear, Linear, ScalarElementalLinear
 from cuda_mace.ops.spherical_harmonics import SphericalHarmonics
 from cuda_mace.ops.symmetric_contraction import SymmetricContraction as CUDAContraction
-from cuda_mace.ops._autograd import EdgeGeometryAutograd, ReadoutEnergyAutograd, _cached
+from cuda_mace import _cabi as cabi
+from cuda_mace.ops._autograd import (EdgeGeometryAutograd, LinearContractionAutograd, ReadoutEnergyAutograd, _cached, groups_of,
+                                     groups_of_one_hot, monomials_from_packed)
 from cuda_mace.utils.irreps import Instruction
 
 
@@ -208,20 +210,30 @@ class InvariantInteraction(torch.nn.Module):
         self.compose_linears = True
 
     def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,
-                edge_lengths=None, edge_spline=None, edge_vectors=None, node_feats_are_up: bool = False):
-        """node_feats_are_up: node_feats is already linear_up(embedding) (the model caches it per species tensor)."""
+                edge_lengths=None, edge_spline=None, edge_vectors=None, node_feats_are_up: bool = False,
+                apply_linear: bool = True):
+        """node_feats_are_up: node_feats is already linear_up(embedding) (the model caches it per species tensor).
+        apply_linear=False returns the message before the channel-mixing linears (the model then runs them fused with
+        the symmetric contraction, see `fused_linear`)."""
         if sender is None:
             sender, receiver = edge_index[1].int(), edge_index[0].int()
         if not node_feats_are_up:
             node_feats = self.linear_up(node_feats)
         message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline,
                                    edge_vectors)
+        if not apply_linear:
+            return message, None
         if self.compose_linears:
             message = self.skip_tp.cuda_obj.forward(message, self.composed_weights, self.composed_weights_transposed, node_attrs)
         else:
             message = self.linear(message)  # 1/avg_num_neighbors is folded into its weights
             message = self.skip_tp(message, node_attrs)
         return message, None
+
+    def fused_linear(self):
+        """(W_T, W, scale, per_element) of the channel mixing between message passing and the contraction."""
+        K = self.composed_weights.shape[-2]
+        return self.composed_weights_transposed, self.composed_weights, 1.0 / sqrt(K), True
 
 
 class InvariantResidualInteraction(torch.nn.Module):
@@ -237,25 +249,33 @@ class InvariantResidualInteraction(torch.nn.Module):
         self.avg_num_neighbors = inter.avg_num_neighbors
 
     def forward(self, node_attrs, node_feats, edge_attrs, edge_feats, edge_index, sender=None, receiver=None,
-                edge_lengths=None, edge_spline=None, edge_vectors=None, node_feats_are_up: bool = False):
+                edge_lengths=None, edge_spline=None, edge_vectors=None, node_feats_are_up: bool = False,
+                apply_linear: bool = True):
         if sender is None:
             sender, receiver = edge_index[1].int(), edge_index[0].int()
         sc = self.skip_tp(node_feats, node_attrs)
         node_feats = self.linear_up(node_feats)
         message = _message_passing(self.tp, node_feats, edge_attrs, edge_feats, sender, receiver, edge_lengths, edge_spline,
                                    edge_vectors)
-        message = self.linear(message)  # 1/avg_num_neighbors is folded into its weights
+        if apply_linear:
+            message = self.linear(message)  # 1/avg_num_neighbors is folded into its weights
         return message, sc
+
+    def fused_linear(self):
+        K = self.linear.weights.shape[-2]
+        return self.linear.weights_transposed, self.linear.weights, 1.0 / sqrt(K), False
 
 
 class OptimizedInvariantMACE(torch.nn.Module):
     def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True,
-                 fused_readout: bool = True):
+                 fused_readout: bool = True, fused_contraction: bool = True):
         """fused_radial=True evaluates the spherical harmonics and the radial spline inside the message-passing kernels
         (same numbers; no [16, nedges] or [nedges, 4C] tensors in memory); False keeps the reference's separate
         SphericalHarmonics -> CubicSpline -> message passing steps.  fused_readout=True evaluates both readouts, scale
         and shift in one fp64 kernel per direction when the readout modules have the standard form; False (or any other
-        form, or several heads) runs the modules themselves in fp64 as the reference does."""
+        form, or several heads) runs the modules themselves in fp64 as the reference does.  fused_contraction=True runs the
+        channel-mixing linear before each symmetric contraction and the contraction as one autograd node whose backward is
+        a single kernel; False keeps the reference's separate Linear / ElementalLinear and SymmetricContraction ops."""
         super().__init__()
         self.fused_radial = bool(fused_radial)
         assert int(mace_model.num_interactions) == 2, "exactly two interaction layers are supported"
@@ -301,7 +321,11 @@ class OptimizedInvariantMACE(torch.nn.Module):
             self.register_buffer("readout_W2a", fused["W2a"])
             self.register_buffer("readout_w2b", fused["w2b"])
             self.readout_constants = (fused["act_cst"], fused["scale"], fused["shift"])
+        self.fused_contraction = bool(fused_contraction)
         self.to(device)
+        self._contraction_builtin = None  # folded coefficient tables are made on the GPU, at the latest by the first step
+        if self.fused_contraction and torch.device(device).type == "cuda":
+            self._fold_contraction_tables()
         # inference model: the custom ops differentiate with respect to features and geometry only, so no weight
         # needs a gradient; frozen weights also let autograd skip dX of the first layer, whose input depends on
         # the species alone
@@ -310,6 +334,27 @@ class OptimizedInvariantMACE(torch.nn.Module):
         # kept for reference like upstream does, but not as a registered sub-module: moving or casting the
         # optimised model must not touch the caller's original model
         object.__setattr__(self, "orig_model", mace_model)
+
+    def _fold_contraction_tables(self):
+        """Per layer: the packed coupling tables regrouped into monomials (host, once) and folded with the per-element
+        weights into coefficient tables on the device."""
+        builtin3, builtin2 = cabi.symcon_builtin_structure()
+        self._contraction_builtin = []
+        for i, product in enumerate(self.products):
+            mod = product.symmetric_contractions.symmetric_contractions
+            (m3, o3, p3, v3), (m2, o2, p2, v2) = monomials_from_packed(mod.U3_num_nonsparse, mod.U3_indices, mod.U3_values,
+                                                                       mod.U2_num_nonsparse, mod.U2_indices, mod.U2_values)
+            dev = mod.weights_3.device
+            t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)  # noqa: E731
+            T3, T2, T1 = cabi.symcon_tables(t(o3), t(p3), t(v3), t(o2), t(p2), t(v2), mod.weights_3[0].contiguous(),
+                                            mod.weights_2[0].contiguous(), mod.weights_1[0].contiguous())
+            self._contraction_builtin.append(bool(np.array_equal(m3, builtin3) and np.array_equal(m2, builtin2)))
+            for name, val in (("mono3", t(m3)), ("mono2", t(m2)), ("T3", T3), ("T2", T2), ("T1", T1)):
+                self.register_buffer("contraction_%s_%d" % (name, i), val)
+
+    def _contraction_tables(self, i: int):
+        g = lambda name: getattr(self, "contraction_%s_%d" % (name, i))  # noqa: E731
+        return g("mono3"), g("mono2"), g("T3"), g("T2"), g("T1"), self._contraction_builtin[i]
 
     def forward(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
                 compute_virials: bool = False, compute_stress: bool = False,
@@ -366,8 +411,22 @@ class OptimizedInvariantMACE(torch.nn.Module):
                                          node_feats=node_feats_up if node_feats is None else node_feats,
                                          edge_attrs=edge_attrs, edge_feats=edge_feats, edge_index=data["edge_index"],
                                          sender=sender, receiver=receiver, edge_lengths=lengths32, edge_spline=edge_spline,
-                                         edge_vectors=vectors32, node_feats_are_up=node_feats is None)
-            node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types)  # fp32 [N, C]
+                                         edge_vectors=vectors32, node_feats_are_up=node_feats is None,
+                                         apply_linear=not self.fused_contraction)
+            if self.fused_contraction:
+                if self._contraction_builtin is None:
+                    self._fold_contraction_tables()
+                layer = len(node_feats_list)
+                W_T, W, scale, per_element = interaction.fused_linear()
+                ne = node_attrs32.shape[1]
+                contracted = LinearContractionAutograd.apply(
+                    node_feats, W_T, W, scale, groups_of_one_hot(node_attrs32) if per_element else None,
+                    groups_of(atom_types, ne), self._contraction_tables(layer))
+                node_feats = product.linear(contracted)  # fp32 [N, C]
+                if sc is not None and getattr(product, "use_sc", True):
+                    node_feats = node_feats + sc
+            else:
+                node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types)  # fp32 [N, C]
             node_feats_list.append(node_feats)
             if not fused_readout:
                 heads = zero_heads if node_heads is None else node_heads

@@ -168,6 +168,40 @@ class EdgeGeometryAutograd(torch.autograd.Function):
         return gpos, gshift, None, None
 
 
+class LinearContractionAutograd(torch.autograd.Function):
+    """Per-l (or per-element, per-l) linear followed by the symmetric contraction, as one autograd node:
+
+        Y = linear(X),  out = contraction(Y)          forward (Y is dropped, the contraction's gradient table kept)
+        gX = linear^T(grad_out[:, None, :] * grad)    backward, ONE kernel: the contraction's backward is folded into
+                                                      the operand load of the linear's backward
+
+    Same numbers as Linear / ElementalLinear -> SymmetricContraction; saves the [N,16,C] write and read between the two
+    backward kernels.  X [N,16,K]; W_T / W the transposed / plain weight blocks ([4,..] or [ne,4,..]) with `scale`;
+    lin_groups = (perm, offsets) for per-element weights or None; sym_groups = nodes grouped by element;
+    tables = (mono3, mono2, T3, T2, T1, builtin)."""
+
+    @staticmethod
+    def forward(ctx, X, W_T, W, scale, lin_groups, sym_groups, tables):
+        mono3, mono2, T3, T2, T1, builtin = tables
+        lp, lo = lin_groups if lin_groups is not None else (None, None)
+        # per-element weights: the grouping by one-hot row has one more group than there are weight blocks, for rows
+        # that name no element; those rows come out as zeros
+        Y = cabi.linear(X.contiguous(), W_T, lp, lo, scale, zero_last_group=lin_groups is not None)
+        out, grad = cabi.symcon_forward(Y, sym_groups[0], sym_groups[1], mono3, mono2, T3, T2, T1, want_grad=True,
+                                        builtin=builtin, zero_init=False)
+        ctx.save_for_backward(grad, W)
+        ctx.scale, ctx.lin_groups = scale, lin_groups
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        grad, W = ctx.saved_tensors
+        lp, lo = ctx.lin_groups if ctx.lin_groups is not None else (None, None)
+        gX = cabi.linear(grad, W, lp, lo, ctx.scale, zero_last_group=ctx.lin_groups is not None,
+                         row_scale=grad_out.contiguous())
+        return gX, None, None, None, None, None, None
+
+
 class ReadoutEnergyAutograd(torch.autograd.Function):
     """(h1, h2 fp32 [N, C]) -> (node energies fp64 [N], node_feats fp64 [N, 2C]): both readouts, scale and shift in one
     kernel; the derivative with respect to h2 is produced by the same pass and only scaled in the backward."""

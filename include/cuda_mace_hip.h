@@ -205,10 +205,15 @@ int cm_spline_backward(const float *r, const float *r_knots, const float *coeffs
  *   ngroups groups has no weights (W_T holds ngroups - 1 groups) and its rows are written as zeros: that is
  *   where nodes whose one-hot row names no element go.
  *   K and Nout: multiples of 32 in [32, 256].
+ *   row_scale fp32 [nnodes, K] or NULL: when given, X[n, m, k] is multiplied by row_scale[n, k] as it is read.
+ *   That is the backward of the symmetric contraction (gX[n, m, k] = grad_out[n, k] * grad[n, m, k],
+ *   cuda/src/symmetric_contraction_impl.cu:198-234) folded into the backward of the linear layer that precedes
+ *   the contraction: pass grad as X and grad_out as row_scale, and no [nnodes, 16, K] product is written.
  */
 int cm_linear(const float *X, const float *W_T, const int32_t *node_perm,
               const int32_t *group_offsets, int64_t nnodes, int ngroups, int zero_last_group,
-              int ncomp, int K, int Nout, float scale, float *OUT, cm_stream_t stream);
+              int ncomp, int K, int Nout, float scale, const float *row_scale, float *OUT,
+              cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Symmetric contraction, correlation 3, scalar (L = 0) output, with its analytic gradient.

@@ -20,12 +20,13 @@ def _say(*a):
     print(*a, flush=True)
 
 
-def _build(channels, numbers, data, seed, fused=True, fused_readout=True):
+def _build(channels, numbers, data, seed, fused=True, fused_readout=True, fused_contraction=True):
     from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
 
     avg = data["edge_index"].shape[1] / data["positions"].shape[0]
     up = SyntheticInvariantMACE(channels=channels, atomic_numbers=numbers, avg_num_neighbors=avg, seed=seed)
-    model = OptimizedInvariantMACE(up, device="cuda", fused_radial=fused, fused_readout=fused_readout)
+    model = OptimizedInvariantMACE(up, device="cuda", fused_radial=fused, fused_readout=fused_readout,
+                                   fused_contraction=fused_contraction)
     assert model.fused_readout == fused_readout
     return up.export_params(), model
 
@@ -54,6 +55,8 @@ def test_cluster_config1(cabi):
     _compare(params, unfused, data)
     _, module_readouts = _build(64, (1, 6, 7, 8), data, seed=0, fused_readout=False)  # the readout modules themselves
     _compare(params, module_readouts, data)
+    _, separate_ops = _build(64, (1, 6, 7, 8), data, seed=0, fused_contraction=False)  # Linear -> SymmetricContraction ops
+    _compare(params, separate_ops, data)
     assert out["energy"].shape == (1,) and out["forces"].shape == (21, 3)
     assert set(out) == {"energy", "node_energy", "interaction_energy", "forces", "virials", "stress", "hessian",
                         "displacement", "node_feats", "edge_forces"}
@@ -66,7 +69,7 @@ def test_periodic_box(cabi, natoms, channels, seed, fused):
     spline evaluated inside the message-passing kernels and with the reference's separate spline step."""
     _say("model periodic: N=%d C=%d seed=%d fused=%s" % (natoms, channels, seed, fused))
     data = make_system(natoms, 10, seed=seed, density=0.1)
-    params, model = _build(channels, tuple(range(1, 11)), data, seed=seed, fused=fused)
+    params, model = _build(channels, tuple(range(1, 11)), data, seed=seed, fused=fused, fused_contraction=fused)
     _compare(params, model, data)
 
 

@@ -381,3 +381,15 @@ def test_readout_forward_backward(cabi, N, C, H, seed):
     close(g2, a2.grad, 1e-6, 1e-7)
     only2 = cabi.readout_backward(dev(gn), dev(w1), d2, scale, need_h1=False)
     assert only2[0] is None and torch.equal(only2[1], g2)
+
+
+def test_linear_row_scale(cabi):
+    """row_scale folds an element-wise factor shared by the 16 components into the operand load."""
+    g = torch.Generator().manual_seed(3)
+    N, K, Nout = 300, 96, 128
+    X = torch.randn(N, 16, K, generator=g, dtype=torch.float64).float().double()
+    S = torch.randn(N, K, generator=g, dtype=torch.float64).float().double()
+    W = torch.randn(4, K, Nout, generator=g, dtype=torch.float64).float().double()
+    ref = O.linear(X * S[:, None, :], W)
+    got = cabi.linear(X.float().to(DEV), W.transpose(-1, -2).contiguous().float().to(DEV), row_scale=S.float().to(DEV))
+    close(got, ref, 1e-5, 2e-6)
