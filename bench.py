@@ -101,8 +101,8 @@ def isolated_ops(args, torch, cabi, make_system, reps=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--atoms", type=int, default=25000)
     ap.add_argument("--channels", type=int, default=128)
     ap.add_argument("--elements", type=int, default=10)

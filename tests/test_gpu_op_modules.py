@@ -145,3 +145,19 @@ def test_model_pickle_round_trip(cabi, tmp_path):
     back = torch.load(path, weights_only=False)
     out2 = back(to_device(data, DEV))
     assert torch.equal(out["energy"], out2["energy"]) and torch.equal(out["forces"], out2["forces"])
+
+
+def test_model_surgery_tool(cabi, tmp_path, capsys):
+    """The conversion tool end to end on a random-init model: optimise, time on the diamond test structure, save, reload."""
+    from cuda_mace.tools import model_surgery
+
+    path = tmp_path / "optimized.model"
+    model_surgery.main(["--synthetic", "32", "--size", "2", "--benchmark", "--accuracy", "--output", str(path)])
+    printed = capsys.readouterr().out
+    assert "optimized model time" in printed and "Saving optimized model" in printed
+    back = torch.load(path, weights_only=False)
+    batch = model_surgery.test_batch(back, 2)
+    assert batch["positions"].shape[0] == 64 and batch["edge_index"].shape[1] > 64 * 30
+    out = back(batch)
+    assert bool(torch.isfinite(out["energy"]).all()) and out["forces"].shape == (64, 3)
+    assert float(out["forces"].sum(0).abs().max()) < 1e-4 * max(1.0, float(out["forces"].abs().max()))
