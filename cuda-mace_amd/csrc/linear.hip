@@ -82,12 +82,14 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
   const int wave = tid / kWave;
-  const int m = blockIdx.y;  // component 0..ncomp-1
+  // the components of a tile are neighbours in the launch order: they share the tile's row_scale rows and touch
+  // adjacent rows of X and OUT while those are hot
+  const int m = blockIdx.x % ncomp;  // component 0..ncomp-1
   const int l = ncomp == 1 ? 0 : l_of_m(m);
   const int nblocks = ncomp == 1 ? 1 : 4;  // weight blocks per group
 
   // locate (group, first position in the grouped node order) of this tile
-  int tile = blockIdx.x;
+  int tile = blockIdx.x / ncomp;
   int g = 0, pos0 = 0, gend = nnodes;
   if (group_offsets) {
     bool found = false;
@@ -261,7 +263,7 @@ template <int NT>
 int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
            int zero_last_group, int ncomp, int K, float scale, const float *row_scale, float *OUT, hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
-  const dim3 grid(static_cast<unsigned>(tiles), ncomp), block(kWaves * kWave);
+  const dim3 grid(static_cast<unsigned>(tiles * ncomp)), block(kWaves * kWave);
   constexpr bool kSplit = NT <= 4 && CM_LINEAR_SPLIT_BF16;
   if (row_scale)
     hipLaunchKernelGGL((linear_kernel<NT, true, kSplit>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes),
