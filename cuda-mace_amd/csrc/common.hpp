@@ -65,6 +65,69 @@ __device__ __forceinline__ void st4_stream(float *p, f4 v) {
 __device__ __forceinline__ float hsum4(f4 a) { return (a.x + a.y) + (a.z + a.w); }
 // a . b as one multiply and three fused multiply-adds
 __device__ __forceinline__ float dot4(f4 a, f4 b) { return fmaf(a.w, b.w, fmaf(a.z, b.z, fmaf(a.y, b.y, a.x * b.x))); }
+// Three-wide variant for channel counts that fill the wave with three channels per lane (96, 192).  Loads and stores
+// are 12 bytes at 4-byte alignment.
+typedef float f3 __attribute__((ext_vector_type(3)));
+
+template <int V>
+struct VecOf;
+template <>
+struct VecOf<4> {
+  using type = f4;
+};
+template <>
+struct VecOf<3> {
+  using type = f3;
+};
+
+template <class T>
+__device__ __forceinline__ T zerov();
+template <>
+__device__ __forceinline__ f4 zerov<f4>() {
+  return zero4();
+}
+template <>
+__device__ __forceinline__ f3 zerov<f3>() {
+  return f3{0.f, 0.f, 0.f};
+}
+
+template <class T>
+__device__ __forceinline__ T ldv(const float *p);
+template <>
+__device__ __forceinline__ f4 ldv<f4>(const float *p) {
+  return ld4(p);
+}
+template <>
+__device__ __forceinline__ f3 ldv<f3>(const float *p) {
+  return f3{p[0], p[1], p[2]};
+}
+template <class T>
+__device__ __forceinline__ T ldv_stream(const float *p);
+template <>
+__device__ __forceinline__ f4 ldv_stream<f4>(const float *p) {
+  return ld4_stream(p);
+}
+template <>
+__device__ __forceinline__ f3 ldv_stream<f3>(const float *p) {
+  return f3{__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + 1), __builtin_nontemporal_load(p + 2)};
+}
+__device__ __forceinline__ void stv(float *p, f4 v) { st4(p, v); }
+__device__ __forceinline__ void stv(float *p, f3 v) {
+  p[0] = v.x;
+  p[1] = v.y;
+  p[2] = v.z;
+}
+__device__ __forceinline__ void stv_stream(float *p, f4 v) { st4_stream(p, v); }
+__device__ __forceinline__ void stv_stream(float *p, f3 v) {
+  __builtin_nontemporal_store(v.x, p);
+  __builtin_nontemporal_store(v.y, p + 1);
+  __builtin_nontemporal_store(v.z, p + 2);
+}
+__device__ __forceinline__ float hsumv(f4 a) { return hsum4(a); }
+__device__ __forceinline__ float hsumv(f3 a) { return (a.x + a.y) + a.z; }
+__device__ __forceinline__ float dotv(f4 a, f4 b) { return dot4(a, b); }
+__device__ __forceinline__ float dotv(f3 a, f3 b) { return fmaf(a.z, b.z, fmaf(a.y, b.y, a.x * b.x)); }
+
 __device__ __forceinline__ f4 shfl_down4(f4 v, int delta) {
   f4 r;
   r.x = __shfl_down(v.x, delta);
@@ -72,6 +135,10 @@ __device__ __forceinline__ f4 shfl_down4(f4 v, int delta) {
   r.z = __shfl_down(v.z, delta);
   r.w = __shfl_down(v.w, delta);
   return r;
+}
+__device__ __forceinline__ f4 shfl_downv(f4 v, int delta) { return shfl_down4(v, delta); }
+__device__ __forceinline__ f3 shfl_downv(f3 v, int delta) {
+  return f3{__shfl_down(v.x, delta), __shfl_down(v.y, delta), __shfl_down(v.z, delta)};
 }
 
 }  // namespace cm

@@ -62,6 +62,8 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
     const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes,
     int64_t nedges, float *__restrict__ out) {
   using K = Cfg<C>;
+  using vec = typename K::vec;
+  constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
 
@@ -73,9 +75,9 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
   const int e0 = first_occ[node];
   const int e1 = first_occ[nnodes + node];
 
-  f4 acc[16];
+  vec acc[16];
 #pragma unroll
-  for (int m = 0; m < 16; ++m) acc[m] = zero4();
+  for (int m = 0; m < 16; ++m) acc[m] = zerov<vec>();
 
   for (int base = e0; base < e1; base += kChunk) {
     const int cnt = min(kChunk, e1 - base);
@@ -87,16 +89,16 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
       for (int j = slot; j < cnt; j += K::EPW) {
         const int64_t e = base + j;
         const int s = sS[j];
-        const float *rp = R + e * (4 * C) + 4 * cl;
-        f4 r0 = ld4_stream(rp);
-        f4 r1 = ld4_stream(rp + C);
-        f4 r2 = ld4_stream(rp + 2 * C);
-        f4 r3 = ld4_stream(rp + 3 * C);
-        f4 x = zero4();
-        if (static_cast<unsigned>(s) < static_cast<unsigned>(nnodes)) x = ld4(X + static_cast<int64_t>(s) * C + 4 * cl);
+        const float *rp = R + e * (4 * C) + V * cl;
+        vec r0 = ldv_stream<vec>(rp);
+        vec r1 = ldv_stream<vec>(rp + C);
+        vec r2 = ldv_stream<vec>(rp + 2 * C);
+        vec r3 = ldv_stream<vec>(rp + 3 * C);
+        vec x = zerov<vec>();
+        if (static_cast<unsigned>(s) < static_cast<unsigned>(nnodes)) x = ldv<vec>(X + static_cast<int64_t>(s) * C + V * cl);
         const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
         const f4 ya = yp[0], yb = yp[1], yc = yp[2], yd = yp[3];
-        const f4 t0 = x * r0, t1 = x * r1, t2 = x * r2, t3 = x * r3;
+        const vec t0 = x * r0, t1 = x * r1, t2 = x * r2, t3 = x * r3;
         acc[0] += ya.x * t0;
         acc[1] += ya.y * t1;
         acc[2] += ya.z * t1;
@@ -121,12 +123,12 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
 #pragma unroll
   for (int off = kWave / 2; off >= K::SW; off >>= 1) {
 #pragma unroll
-    for (int m = 0; m < 16; ++m) acc[m] += shfl_down4(acc[m], off);
+    for (int m = 0; m < 16; ++m) acc[m] += shfl_downv(acc[m], off);
   }
   if (slot == 0 && active) {
-    float *op = out + static_cast<int64_t>(node) * (16 * C) + 4 * cl;
+    float *op = out + static_cast<int64_t>(node) * (16 * C) + V * cl;
 #pragma unroll
-    for (int m = 0; m < 16; ++m) st4(op + m * C, acc[m]);
+    for (int m = 0; m < 16; ++m) stv(op + m * C, acc[m]);
   }
 }
 
@@ -140,6 +142,8 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
     const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges, float *__restrict__ gY,
     float *__restrict__ gR, float *__restrict__ gXe) {
   using K = Cfg<C>;
+  using vec = typename K::vec;
+  constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
   __shared__ float sGY[16 * kChunk];  // [m][edge]
@@ -153,11 +157,11 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
   const int e1 = first_occ[nnodes + node];
   if (e0 >= e1) return;
 
-  f4 g[16];
+  vec g[16];
   {
-    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + 4 * cl;
+    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + V * cl;
 #pragma unroll
-    for (int m = 0; m < 16; ++m) g[m] = active ? ld4(gp + m * C) : zero4();
+    for (int m = 0; m < 16; ++m) g[m] = active ? ldv<vec>(gp + m * C) : zerov<vec>();
   }
   // which m this lane ends up holding after slot_reduce16
   const int myrev = ((cl & 1) << 3) | ((cl & 2) << 1) | ((cl & 4) >> 1) | ((cl & 8) >> 3);
@@ -171,57 +175,57 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
     for (int j = slot; j < cnt; j += K::EPW) {
       const int64_t e = base + j;
       const int s = sS[j];
-      f4 r0 = zero4(), r1 = zero4(), r2 = zero4(), r3 = zero4(), x = zero4();
+      vec r0 = zerov<vec>(), r1 = zerov<vec>(), r2 = zerov<vec>(), r3 = zerov<vec>(), x = zerov<vec>();
       if (active) {
-        const float *rp = R + e * (4 * C) + 4 * cl;
-        r0 = ld4_stream(rp);
-        r1 = ld4_stream(rp + C);
-        r2 = ld4_stream(rp + 2 * C);
-        r3 = ld4_stream(rp + 3 * C);
-        if (static_cast<unsigned>(s) < static_cast<unsigned>(nnodes)) x = ld4(X + static_cast<int64_t>(s) * C + 4 * cl);
+        const float *rp = R + e * (4 * C) + V * cl;
+        r0 = ldv_stream<vec>(rp);
+        r1 = ldv_stream<vec>(rp + C);
+        r2 = ldv_stream<vec>(rp + 2 * C);
+        r3 = ldv_stream<vec>(rp + 3 * C);
+        if (static_cast<unsigned>(s) < static_cast<unsigned>(nnodes)) x = ldv<vec>(X + static_cast<int64_t>(s) * C + V * cl);
       }
       const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
       const f4 ya = yp[0], yb = yp[1], yc = yp[2], yd = yp[3];
 
       if constexpr (WANT_GR || WANT_GX) {
         // q_l = sum_{m in l} Y[m] g[m]
-        const f4 q0 = ya.x * g[0];
-        const f4 q1 = ya.y * g[1] + ya.z * g[2] + ya.w * g[3];
-        const f4 q2 = yb.x * g[4] + yb.y * g[5] + yb.z * g[6] + yb.w * g[7] + yc.x * g[8];
-        const f4 q3 = yc.y * g[9] + yc.z * g[10] + yc.w * g[11] + yd.x * g[12] + yd.y * g[13] +
+        const vec q0 = ya.x * g[0];
+        const vec q1 = ya.y * g[1] + ya.z * g[2] + ya.w * g[3];
+        const vec q2 = yb.x * g[4] + yb.y * g[5] + yb.z * g[6] + yb.w * g[7] + yc.x * g[8];
+        const vec q3 = yc.y * g[9] + yc.z * g[10] + yc.w * g[11] + yd.x * g[12] + yd.y * g[13] +
                       yd.z * g[14] + yd.w * g[15];
         if (active) {
           if constexpr (WANT_GR) {
-            float *gp = gR + e * (4 * C) + 4 * cl;
-            st4_stream(gp, x * q0);
-            st4_stream(gp + C, x * q1);
-            st4_stream(gp + 2 * C, x * q2);
-            st4_stream(gp + 3 * C, x * q3);
+            float *gp = gR + e * (4 * C) + V * cl;
+            stv_stream(gp, x * q0);
+            stv_stream(gp + C, x * q1);
+            stv_stream(gp + 2 * C, x * q2);
+            stv_stream(gp + 3 * C, x * q3);
           }
           if constexpr (WANT_GX) {
-            st4(gXe + e * C + 4 * cl, r0 * q0 + r1 * q1 + r2 * q2 + r3 * q3);
+            stv(gXe + e * C + V * cl, r0 * q0 + r1 * q1 + r2 * q2 + r3 * q3);
           }
         }
       }
       if constexpr (WANT_GY) {
-        const f4 t0 = x * r0, t1 = x * r1, t2 = x * r2, t3 = x * r3;
+        const vec t0 = x * r0, t1 = x * r1, t2 = x * r2, t3 = x * r3;
         float p[16];
-        p[0] = dot4(g[0], t0);
-        p[1] = dot4(g[1], t1);
-        p[2] = dot4(g[2], t1);
-        p[3] = dot4(g[3], t1);
-        p[4] = dot4(g[4], t2);
-        p[5] = dot4(g[5], t2);
-        p[6] = dot4(g[6], t2);
-        p[7] = dot4(g[7], t2);
-        p[8] = dot4(g[8], t2);
-        p[9] = dot4(g[9], t3);
-        p[10] = dot4(g[10], t3);
-        p[11] = dot4(g[11], t3);
-        p[12] = dot4(g[12], t3);
-        p[13] = dot4(g[13], t3);
-        p[14] = dot4(g[14], t3);
-        p[15] = dot4(g[15], t3);
+        p[0] = dotv(g[0], t0);
+        p[1] = dotv(g[1], t1);
+        p[2] = dotv(g[2], t1);
+        p[3] = dotv(g[3], t1);
+        p[4] = dotv(g[4], t2);
+        p[5] = dotv(g[5], t2);
+        p[6] = dotv(g[6], t2);
+        p[7] = dotv(g[7], t2);
+        p[8] = dotv(g[8], t2);
+        p[9] = dotv(g[9], t3);
+        p[10] = dotv(g[10], t3);
+        p[11] = dotv(g[11], t3);
+        p[12] = dotv(g[12], t3);
+        p[13] = dotv(g[13], t3);
+        p[14] = dotv(g[14], t3);
+        p[15] = dotv(g[15], t3);
         slot_reduce16<K::SW>(p, cl);
         if constexpr (K::SW >= 16) {
           if (cl < 16) sGY[myrev * kChunk + j] = p[0];
@@ -251,6 +255,8 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
     const float *__restrict__ gXe, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ offsets, int nnodes, int64_t nedges, float *__restrict__ gX) {
   using K = Cfg<C>;
+  using vec = typename K::vec;
+  constexpr int V = K::V;
   const int node = blockIdx.x;
   const int lane = threadIdx.x;
   const int slot = lane / K::SW;
@@ -258,26 +264,26 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
   const bool active = cl < K::LPE;
   const int k0 = offsets[node];
   const int k1 = offsets[node + 1];
-  f4 acc = zero4();
+  vec acc = zerov<vec>();
   if (active) {
     // four independent row gathers in flight per slot; the summation order stays fixed
     int k = k0 + slot;
     for (; k + 3 * K::EPW < k1; k += 4 * K::EPW) {
       const int ea = perm[k], eb = perm[k + K::EPW], ec = perm[k + 2 * K::EPW], ed = perm[k + 3 * K::EPW];
-      const f4 va = static_cast<unsigned>(ea) < static_cast<uint64_t>(nedges) ? ld4(gXe + static_cast<int64_t>(ea) * C + 4 * cl) : zero4();
-      const f4 vb = static_cast<unsigned>(eb) < static_cast<uint64_t>(nedges) ? ld4(gXe + static_cast<int64_t>(eb) * C + 4 * cl) : zero4();
-      const f4 vc = static_cast<unsigned>(ec) < static_cast<uint64_t>(nedges) ? ld4(gXe + static_cast<int64_t>(ec) * C + 4 * cl) : zero4();
-      const f4 vd = static_cast<unsigned>(ed) < static_cast<uint64_t>(nedges) ? ld4(gXe + static_cast<int64_t>(ed) * C + 4 * cl) : zero4();
+      const vec va = static_cast<unsigned>(ea) < static_cast<uint64_t>(nedges) ? ldv<vec>(gXe + static_cast<int64_t>(ea) * C + V * cl) : zerov<vec>();
+      const vec vb = static_cast<unsigned>(eb) < static_cast<uint64_t>(nedges) ? ldv<vec>(gXe + static_cast<int64_t>(eb) * C + V * cl) : zerov<vec>();
+      const vec vc = static_cast<unsigned>(ec) < static_cast<uint64_t>(nedges) ? ldv<vec>(gXe + static_cast<int64_t>(ec) * C + V * cl) : zerov<vec>();
+      const vec vd = static_cast<unsigned>(ed) < static_cast<uint64_t>(nedges) ? ldv<vec>(gXe + static_cast<int64_t>(ed) * C + V * cl) : zerov<vec>();
       acc += (va + vb) + (vc + vd);
     }
     for (; k < k1; k += K::EPW) {
       const int e = perm[k];
-      if (static_cast<unsigned>(e) < static_cast<uint64_t>(nedges)) acc += ld4(gXe + static_cast<int64_t>(e) * C + 4 * cl);
+      if (static_cast<unsigned>(e) < static_cast<uint64_t>(nedges)) acc += ldv<vec>(gXe + static_cast<int64_t>(e) * C + V * cl);
     }
   }
 #pragma unroll
-  for (int off = kWave / 2; off >= K::SW; off >>= 1) acc += shfl_down4(acc, off);
-  if (slot == 0 && active) st4(gX + static_cast<int64_t>(node) * C + 4 * cl, acc);
+  for (int off = kWave / 2; off >= K::SW; off >>= 1) acc += shfl_downv(acc, off);
+  if (slot == 0 && active) stv(gX + static_cast<int64_t>(node) * C + V * cl, acc);
 }
 
 template <int C>

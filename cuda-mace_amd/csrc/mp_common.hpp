@@ -16,10 +16,14 @@ constexpr int pow2ceil(int v) {
 
 template <int C>
 struct Cfg {
-  static constexpr int LPE = C / 4;          // lanes that carry one edge
+  // channels per lane: four (one 16-byte access per row), except where three fill the lanes exactly (96 -> 32 lanes,
+  // 192 -> 64 lanes) and four would leave a quarter of them idle
+  static constexpr int V = (C == 96 || C == 192) ? 3 : 4;
+  static constexpr int LPE = C / V;          // lanes that carry one edge
   static constexpr int SW = pow2ceil(LPE);   // slot width in lanes (power of two)
   static constexpr int EPW = kWave / SW;     // edges in flight per wave
-  static_assert(C % 32 == 0 && C >= 32 && C <= 256, "channel count");
+  using vec = typename VecOf<V>::type;
+  static_assert(C % 32 == 0 && C >= 32 && C <= 256 && C % V == 0, "channel count");
 };
 
 // Stages Y[0:16, base:base+cnt] (transposed to [edge][16]) and sender[base:base+cnt] in LDS.

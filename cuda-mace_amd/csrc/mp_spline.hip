@@ -112,6 +112,8 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
                                                                  const int32_t *__restrict__ first_occ, int nnodes,
                                                                  int64_t nedges, float *__restrict__ out) {
   using K = Cfg<C>;
+  using vec = typename K::vec;
+  constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
   __shared__ int sIdx[kChunk];
@@ -125,9 +127,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
   const int e0 = first_occ[node];
   const int e1 = first_occ[nnodes + node];
 
-  f4 acc[16];
+  vec acc[16];
 #pragma unroll
-  for (int m = 0; m < 16; ++m) acc[m] = zero4();
+  for (int m = 0; m < 16; ++m) acc[m] = zerov<vec>();
 
   for (int base = e0; base < e1; base += kChunk) {
     const int cnt = min(kChunk, e1 - base);
@@ -140,7 +142,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
         const int idx = sIdx[j];
         if (idx < 0 || static_cast<unsigned>(s) >= static_cast<unsigned>(nnodes)) continue;
         const float xr = sXr[j];
-        const f4 x = ld4(X + (static_cast<unsigned>(s) * C + 4u * cl));
+        const vec x = ldv<vec>(X + (static_cast<unsigned>(s) * C + unsigned(V) * cl));
         float y[16];
         {
           const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
@@ -150,13 +152,13 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
             y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
           }
         }
-        const unsigned co = static_cast<unsigned>(idx) * (16u * C) + 4u * cl;  // 32-bit offset from the uniform table base
+        const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(V) * cl;  // 32-bit offset from the uniform table base
         const float *__restrict__ tab = sp.coeffs;
         auto per_l = [&](auto lc) {
           constexpr int L = decltype(lc)::value;
-          const f4 a = ld4(tab + (co + L * C)), b = ld4(tab + (co + (4 * C + L * C))), c = ld4(tab + (co + (8 * C + L * C))),
-                   d = ld4(tab + (co + (12 * C + L * C)));
-          const f4 t = x * (a + xr * (b + xr * (c + xr * d)));
+          const vec a = ldv<vec>(tab + (co + L * C)), b = ldv<vec>(tab + (co + (4 * C + L * C))), c = ldv<vec>(tab + (co + (8 * C + L * C))),
+                   d = ldv<vec>(tab + (co + (12 * C + L * C)));
+          const vec t = x * (a + xr * (b + xr * (c + xr * d)));
 #pragma unroll
           for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) acc[m] += y[m] * t;
         };
@@ -171,12 +173,12 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
 #pragma unroll
   for (int off = kWave / 2; off >= K::SW; off >>= 1) {
 #pragma unroll
-    for (int m = 0; m < 16; ++m) acc[m] += shfl_down4(acc[m], off);
+    for (int m = 0; m < 16; ++m) acc[m] += shfl_downv(acc[m], off);
   }
   if (slot == 0 && active) {
-    float *op = out + static_cast<int64_t>(node) * (16 * C) + 4 * cl;
+    float *op = out + static_cast<int64_t>(node) * (16 * C) + V * cl;
 #pragma unroll
-    for (int m = 0; m < 16; ++m) st4(op + m * C, acc[m]);
+    for (int m = 0; m < 16; ++m) stv(op + m * C, acc[m]);
   }
 }
 
@@ -189,6 +191,8 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
     const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges,
     float *__restrict__ gY, float *__restrict__ g_r, float *__restrict__ gXe) {
   using K = Cfg<C>;
+  using vec = typename K::vec;
+  constexpr int V = K::V;
   constexpr bool kRotate = !WANT_GX;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
@@ -207,11 +211,11 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
   const int e1 = first_occ[nnodes + node];
   if (e0 >= e1) return;
 
-  f4 g[16];
+  vec g[16];
   {
-    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + 4 * cl;
+    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + V * cl;
 #pragma unroll
-    for (int m = 0; m < 16; ++m) g[m] = active ? ld4(gp + m * C) : zero4();
+    for (int m = 0; m < 16; ++m) g[m] = active ? ldv<vec>(gp + m * C) : zerov<vec>();
   }
 
   for (int base = e0; base < e1; base += kChunk) {
@@ -224,7 +228,7 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
     // rotated form the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
     // arithmetic of the current one, so they travel while the cross-lane reductions (a chain of dependent lane
     // exchanges) run.
-    f4 x, ca[4], cb[4], cc[4], cd[4];
+    vec x, ca[4], cb[4], cc[4], cd[4];
     float xr;
     bool live;
     auto fetch = [&](int j) {
@@ -232,15 +236,15 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
       const int idx = sIdx[j];
       live = idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
       xr = sXr[j];
-      x = ld4(X + ((live ? static_cast<unsigned>(s) : 0u) * C + 4u * cla));
-      const unsigned co = static_cast<unsigned>(idx < 0 ? 0 : idx) * (16u * C) + 4u * cla;
+      x = ldv<vec>(X + ((live ? static_cast<unsigned>(s) : 0u) * C + unsigned(V) * cla));
+      const unsigned co = static_cast<unsigned>(idx < 0 ? 0 : idx) * (16u * C) + unsigned(V) * cla;
       const float *__restrict__ tab = sp.coeffs;
 #pragma unroll
       for (int L = 0; L < 4; ++L) {
-        ca[L] = ld4(tab + (co + L * C));
-        cb[L] = ld4(tab + (co + (4 * C + L * C)));
-        cc[L] = ld4(tab + (co + (8 * C + L * C)));
-        cd[L] = ld4(tab + (co + (12 * C + L * C)));
+        ca[L] = ldv<vec>(tab + (co + L * C));
+        cb[L] = ldv<vec>(tab + (co + (4 * C + L * C)));
+        cc[L] = ldv<vec>(tab + (co + (8 * C + L * C)));
+        cd[L] = ldv<vec>(tab + (co + (12 * C + L * C)));
       }
     };
     if constexpr (kRotate) {
@@ -260,19 +264,19 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
       }
       const float xr2 = 2.f * xr, xr3 = 3.f * xr * xr;
       float p[16];
-      f4 gxe = zero4();
-      f4 grq = zero4();
+      vec gxe = zerov<vec>();
+      vec grq = zerov<vec>();
       auto per_l = [&](auto lc) {
         constexpr int L = decltype(lc)::value;
-        const f4 a = ca[L], b = cb[L], c = cc[L], d = cd[L];
-        const f4 rl = a + xr * (b + xr * (c + xr * d));
-        f4 q = zero4();
+        const vec a = ca[L], b = cb[L], c = cc[L], d = cd[L];
+        const vec rl = a + xr * (b + xr * (c + xr * d));
+        vec q = zerov<vec>();
 #pragma unroll
         for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) q += y[m] * g[m];
         if constexpr (WANT_GY) {
-          const f4 t = x * rl;
+          const vec t = x * rl;
 #pragma unroll
-          for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) p[m] = dot4(g[m], t);
+          for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) p[m] = dotv(g[m], t);
         }
         if constexpr (WANT_GX) gxe += rl * q;
         if constexpr (WANT_GR) grq += q * (b + xr2 * c + xr3 * d);  // q_l * dR_l/dr
@@ -281,16 +285,16 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
       per_l(std::integral_constant<int, 1>{});
       per_l(std::integral_constant<int, 2>{});
       per_l(std::integral_constant<int, 3>{});
-      if constexpr (WANT_GX) gxe = live ? gxe : zero4();
+      if constexpr (WANT_GX) gxe = live ? gxe : zerov<vec>();
       float grv = 0.f;
-      if constexpr (WANT_GR) grv = hsum4(x * grq);
+      if constexpr (WANT_GR) grv = hsumv(x * grq);
 
       if constexpr (kRotate) {
         if (j + K::EPW < cnt) fetch(j + K::EPW);
       }
 
       if constexpr (WANT_GX) {
-        if (active) st4(gXe + e * C + 4 * cl, gxe);
+        if (active) stv(gXe + e * C + V * cl, gxe);
       }
       if constexpr (WANT_GR) {
         const float tot = slot_sum<K::SW>(grv);
