@@ -156,8 +156,11 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
         const float *__restrict__ tab = sp.coeffs;
         auto per_l = [&](auto lc) {
           constexpr int L = decltype(lc)::value;
-          const vec a = ldv<vec>(tab + (co + L * C)), b = ldv<vec>(tab + (co + (4 * C + L * C))), c = ldv<vec>(tab + (co + (8 * C + L * C))),
-                   d = ldv<vec>(tab + (co + (12 * C + L * C)));
+          // addressed from the middle of the interval's 16C-float row: all 16 pieces lie within +-8C floats of it, which
+          // up to C = 128 fits the signed immediate offset of a load, so one address serves them all
+          const float *mid = tab + (co + 8 * C);
+          const vec a = ldv<vec>(mid + (L * C - 8 * C)), b = ldv<vec>(mid + (L * C - 4 * C)), c = ldv<vec>(mid + L * C),
+                    d = ldv<vec>(mid + (L * C + 4 * C));
           const vec t = x * (a + xr * (b + xr * (c + xr * d)));
 #pragma unroll
           for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) acc[m] += y[m] * t;
@@ -241,10 +244,21 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
       const float *__restrict__ tab = sp.coeffs;
 #pragma unroll
       for (int L = 0; L < 4; ++L) {
-        ca[L] = ldv<vec>(tab + (co + L * C));
-        cb[L] = ldv<vec>(tab + (co + (4 * C + L * C)));
-        cc[L] = ldv<vec>(tab + (co + (8 * C + L * C)));
-        cd[L] = ldv<vec>(tab + (co + (12 * C + L * C)));
+        if constexpr (kRotate || V == 3) {
+          // addressed from the middle of the interval's 16C-float row (offsets within +-8C floats: one address and
+          // immediate offsets, up to C = 128)
+          const float *mid = tab + (co + 8 * C);
+          ca[L] = ldv<vec>(mid + (L * C - 8 * C));
+          cb[L] = ldv<vec>(mid + (L * C - 4 * C));
+          cc[L] = ldv<vec>(mid + L * C);
+          cd[L] = ldv<vec>(mid + (L * C + 4 * C));
+        } else {
+          // the variant with gX at four channels per lane measured faster with 32-bit offsets from the table base
+          ca[L] = ldv<vec>(tab + (co + L * C));
+          cb[L] = ldv<vec>(tab + (co + (4 * C + L * C)));
+          cc[L] = ldv<vec>(tab + (co + (8 * C + L * C)));
+          cd[L] = ldv<vec>(tab + (co + (12 * C + L * C)));
+        }
       }
     };
     if constexpr (kRotate) {
