@@ -25,13 +25,14 @@ constexpr int kNodes = 16;    // nodes per workgroup
 constexpr int kHidden = 16;   // threads per node = largest hidden width handled
 constexpr int kMaxC = 256;
 constexpr int kLdW = kHidden + 1;  // padded row stride of the weight tile in LDS (doubles)
+constexpr int kLdS = kMaxC + 1;    // padded row stride of the feature tile: the four nodes of a wave hit different banks
 
 __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     const float *__restrict__ h1, const float *__restrict__ h2, const double *__restrict__ w1, const double *__restrict__ W2a,
     const double *__restrict__ w2b, double act_cst, double scale, double shift, int nnodes, int C, int H,
     double *__restrict__ node_es, float *__restrict__ d2, double *__restrict__ feats64) {
   __shared__ double sW[kMaxC * kLdW];      // W2a [C, H], H padded to 16 columns with zeros
-  __shared__ float s2[kNodes * kMaxC];
+  __shared__ float s2[kNodes * kLdS];
   __shared__ double sD[kNodes * kHidden];  // w2b[j] * act'(z_j) per node
   const int t = threadIdx.x;
   const int node0 = blockIdx.x * kNodes;
@@ -44,7 +45,7 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     const int r = i / C, c = i % C;
     const float b = h2[static_cast<int64_t>(node0 + r) * C + c];
     const float a = feats64 ? h1[static_cast<int64_t>(node0 + r) * C + c] : 0.f;
-    s2[r * kMaxC + c] = b;
+    s2[r * kLdS + c] = b;
     if (feats64) {
       feats64[static_cast<int64_t>(node0 + r) * (2 * C) + c] = a;
       feats64[static_cast<int64_t>(node0 + r) * (2 * C) + C + c] = b;
@@ -58,7 +59,7 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
   if (live) {
     const float *row1 = h1 + static_cast<int64_t>(node0 + r) * C;
     for (int c = j; c < C; c += kHidden) e1 += static_cast<double>(row1[c]) * w1[c];
-    for (int c = 0; c < C; ++c) z += static_cast<double>(s2[r * kMaxC + c]) * sW[c * kLdW + j];
+    for (int c = 0; c < C; ++c) z += static_cast<double>(s2[r * kLdS + c]) * sW[c * kLdW + j];
   }
   double e2 = 0.0, dj = 0.0;
   if (live && j < H) {

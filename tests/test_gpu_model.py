@@ -34,7 +34,7 @@ def _build(channels, numbers, data, seed, fused=True, fused_readout=True, fused_
 def _compare(params, model, data):
     ref = M.energy_and_forces(params, data)
     out = model(to_device(data, "cuda"))
-    e, e_ref = float(out["interaction_energy"].cpu()), float(ref["interaction_energy"])
+    e, e_ref = float(out["interaction_energy"].detach().cpu()), float(ref["interaction_energy"])
     f_err = float((out["forces"].double().cpu() - ref["forces"]).abs().max())
     _say("  E %.10g ref %.10g rel %.2e | max|dF| %.2e (max|F| %.3g)" % (e, e_ref, abs(e - e_ref) / abs(e_ref), f_err,
                                                                        float(ref["forces"].abs().max())))
