@@ -171,6 +171,21 @@ def main():
 
     setattr(cabi, bwd_name, timed(bwd_name, originals[bwd_name], lambda k: not k.get("need_gX", True)))
     setattr(cabi, fwd_name, timed(fwd_name, originals[fwd_name], lambda k: True))
+    # the 16-component channel-mixing launches (forward ones: no row_scale), when the model routes them through the C ABI
+    events["linear"] = []
+    originals["linear"] = cabi.linear
+
+    def timed_linear(X, *a, **k):
+        if X.dim() != 3 or k.get("row_scale") is not None:
+            return originals["linear"](X, *a, **k)
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        r = originals["linear"](X, *a, **k)
+        e.record()
+        events["linear"].append((s, e))
+        return r
+
+    cabi.linear = timed_linear
 
     torch.cuda.synchronize()
     t_start = time.perf_counter()
@@ -204,20 +219,35 @@ def main():
     t_bwd, t_fwd = avg_ms(bwd_name), avg_ms(fwd_name)
     if fused:
         sh_b, spline_b = 88 * E, 4 * (8 * E * C + E)  # harmonics backward, spline backward (each operand once)
-        roofline = entry("mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb, t_bwd,
-                         launches_timed=len(events[bwd_name]),
-                         note="harmonics and radial weights are evaluated in-kernel, so the kernel's own HBM operands are "
-                              "small; the radial coefficients come from the 2 MB spline table in L2 (16 loads of 16 B per "
-                              "lane and edge) and the backward occupies ~80% of all VALU issue slots: bounded by VALU issue "
-                              "and L1 delivery, not HBM; see roofline_other_kernels for the HBM-bound message passing with "
-                              "tabulated R[E,4,C]",
+        sh_f, spline_f = 76 * E, 4 * (E + 8 * E * C)  # harmonics forward, spline forward (each operand once)
+        roofline = entry("mp_spline_forward_kernel<%d,true>" % C, fwd_fb, t_fwd, launches_timed=len(events[fwd_name]),
+                         note="dominant kernel of the step by total time (two launches per step). Harmonics and radial "
+                              "weights are evaluated in-kernel, so its own HBM operands are small: the radial coefficients "
+                              "come from the 2 MB spline table in L2 (16 loads of 16 B per lane and edge, texture-address "
+                              "units ~80% busy): bounded by L1 delivery, not HBM; see roofline_other_kernels for the "
+                              "HBM-bound message passing with tabulated R[E,4,C] and for the matrix-core linear",
                          unfused_equivalent={
-                             "bytes": bwd_b + sh_b + spline_b,
-                             "GB/s": round((bwd_b + sh_b + spline_b) / (t_bwd * 1e-3) / 1e9, 1),
-                             "meaning": "algorithmic HBM bytes of the three separate kernels this launch replaces (message-"
-                                        "passing backward with tabulated R, spline backward, harmonics backward) divided by "
-                                        "this launch's duration"})
-        others = [entry("mp_spline_forward_kernel<%d,true>" % C, fwd_fb, t_fwd)]
+                             "bytes": fwd_b + sh_f + spline_f,
+                             "GB/s": round((fwd_b + sh_f + spline_f) / (t_fwd * 1e-3) / 1e9, 1),
+                             "meaning": "algorithmic HBM bytes of the three separate kernels this launch replaces (message "
+                                        "passing with tabulated R, spline evaluation, harmonics) divided by this launch's "
+                                        "duration"})
+        others = [entry("mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb, t_bwd,
+                        launches_timed=len(events[bwd_name]),
+                        note="bounded by VALU issue (~80% of all issue slots), see the counter summary")]
+        t_lin = avg_ms("linear")
+        if t_lin:
+            flops = 32 * N * C * C
+            tf = flops / (t_lin * 1e-3) / 1e12
+            others.append({"kernel": "linear_kernel<%d,false>" % (C // 32), "bound": "mfma", "achieved": round(tf, 1),
+                           "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4), "traffic": None,
+                           "algorithmic_flops_per_launch": flops, "avg_launch_ms": round(t_lin, 4),
+                           "launches_timed": len(events["linear"]),
+                           "note": "fp32-equivalent flops of the [N,16,C] x [C,C] channel mixing against the fp32 matrix "
+                                   "peak; the kernel computes them as six bf16 piece products per fp32 product on "
+                                   "v_mfma_f32_32x32x16_bf16 (6x the instruction flops: %.0f TFLOP/s of the 2500 TFLOP/s "
+                                   "bf16 peak) and is bound by its %d MB of memory traffic per launch"
+                                   % (6 * tf, 4 * (32 * N * C + 4 * C * C) // 10**6)})
     else:
         roofline = entry("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b, t_bwd,
                          launches_timed=len(events[bwd_name]))
