@@ -61,39 +61,46 @@ __device__ __forceinline__ void locate(const Spline &sp, float re, int &idx, flo
   }
 }
 
-// Stages, for the chunk's edges, sender, Y (transposed to [edge][16]), knot interval and offset.  FROM_VEC: Y and the
-// length come from the edge vector; otherwise from the Y and r arrays.
+// Stages the chunk's LIVE edges -- those inside the cutoff whose sender index is valid -- densely, in their original
+// order: sender, Y (as [edge][16]), knot interval, offset inside it, and the position of the edge in the chunk.  Returns
+// their number (the same in every lane); my_live tells a lane whether the edge base + lane is one of them.  Edges
+// beyond the cutoff (a neighbour list with a skin has many) cost nothing after this point.  FROM_VEC: Y and the length
+// come from the edge vector; otherwise from the Y and r arrays.
 template <bool FROM_VEC>
-__device__ __forceinline__ void stage_edges(const float *__restrict__ Y, const int32_t *__restrict__ sender, const Spline &sp,
-                                            int64_t nedges, int base, int cnt, int lane, float *sY, int *sS, int *sIdx,
-                                            float *sXr) {
-  if constexpr (!FROM_VEC) {
-    stage_chunk(Y, sender, nedges, base, cnt, lane, sY, sS);
-    if (lane < cnt) {
-      int idx;
-      float x;
-      locate(sp, sp.r[base + lane], idx, x);
-      sIdx[lane] = idx;
-      sXr[lane] = x;
-    }
-  } else {
-    if (lane < cnt) {
-      const int64_t e = base + lane;
-      sS[lane] = sender[e];
-      const float v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
-      const float re = sqrtf(v0 * v0 + v1 * v1 + v2 * v2);
-      int idx;
-      float x;
-      locate(sp, re, idx, x);
-      sIdx[lane] = idx;
-      sXr[lane] = x;
-      float y[16];
-      sh::eval(sh::direction(v0, v1, v2), y);
+__device__ __forceinline__ int stage_edges(const float *__restrict__ Y, const int32_t *__restrict__ sender, const Spline &sp,
+                                           int nnodes, int64_t nedges, int base, int cnt, int lane, float *sY, int *sS,
+                                           int *sIdx, float *sXr, int *sOrig, bool &my_live, unsigned long long &live_mask) {
+  int s = -1, idx = -1;
+  float x = 0.f;
+  float y[16];
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        *reinterpret_cast<f4 *>(sY + lane * 16 + 4 * q) = f4{y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]};
+  for (int m = 0; m < 16; ++m) y[m] = 0.f;
+  if (lane < cnt) {
+    const int64_t e = base + lane;
+    s = sender[e];
+    if constexpr (FROM_VEC) {
+      const float v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
+      locate(sp, sqrtf(v0 * v0 + v1 * v1 + v2 * v2), idx, x);
+      sh::eval(sh::direction(v0, v1, v2), y);
+    } else {
+      locate(sp, sp.r[e], idx, x);
+#pragma unroll
+      for (int m = 0; m < 16; ++m) y[m] = Y[m * nedges + e];
     }
   }
+  my_live = lane < cnt && idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
+  live_mask = __ballot(my_live);
+  if (my_live) {
+    const int pos = __popcll(live_mask & ((1ull << lane) - 1ull));
+    sS[pos] = s;
+    sIdx[pos] = idx;
+    sXr[pos] = x;
+    sOrig[pos] = lane;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      *reinterpret_cast<f4 *>(sY + pos * 16 + 4 * q) = f4{y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]};
+  }
+  return __popcll(live_mask);
 }
 
 template <int L>
@@ -118,6 +125,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
   __shared__ int sS[kChunk];
   __shared__ int sIdx[kChunk];
   __shared__ float sXr[kChunk];
+  __shared__ int sOrig[kChunk];
 
   const int node = blockIdx.x;
   const int lane = threadIdx.x;
@@ -134,13 +142,15 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
   for (int base = e0; base < e1; base += kChunk) {
     const int cnt = min(kChunk, e1 - base);
     __syncthreads();
-    stage_edges<FROM_VEC>(Y, sender, sp, nedges, base, cnt, lane, sY, sS, sIdx, sXr);
+    bool my_live;
+    unsigned long long live_mask;
+    const int nlive = stage_edges<FROM_VEC>(Y, sender, sp, nnodes, nedges, base, cnt, lane, sY, sS, sIdx, sXr, sOrig, my_live,
+                                            live_mask);
     __syncthreads();
     if (active) {
-      for (int j = slot; j < cnt; j += K::EPW) {
+      for (int j = slot; j < nlive; j += K::EPW) {
         const int s = sS[j];
         const int idx = sIdx[j];
-        if (idx < 0 || static_cast<unsigned>(s) >= static_cast<unsigned>(nnodes)) continue;
         const float xr = sXr[j];
         const vec x = ldv<vec>(X + (static_cast<unsigned>(s) * C + unsigned(V) * cl));
         float y[16];
@@ -201,6 +211,7 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
   __shared__ int sS[kChunk];
   __shared__ int sIdx[kChunk];
   __shared__ float sXr[kChunk];
+  __shared__ int sOrig[kChunk];
   __shared__ float sGY[16 * kChunk];  // [m][edge]
   __shared__ float sGr[kChunk];
 
@@ -224,23 +235,23 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
   for (int base = e0; base < e1; base += kChunk) {
     const int cnt = min(kChunk, e1 - base);
     __syncthreads();
-    stage_edges<FROM_VEC>(Y, sender, sp, nedges, base, cnt, lane, sY, sS, sIdx, sXr);
+    bool my_live;
+    unsigned long long live_mask;
+    const int nlive = stage_edges<FROM_VEC>(Y, sender, sp, nnodes, nedges, base, cnt, lane, sY, sS, sIdx, sXr, sOrig, my_live,
+                                            live_mask);
     __syncthreads();
-    // Every lane of a slot takes part in the reductions, so the loop bound is slot-uniform.  Edges beyond the cutoff
-    // or with an invalid sender read clamped addresses and are zeroed where their results are stored.  In the
-    // rotated form the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
+    // Every lane of a slot takes part in the reductions, so the loop bound is slot-uniform; only live edges are staged.
+    // In the rotated form the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
     // arithmetic of the current one, so they travel while the cross-lane reductions (a chain of dependent lane
     // exchanges) run.
     vec x, ca[4], cb[4], cc[4], cd[4];
     float xr;
-    bool live;
     auto fetch = [&](int j) {
       const int s = sS[j];
       const int idx = sIdx[j];
-      live = idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
       xr = sXr[j];
-      x = ldv<vec>(X + ((live ? static_cast<unsigned>(s) : 0u) * C + unsigned(V) * cla));
-      const unsigned co = static_cast<unsigned>(idx < 0 ? 0 : idx) * (16u * C) + unsigned(V) * cla;
+      x = ldv<vec>(X + (static_cast<unsigned>(s) * C + unsigned(V) * cla));
+      const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(V) * cla;
       const float *__restrict__ tab = sp.coeffs;
 #pragma unroll
       for (int L = 0; L < 4; ++L) {
@@ -262,10 +273,9 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
       }
     };
     if constexpr (kRotate) {
-      if (slot < cnt) fetch(slot);
+      if (slot < nlive) fetch(slot);
     }
-    for (int j = slot; j < cnt; j += K::EPW) {
-      const int64_t e = base + j;
+    for (int j = slot; j < nlive; j += K::EPW) {
       if constexpr (!kRotate) fetch(j);
       float y[16];
       {
@@ -299,16 +309,15 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
       per_l(std::integral_constant<int, 1>{});
       per_l(std::integral_constant<int, 2>{});
       per_l(std::integral_constant<int, 3>{});
-      if constexpr (WANT_GX) gxe = live ? gxe : zerov<vec>();
       float grv = 0.f;
       if constexpr (WANT_GR) grv = hsumv(x * grq);
 
       if constexpr (kRotate) {
-        if (j + K::EPW < cnt) fetch(j + K::EPW);
+        if (j + K::EPW < nlive) fetch(j + K::EPW);
       }
 
       if constexpr (WANT_GX) {
-        if (active) stv(gXe + e * C + V * cl, gxe);
+        if (active) stv(gXe + static_cast<int64_t>(base + sOrig[j]) * C + V * cl, gxe);
       }
       if constexpr (WANT_GR) {
         const float tot = slot_sum<K::SW>(grv);
@@ -319,11 +328,30 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
         store_reduced16<K::SW>(p, cl, j, sGY);
       }
     }
+    if constexpr (WANT_GX) {
+      // rows of edges that are not live: zero, the sender pass sums every row
+      for (int k = slot; k < cnt; k += K::EPW)
+        if (!((live_mask >> k) & 1ull) && active) stv(gXe + static_cast<int64_t>(base + k) * C + V * cl, zerov<vec>());
+    }
     if constexpr (WANT_GY || WANT_GR) {
       __syncthreads();
-      if (lane < cnt) {
+      // lane k < nlive finishes the k-th live edge; lanes whose own edge is not live write its zeros
+      if (lane < cnt && !my_live) {
         const int64_t e = base + lane;
-        const bool dead = sIdx[lane] < 0 || static_cast<unsigned>(sS[lane]) >= static_cast<unsigned>(nnodes);
+        if constexpr (FROM_VEC) {
+          gY[3 * e + 0] = 0.f;
+          gY[3 * e + 1] = 0.f;
+          gY[3 * e + 2] = 0.f;
+        } else {
+          if constexpr (WANT_GY) {
+#pragma unroll
+            for (int m = 0; m < 16; ++m) gY[m * nedges + e] = 0.f;
+          }
+          if constexpr (WANT_GR) g_r[e] = 0.f;
+        }
+      }
+      if (lane < nlive) {
+        const int64_t e = base + sOrig[lane];
         if constexpr (FROM_VEC) {
           // gradient with respect to the edge vector: harmonics Jacobian applied to gY, plus g_r along the direction
           // (gY doubles as the output pointer of the [E, 3] vector gradient in this variant)
@@ -334,15 +362,15 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
           for (int m = 0; m < 16; ++m) gy[m] = sGY[m * kChunk + lane];
           sh::vjp(d, gy, gin);
           const float gr = sGr[lane];
-          gY[3 * e + 0] = dead ? 0.f : gin[0] + gr * d.y;
-          gY[3 * e + 1] = dead ? 0.f : gin[1] + gr * d.z;
-          gY[3 * e + 2] = dead ? 0.f : gin[2] + gr * d.x;
+          gY[3 * e + 0] = gin[0] + gr * d.y;
+          gY[3 * e + 1] = gin[1] + gr * d.z;
+          gY[3 * e + 2] = gin[2] + gr * d.x;
         } else {
           if constexpr (WANT_GY) {
 #pragma unroll
-            for (int m = 0; m < 16; ++m) gY[m * nedges + e] = dead ? 0.f : sGY[m * kChunk + lane];
+            for (int m = 0; m < 16; ++m) gY[m * nedges + e] = sGY[m * kChunk + lane];
           }
-          if constexpr (WANT_GR) g_r[e] = dead ? 0.f : sGr[lane];
+          if constexpr (WANT_GR) g_r[e] = sGr[lane];
         }
       }
     }

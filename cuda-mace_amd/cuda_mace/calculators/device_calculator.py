@@ -22,14 +22,19 @@ from cuda_mace.utils.neighbour_list import get_neighborhood
 
 class DeviceCalculator:
     def __init__(self, model: torch.nn.Module, node_attrs: torch.Tensor, cutoff: Optional[float] = None, skin: float = 0.5,
-                 pbc: Sequence[bool] = (False, False, False), cell: Optional[torch.Tensor] = None, use_graph: bool = True,
-                 compute_stress: bool = False):
+                 pbc: Sequence[bool] = (False, False, False), cell: Optional[torch.Tensor] = None,
+                 use_graph: Optional[bool] = None, compute_stress: bool = False):
+        """use_graph: replay the step as one HIP graph between list rebuilds.  None decides by size: up to 8192 atoms the
+        step is bound by host launches and the graph pays for its re-capture after a rebuild; larger systems are bound
+        by the GPU and run eagerly."""
         self.model = model
         self.node_attrs = node_attrs
         self.cutoff = float(model.r_max) if cutoff is None else float(cutoff)
         self.skin = float(skin)
         self.pbc = tuple(bool(b) for b in pbc)
         self.cell = None if cell is None else cell.detach().double().reshape(3, 3).contiguous()
+        if use_graph is None:
+            use_graph = node_attrs.shape[0] <= 8192
         self.use_graph = bool(use_graph) and not compute_stress  # the strain path re-derives shifts from the cell
         self.compute_stress = bool(compute_stress)
         self.builds = 0
@@ -56,7 +61,7 @@ class DeviceCalculator:
             "ptr": torch.tensor([0, n], dtype=torch.int64, device=dev),
         }
         self._ref_positions = pos.clone()
-        self._graph = GraphedStep(self.model, self._data) if self.use_graph else None
+        self._graph = GraphedStep(self.model, self._data, warmup=1) if self.use_graph else None
         self.builds += 1
 
     # -- evaluation ----------------------------------------------------------------------------------------

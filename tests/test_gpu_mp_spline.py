@@ -98,3 +98,46 @@ def test_mp_spline_forward_backward(cabi, case):
     no_x = cabi.mp_spline_backward(d(X), d(Y), d(r), d(knots), d(coeffs), h, 5.0, d(G), snd.cuda(), fo, perm, off, nnodes,
                                    need_gX=False)
     assert no_x[0] is None and torch.equal(no_x[1], gY) and torch.equal(no_x[2], gr)
+
+
+def test_edges_beyond_cutoff_and_invalid_senders_cost_nothing_and_contribute_nothing(cabi):
+    """A list with a wide skin (most edges beyond r_max) and a few out-of-range sender indices: those edges add nothing
+    to the output and get exactly zero gradients; the rest matches the oracle evaluated on the live edges alone."""
+    nnodes, C, seed = 90, 128, 11
+    snd, rcv = random_graph(nnodes, 70, seed)
+    E = snd.numel()
+    X, _, _, G = mp_inputs(nnodes, E, C, seed)
+    g = torch.Generator().manual_seed(seed)
+    r = torch.rand(E, generator=g, dtype=torch.float64) * 9.0 + 0.7  # r_max = 5: about half the edges are beyond it
+    vec = torch.randn(E, 3, generator=g, dtype=torch.float64)
+    vec = (vec / vec.norm(dim=1, keepdim=True) * r[:, None]).float().double()
+    snd = snd.clone()
+    bad = torch.randperm(E, generator=g)[:40]
+    snd[bad[:20]] = nnodes + 3
+    snd[bad[20:]] = -1
+    knots_np, h = np.linspace(1e-12, 6.0, 256, retstep=True)
+    knots = torch.from_numpy(knots_np)
+    table = torch.cos(knots[:, None] * torch.linspace(0.3, 2.0, 4 * C, dtype=torch.float64)[None, :])
+    coeffs = O.spline_coefficients(knots, table).float().double()
+    h = float(np.float32(h))
+    live = (vec.norm(dim=1).float() <= 5.0) & (snd >= 0) & (snd < nnodes)
+    assert 0.3 < float(live.double().mean()) < 0.7
+
+    va = vec[live].clone().requires_grad_(True)
+    Xa = X.clone().requires_grad_(True)
+    Rv = O.spline_eval(va.norm(dim=1), knots.float().double(), coeffs, h, 5.0).view(-1, 4, C)
+    ref = O.mp_forward(Xa, O.spherical_harmonics(va), Rv, snd[live], rcv[live], nnodes)
+    (ref * G).sum().backward()
+
+    d = lambda t: t.float().cuda()
+    fo = cabi.first_occurences(rcv.cuda(), nnodes)
+    perm, off = cabi.stable_key_sort(snd.cuda(), nnodes)
+    out = cabi.mp_edge_forward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, snd.cuda(), fo, nnodes)
+    gX, gvec = cabi.mp_edge_backward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, d(G), snd.cuda(), fo, perm, off, nnodes)
+    close(out, ref.detach(), 2e-5, 2e-6)
+    close(gX, Xa.grad, 2e-5, 2e-6)
+    close(gvec[live.cuda()], va.grad, 5e-5, 5e-6)
+    assert float(gvec[~live.cuda()].abs().max()) == 0.0
+    gvec_only = cabi.mp_edge_backward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, d(G), snd.cuda(), fo, perm, off, nnodes,
+                                      need_gX=False)[1]
+    assert torch.equal(gvec_only, gvec)
