@@ -46,8 +46,17 @@ __device__ __forceinline__ void stage_chunk(const float *__restrict__ Y, const i
   }
 }
 
+// Value of `v` in the lane selected by a DPP control word (data-parallel-primitive operand swizzle of the VALU: no LDS
+// round trip).  0xB1 / 0x4E: quad_perm [1,0,3,2] / [2,3,0,1], i.e. lane ^ 1 / lane ^ 2; 0x124 / 0x128: rotate right by
+// 4 / 8 within each row of 16 lanes.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+
 // Sums p[m] over the SW lanes of a slot.  Butterfly with halving: after the exchange over lane
 // bit b each lane keeps half of its values, so 16 values cost 8+4+2+1 exchanges instead of 16*4.
+// The 12 exchanges over lane bits 0 and 1 stay inside a quad and go through DPP; the rest through ds_bpermute.
 // Returns, in every lane, the total for m = bitrev4(cl & 15) (SW >= 16), or for SW == 8 the two
 // totals m = bitrev3(cl) * 2 + {0, 1} in p[0], p[1].
 template <int SW>
@@ -59,7 +68,7 @@ __device__ __forceinline__ void slot_reduce16(float (&p)[16], int cl) {
     for (int k = 0; k < 8; ++k) {
       const float keep = hi ? p[8 + k] : p[k];
       const float send = hi ? p[k] : p[8 + k];
-      p[k] = keep + __shfl_xor(send, 1);
+      p[k] = keep + dpp_move<0xB1>(send);
     }
   }
   {
@@ -68,7 +77,7 @@ __device__ __forceinline__ void slot_reduce16(float (&p)[16], int cl) {
     for (int k = 0; k < 4; ++k) {
       const float keep = hi ? p[4 + k] : p[k];
       const float send = hi ? p[k] : p[4 + k];
-      p[k] = keep + __shfl_xor(send, 2);
+      p[k] = keep + dpp_move<0x4E>(send);
     }
   }
   {
@@ -90,11 +99,21 @@ __device__ __forceinline__ void slot_reduce16(float (&p)[16], int cl) {
   if constexpr (SW >= 64) p[0] += __shfl_xor(p[0], 32);
 }
 
-// Plain sum of one value over the SW lanes of a slot; every lane gets the total.
+// Plain sum of one value over the SW lanes of a slot; every lane gets the total.  Inside a row of 16 lanes: quad sums,
+// then rotations by 4 and 8 (all DPP); across rows: ds_bpermute.
 template <int SW>
 __device__ __forceinline__ float slot_sum(float v) {
+  static_assert(SW >= 8, "slot width");
+  v += dpp_move<0xB1>(v);
+  v += dpp_move<0x4E>(v);
+  if constexpr (SW >= 16) {
+    v += dpp_move<0x124>(v);
+    v += dpp_move<0x128>(v);
+  } else {
+    v += __shfl_xor(v, 4);
+  }
 #pragma unroll
-  for (int off = 1; off < SW; off <<= 1) v += __shfl_xor(v, off);
+  for (int off = 16; off < SW; off <<= 1) v += __shfl_xor(v, off);
   return v;
 }
 
