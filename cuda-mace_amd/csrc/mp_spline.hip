@@ -21,18 +21,13 @@
 #include "mp_common.hpp"
 #include "sh_device.hpp"
 
-// waves per SIMD the register allocator must leave room for (forward, backward edge pass)
+// waves per SIMD the register allocator must leave room for.  The backward edge pass runs with a rotated edge loop (the
+// next edge's loads are requested before the current edge's reductions), which needs the registers of two waves per SIMD.
 #ifndef CM_FUSED_FWD_WAVES
 #define CM_FUSED_FWD_WAVES 3
 #endif
 #ifndef CM_FUSED_BWD_WAVES
 #define CM_FUSED_BWD_WAVES 2
-#endif
-// The backward edge pass without the per-edge gX output runs with a rotated edge loop (next edge's loads requested
-// before the current edge's reductions), which needs the registers of two waves per SIMD.  The variant with gX is as
-// fast at two waves per SIMD as at three and, unlike at three, never spills (measured at 96, 128 and 192 channels).
-#ifndef CM_FUSED_BWD_ROTATED_WAVES
-#define CM_FUSED_BWD_ROTATED_WAVES 2
 #endif
 
 namespace cm {
@@ -199,14 +194,13 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
 // backward, edge pass: gY, g_r and the per-edge contribution to gX
 // -----------------------------------------------------------------------------------------------
 template <int C, bool FROM_VEC, bool WANT_GY, bool WANT_GR, bool WANT_GX>
-__global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_ROTATED_WAVES) void mp_spline_backward_edge_kernel(
+__global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_edge_kernel(
     const float *__restrict__ X, const float *__restrict__ Y, Spline sp, const float *__restrict__ G,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges,
     float *__restrict__ gY, float *__restrict__ g_r, float *__restrict__ gXe) {
   using K = Cfg<C>;
   using vec = typename K::vec;
   constexpr int V = K::V;
-  constexpr bool kRotate = !WANT_GX;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
   __shared__ int sIdx[kChunk];
@@ -241,7 +235,7 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
                                             live_mask);
     __syncthreads();
     // Every lane of a slot takes part in the reductions, so the loop bound is slot-uniform; only live edges are staged.
-    // In the rotated form the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
+    // The loop is rotated: the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
     // arithmetic of the current one, so they travel while the cross-lane reductions (a chain of dependent lane
     // exchanges) run.
     vec x, ca[4], cb[4], cc[4], cd[4];
@@ -255,28 +249,17 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
       const float *__restrict__ tab = sp.coeffs;
 #pragma unroll
       for (int L = 0; L < 4; ++L) {
-        if constexpr (kRotate || V == 3) {
-          // addressed from the middle of the interval's 16C-float row (offsets within +-8C floats: one address and
-          // immediate offsets, up to C = 128)
-          const float *mid = tab + (co + 8 * C);
-          ca[L] = ldv<vec>(mid + (L * C - 8 * C));
-          cb[L] = ldv<vec>(mid + (L * C - 4 * C));
-          cc[L] = ldv<vec>(mid + L * C);
-          cd[L] = ldv<vec>(mid + (L * C + 4 * C));
-        } else {
-          // the variant with gX at four channels per lane measured faster with 32-bit offsets from the table base
-          ca[L] = ldv<vec>(tab + (co + L * C));
-          cb[L] = ldv<vec>(tab + (co + (4 * C + L * C)));
-          cc[L] = ldv<vec>(tab + (co + (8 * C + L * C)));
-          cd[L] = ldv<vec>(tab + (co + (12 * C + L * C)));
-        }
+        // addressed from the middle of the interval's 16C-float row (offsets within +-8C floats: one address and
+        // immediate offsets, up to C = 128)
+        const float *mid = tab + (co + 8 * C);
+        ca[L] = ldv<vec>(mid + (L * C - 8 * C));
+        cb[L] = ldv<vec>(mid + (L * C - 4 * C));
+        cc[L] = ldv<vec>(mid + L * C);
+        cd[L] = ldv<vec>(mid + (L * C + 4 * C));
       }
     };
-    if constexpr (kRotate) {
-      if (slot < nlive) fetch(slot);
-    }
+    if (slot < nlive) fetch(slot);
     for (int j = slot; j < nlive; j += K::EPW) {
-      if constexpr (!kRotate) fetch(j);
       float y[16];
       {
         const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
@@ -312,9 +295,7 @@ __global__ __launch_bounds__(kWave, WANT_GX ? CM_FUSED_BWD_WAVES : CM_FUSED_BWD_
       float grv = 0.f;
       if constexpr (WANT_GR) grv = hsumv(x * grq);
 
-      if constexpr (kRotate) {
-        if (j + K::EPW < nlive) fetch(j + K::EPW);
-      }
+      if (j + K::EPW < nlive) fetch(j + K::EPW);
 
       if constexpr (WANT_GX) {
         if (active) stv(gXe + static_cast<int64_t>(base + sOrig[j]) * C + V * cl, gxe);
