@@ -107,6 +107,9 @@ def main():
     ap.add_argument("--channels", type=int, default=128)
     ap.add_argument("--elements", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-md-loop", action="store_true",
+                    help="skip the MD-like loop through the device calculator (keeps a kernel trace of this run to the "
+                         "timed steps and the isolated ops)")
     ap.add_argument("--tabulated-radial", action="store_true",
                     help="keep the reference's separate spline step (R[E,4,C] in HBM) instead of the fused kernels")
     ap.add_argument("--cpu-atoms", type=int, default=1500, help="size of the box the CPU baseline is timed on")
@@ -308,7 +311,7 @@ def main():
     calc = DeviceCalculator(model, data["node_attrs"], cutoff=5.0, skin=0.5, pbc=(True, True, True), cell=data["cell"])
     gen = torch.Generator(device="cuda").manual_seed(0)
     pos = data["positions"].detach().clone()
-    md_steps = 60
+    md_steps = 0 if args.no_md_loop else 60
 
     def md_step(p):
         d = torch.randn(p.shape, device="cuda", dtype=p.dtype, generator=gen)
@@ -316,7 +319,7 @@ def main():
         calc.compute(p)
         return p
 
-    for _ in range(5):
+    for _ in range(5 if md_steps else 0):
         pos = md_step(pos)
     builds0 = calc.builds
     torch.cuda.synchronize()
@@ -324,7 +327,8 @@ def main():
     for _ in range(md_steps):
         pos = md_step(pos)
     torch.cuda.synchronize()
-    md_loop = {"ms_per_step": round(1e3 * (time.perf_counter() - t_md) / md_steps, 4), "steps": md_steps,
+    md_loop = None if not md_steps else {
+               "ms_per_step": round(1e3 * (time.perf_counter() - t_md) / md_steps, 4), "steps": md_steps,
                "list_rebuilds": calc.builds - builds0, "skin_A": 0.5, "move_per_step_A": 0.02,
                "hip_graph": calc.use_graph,
                "note": "energy+forces through DeviceCalculator incl. neighbour-list rebuilds on the device; the list holds "
