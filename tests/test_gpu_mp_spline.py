@@ -18,6 +18,8 @@ CASES = [
     (30, 160, 128, 0.0, 4),
     (120, 40, 192, 0.1, 5),
     (60, 20, 256, 0.0, 6),
+    (70, 30, 160, 0.1, 7),   # 40 of 64 lanes carry channels
+    (50, 90, 224, 0.0, 8),   # 56 of 64 lanes; segments longer than one 64-edge chunk
 ]
 
 
