@@ -134,3 +134,50 @@ def test_batch_of_graphs(cabi):
         torch.testing.assert_close(batch["virials"][g], single["virials"][0], rtol=1e-5, atol=1e-5 * float(single["virials"].abs().max()))
         torch.testing.assert_close(batch["stress"][g], single["stress"][0], rtol=1e-5, atol=1e-5 * float(single["stress"].abs().max()))
         start += n
+
+
+def test_config3_full_size_against_reference(cabi):
+    """BASELINE config 3 at its real size (5 000 atoms, 96 channels, 10 elements): energy and forces against the fp64
+    reference evaluated in edge chunks."""
+    _say("model c3: 5000-atom periodic box, C=96")
+    data = make_system(5000, 10, seed=0, density=0.1)
+    params, model = _build(96, tuple(range(1, 11)), data, seed=0)
+    ref = M.energy_and_forces(params, data, edge_chunk=65536)
+    out = model(to_device(data, "cuda"))
+    e, e_ref = float(out["interaction_energy"].detach().cpu()), float(ref["interaction_energy"])
+    f_err = float((out["forces"].double().cpu() - ref["forces"]).abs().max())
+    _say("  E %.10g ref %.10g rel %.2e | max|dF| %.2e" % (e, e_ref, abs(e - e_ref) / abs(e_ref), f_err))
+    assert abs(e - e_ref) <= E_RTOL * abs(e_ref)
+    assert f_err <= F_ATOL
+
+
+def test_config4_full_size_properties(cabi):
+    """BASELINE config 4 at its real size (25 000 atoms, 128 channels), where the fp64 reference is out of reach: forces
+    sum to zero, two evaluations agree bit for bit, and rotating the whole periodic system (positions, cell, shifts)
+    leaves the energy unchanged and rotates the forces."""
+    _say("model c4: 25000-atom periodic box, C=128")
+    data = make_system(25000, 10, seed=0, density=0.1)
+    _, model = _build(128, tuple(range(1, 11)), data, seed=0)
+    dev = to_device(data, "cuda")
+    a = model(dict(dev))
+    b = model(dict(dev))
+    assert torch.equal(a["energy"], b["energy"]) and torch.equal(a["forces"], b["forces"])
+    fmax = float(a["forces"].abs().max())
+    assert float(a["forces"].sum(0).abs().max()) < 1e-4 * 25000 ** 0.5 * max(fmax, 1.0) * 1e-1
+
+    # a proper rotation from a QR decomposition
+    g = torch.Generator().manual_seed(3)
+    Q, _ = torch.linalg.qr(torch.randn(3, 3, generator=g, dtype=torch.float64))
+    if torch.det(Q) < 0:
+        Q[:, 0] = -Q[:, 0]
+    Q = Q.to("cuda")
+    rot = dict(dev)
+    rot["positions"] = dev["positions"].detach() @ Q
+    rot["cell"] = dev["cell"] @ Q
+    rot["shifts"] = dev["shifts"] @ Q
+    c = model(rot)
+    e0, e1 = float(a["interaction_energy"].detach()), float(c["interaction_energy"].detach())
+    _say("  E %.10g rotated %.10g rel %.2e" % (e0, e1, abs(e0 - e1) / abs(e0)))
+    assert abs(e0 - e1) <= 2e-6 * abs(e0)
+    f_rot = a["forces"].detach() @ Q
+    assert float((c["forces"].detach() - f_rot).abs().max()) <= 2e-5 * max(fmax, 1.0)
