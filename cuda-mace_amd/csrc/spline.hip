@@ -63,6 +63,57 @@ __global__ __launch_bounds__(256) void spline_backward_kernel(
   if (lane == 0) gr[e] = sum;
 }
 
+// fp64 variants (the reference dispatches the spline on float and double, jit_wrappers/src/cubic_spline_wrapper.cpp:50,
+// :123): one thread per output, same knot lookup and Horner forms as above.
+__device__ __forceinline__ int knot_index(double r, double r_width, int nknots) {
+  int idx = static_cast<int>(r / r_width);
+  return idx < 0 ? 0 : (idx > nknots - 2 ? nknots - 2 : idx);
+}
+
+template <bool DERIV>
+__global__ void spline_forward_f64_kernel(const double *__restrict__ r, const double *__restrict__ r_knots,
+                                          const double *__restrict__ coeffs, int64_t nedges, int nknots, int J,
+                                          double r_width, double r_max, double *__restrict__ R_out,
+                                          double *__restrict__ R_deriv) {
+  const int64_t t = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (t >= nedges * J) return;
+  const int64_t e = t / J;
+  const int j = static_cast<int>(t - e * J);
+  const double re = r[e];
+  double val = 0.0, der = 0.0;
+  if (re <= r_max) {
+    const int idx = knot_index(re, r_width, nknots);
+    const double x = re - r_knots[idx];
+    const double *cp = coeffs + static_cast<int64_t>(idx) * 4 * J + j;
+    const double a = cp[0], b = cp[J], c = cp[2 * J], d = cp[3 * J];
+    val = a + x * (b + x * (c + x * d));
+    if (DERIV) der = b + x * (2.0 * c + (3.0 * x) * d);
+  }
+  R_out[t] = val;
+  if (DERIV) R_deriv[t] = der;
+}
+
+__global__ __launch_bounds__(256) void spline_backward_f64_kernel(
+    const double *__restrict__ r, const double *__restrict__ r_knots, const double *__restrict__ coeffs,
+    const double *__restrict__ gR, int64_t nedges, int nknots, int J, double r_width, double r_max,
+    double *__restrict__ gr) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t e = blockIdx.x * static_cast<int64_t>(blockDim.x / kWave) + threadIdx.x / kWave;
+  if (e >= nedges) return;
+  const double re = r[e];
+  double sum = 0.0;
+  if (re <= r_max) {
+    const int idx = knot_index(re, r_width, nknots);
+    const double x = re - r_knots[idx];
+    const double *cp = coeffs + static_cast<int64_t>(idx) * 4 * J;
+    const double *gp = gR + e * J;
+    for (int j = lane; j < J; j += kWave) sum += gp[j] * (cp[J + j] + x * (2.0 * cp[2 * J + j] + (3.0 * x) * cp[3 * J + j]));
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  if (lane == 0) gr[e] = sum;
+}
+
 }  // namespace
 }  // namespace cm
 
@@ -102,4 +153,42 @@ extern "C" int cm_spline_backward(const float *r, const float *r_knots, const fl
   hipLaunchKernelGGL(cm::spline_backward_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nedges, per))), dim3(block), 0,
                      cm::as_stream(stream), r, r_knots, coeffs, grad_R, nedges, nknots, noutputs, r_width, r_max, grad_r);
   return cm::check_launch("cm_spline_backward");
+}
+
+extern "C" int cm_spline_forward_f64(const double *r, const double *r_knots, const double *coeffs, int64_t nedges,
+                                     int nknots, int noutputs, double r_width, double r_max, double *R_out,
+                                     double *R_deriv, cm_stream_t stream) {
+  CM_REQUIRE(nedges >= 0, "cm_spline_forward_f64: negative size");
+  CM_REQUIRE(nknots >= 2, "cm_spline_forward_f64: need at least two knots, got %d", nknots);
+  CM_REQUIRE(noutputs > 0, "cm_spline_forward_f64: noutputs=%d must be positive", noutputs);
+  CM_REQUIRE(r_width > 0.0, "cm_spline_forward_f64: r_width must be positive");
+  if (nedges == 0) return CM_OK;
+  CM_REQUIRE(r && r_knots && coeffs && R_out, "cm_spline_forward_f64: NULL pointer");
+  const int block = 256;
+  const int64_t threads = nedges * noutputs;
+  CM_REQUIRE(cm::ceil_div(threads, block) < INT32_MAX, "cm_spline_forward_f64: problem too large for one launch");
+  const dim3 grid(static_cast<unsigned>(cm::ceil_div(threads, block)));
+  if (R_deriv)
+    hipLaunchKernelGGL(cm::spline_forward_f64_kernel<true>, grid, dim3(block), 0, cm::as_stream(stream), r, r_knots, coeffs,
+                       nedges, nknots, noutputs, r_width, r_max, R_out, R_deriv);
+  else
+    hipLaunchKernelGGL(cm::spline_forward_f64_kernel<false>, grid, dim3(block), 0, cm::as_stream(stream), r, r_knots, coeffs,
+                       nedges, nknots, noutputs, r_width, r_max, R_out, R_deriv);
+  return cm::check_launch("cm_spline_forward_f64");
+}
+
+extern "C" int cm_spline_backward_f64(const double *r, const double *r_knots, const double *coeffs, const double *grad_R,
+                                      int64_t nedges, int nknots, int noutputs, double r_width, double r_max,
+                                      double *grad_r, cm_stream_t stream) {
+  CM_REQUIRE(nedges >= 0, "cm_spline_backward_f64: negative size");
+  CM_REQUIRE(nknots >= 2, "cm_spline_backward_f64: need at least two knots, got %d", nknots);
+  CM_REQUIRE(noutputs > 0, "cm_spline_backward_f64: noutputs=%d must be positive", noutputs);
+  CM_REQUIRE(r_width > 0.0, "cm_spline_backward_f64: r_width must be positive");
+  if (nedges == 0) return CM_OK;
+  CM_REQUIRE(r && r_knots && coeffs && grad_R && grad_r, "cm_spline_backward_f64: NULL pointer");
+  const int block = 256;
+  const int per = block / cm::kWave;
+  hipLaunchKernelGGL(cm::spline_backward_f64_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nedges, per))), dim3(block), 0,
+                     cm::as_stream(stream), r, r_knots, coeffs, grad_R, nedges, nknots, noutputs, r_width, r_max, grad_r);
+  return cm::check_launch("cm_spline_backward_f64");
 }

@@ -19,6 +19,7 @@
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <type_traits>
 #include <vector>
 
 #include "cuda_mace_hip.h"
@@ -40,6 +41,37 @@ void need(const Tensor &t, c10::ScalarType dtype, const char *name) {
 }
 
 const float *fptr(const Tensor &t) { return t.numel() ? t.data_ptr<float>() : nullptr; }
+template <typename T>
+T *ptr(const Tensor &t) {
+  return t.defined() && t.numel() ? t.data_ptr<T>() : nullptr;
+}
+
+// Message passing, harmonics, spline and contraction take float or double tensors, as the reference's
+// AT_DISPATCH_FLOATING_TYPES does (jit_wrappers/src/invariant_message_passing_wrapper.cpp:102 and siblings); the
+// linears are float only (linear_wrapper.cpp:67).
+c10::ScalarType float_type_of(const Tensor &t, const char *name) {
+  TORCH_CHECK(t.scalar_type() == torch::kFloat32 || t.scalar_type() == torch::kFloat64, name,
+              " must be float32 or float64 (got ", t.scalar_type(), ")");
+  return t.scalar_type();
+}
+
+// Calls f with a value of the scalar type that dt names.
+template <typename F>
+void by_dtype(c10::ScalarType dt, F &&f) {
+  if (dt == torch::kFloat64)
+    f(double{});
+  else
+    f(float{});
+}
+
+// The fp32 or the fp64 entry point of a pair, by scalar type.
+template <typename T, typename A, typename B>
+auto pick(A f32, B f64) {
+  if constexpr (std::is_same_v<T, double>)
+    return f64;
+  else
+    return f32;
+}
 const int32_t *iptr(const Tensor &t) { return t.numel() ? t.data_ptr<int32_t>() : nullptr; }
 
 // ---- cache of derived tensors -------------------------------------------------------------------------------
@@ -146,7 +178,8 @@ class InvariantMessagePassingTPAutograd : public torch::autograd::Function<Invar
                         int64_t nnodes) {
     X = X.contiguous(), Y = Y.contiguous();
     Tensor R = radial.contiguous();
-    need(X, torch::kFloat32, "X"), need(Y, torch::kFloat32, "Y"), need(R, torch::kFloat32, "radial");
+    const auto dt = float_type_of(X, "X");
+    need(X, dt, "X"), need(Y, dt, "Y"), need(R, dt, "radial");
     need(sender_list, torch::kInt32, "sender_list"), need(receiver_list, torch::kInt32, "receiver_list");
     TORCH_CHECK(X.dim() == 2 && X.size(0) == nnodes, "X must be [nnodes, channels]");
     const int64_t E = sender_list.numel(), C = X.size(1);
@@ -154,8 +187,11 @@ class InvariantMessagePassingTPAutograd : public torch::autograd::Function<Invar
     TORCH_CHECK(R.numel() == E * 4 * C, "radial must hold nedges * 4 * channels values");
     Tensor first_occ = csr_of(receiver_list, nnodes);
     Tensor out = torch::empty({nnodes, 16, C}, X.options());
-    CM_CALL(cm_mp_forward(fptr(X), fptr(Y), fptr(R), iptr(sender_list), iptr(first_occ), nnodes, E, static_cast<int>(C),
-                          out.data_ptr<float>(), stream_of(X)));
+    by_dtype(dt, [&](auto tag) {
+      using T = decltype(tag);
+      CM_CALL(pick<T>(cm_mp_forward, cm_mp_forward_f64)(ptr<T>(X), ptr<T>(Y), ptr<T>(R), iptr(sender_list), iptr(first_occ),
+                                                        nnodes, E, static_cast<int>(C), ptr<T>(out), stream_of(X)));
+    });
     if (X.requires_grad() || Y.requires_grad() || radial.requires_grad()) {
       ctx->saved_data["nnodes"] = nnodes;
       ctx->saved_data["radial_sizes"] = radial.sizes().vec();
@@ -171,6 +207,7 @@ class InvariantMessagePassingTPAutograd : public torch::autograd::Function<Invar
     const int64_t E = sender.numel(), C = X.size(1);
     const bool need_x = ctx->needs_input_grad(0), need_y = ctx->needs_input_grad(1), need_r = ctx->needs_input_grad(2);
     Tensor g = grad_outputs[0].contiguous();
+    need(g, X.scalar_type(), "grad_output");
     Tensor gX, gY, gR, scratch, perm, off;
     if (need_x) {
       auto view = sorted_view_of(sender, nnodes);
@@ -180,10 +217,13 @@ class InvariantMessagePassingTPAutograd : public torch::autograd::Function<Invar
     }
     if (need_y) gY = torch::empty({16, E}, X.options());
     if (need_r) gR = torch::empty(ctx->saved_data["radial_sizes"].toIntVector(), X.options());
-    CM_CALL(cm_mp_backward(fptr(X), fptr(Y), fptr(R), fptr(g), iptr(sender), iptr(first_occ), need_x ? iptr(perm) : nullptr,
-                           need_x ? iptr(off) : nullptr, nnodes, E, static_cast<int>(C), need_x ? gX.data_ptr<float>() : nullptr,
-                           need_y && E ? gY.data_ptr<float>() : nullptr, need_r && E ? gR.data_ptr<float>() : nullptr,
-                           need_x && E ? scratch.data_ptr<float>() : nullptr, stream_of(X)));
+    by_dtype(X.scalar_type(), [&](auto tag) {
+      using T = decltype(tag);
+      CM_CALL(pick<T>(cm_mp_backward, cm_mp_backward_f64)(
+          ptr<T>(X), ptr<T>(Y), ptr<T>(R), ptr<T>(g), iptr(sender), iptr(first_occ), need_x ? iptr(perm) : nullptr,
+          need_x ? iptr(off) : nullptr, nnodes, E, static_cast<int>(C), ptr<T>(gX), ptr<T>(gY), ptr<T>(gR), ptr<T>(scratch),
+          stream_of(X)));
+    });
     return {gX, gY, gR, Tensor(), Tensor(), Tensor()};
   }
 };
@@ -193,18 +233,26 @@ class SphericalHarmonicsAutograd : public torch::autograd::Function<SphericalHar
  public:
   static Tensor forward(AutogradContext *ctx, Tensor xyz) {
     xyz = xyz.contiguous();
-    need(xyz, torch::kFloat32, "xyz");
+    const auto dt = float_type_of(xyz, "xyz");
+    need(xyz, dt, "xyz");
     TORCH_CHECK(xyz.dim() == 2 && xyz.size(1) == 3, "xyz must be [nedges, 3]");
     Tensor Y = torch::empty({16, xyz.size(0)}, xyz.options());
-    CM_CALL(cm_sh_forward(fptr(xyz), xyz.size(0), xyz.size(0) ? Y.data_ptr<float>() : nullptr, stream_of(xyz)));
+    by_dtype(dt, [&](auto tag) {
+      using T = decltype(tag);
+      CM_CALL(pick<T>(cm_sh_forward, cm_sh_forward_f64)(ptr<T>(xyz), xyz.size(0), ptr<T>(Y), stream_of(xyz)));
+    });
     if (xyz.requires_grad()) ctx->save_for_backward({xyz});
     return Y;
   }
   static variable_list backward(AutogradContext *ctx, variable_list grad_outputs) {
     const Tensor xyz = ctx->get_saved_variables()[0];
     Tensor g = grad_outputs[0].contiguous();
+    need(g, xyz.scalar_type(), "grad_output");
     Tensor out = torch::empty_like(xyz);
-    CM_CALL(cm_sh_backward(fptr(xyz), fptr(g), xyz.size(0), xyz.size(0) ? out.data_ptr<float>() : nullptr, stream_of(xyz)));
+    by_dtype(xyz.scalar_type(), [&](auto tag) {
+      using T = decltype(tag);
+      CM_CALL(pick<T>(cm_sh_backward, cm_sh_backward_f64)(ptr<T>(xyz), ptr<T>(g), xyz.size(0), ptr<T>(out), stream_of(xyz)));
+    });
     return {out};
   }
 };
@@ -214,14 +262,19 @@ class CubicSplineAutograd : public torch::autograd::Function<CubicSplineAutograd
  public:
   static Tensor forward(AutogradContext *ctx, Tensor r, Tensor r_knots, Tensor coeffs, double r_width, double r_max) {
     Tensor rc = r.contiguous().view({-1});
-    need(rc, torch::kFloat32, "r"), need(r_knots, torch::kFloat32, "r_knots"), need(coeffs, torch::kFloat32, "coeffs");
+    const auto dt = float_type_of(rc, "r");
+    need(rc, dt, "r"), need(r_knots, dt, "r_knots"), need(coeffs, dt, "coeffs");
     TORCH_CHECK(coeffs.dim() == 3 && coeffs.size(0) == r_knots.numel() - 1 && coeffs.size(1) == 4,
                 "coeffs must be [nknots - 1, 4, noutputs]");
     const int64_t E = rc.numel(), J = coeffs.size(2);
     Tensor R = torch::empty({E, J}, rc.options());
-    CM_CALL(cm_spline_forward(fptr(rc), fptr(r_knots), fptr(coeffs), E, static_cast<int>(r_knots.numel()), static_cast<int>(J),
-                              static_cast<float>(r_width), static_cast<float>(r_max), E ? R.data_ptr<float>() : nullptr, nullptr,
-                              stream_of(rc)));
+    // the reference hands r_width and r_max to its kernels as float in both precisions (cuda/src/cubic_spline_impl.cu:9-10)
+    by_dtype(dt, [&](auto tag) {
+      using T = decltype(tag);
+      CM_CALL(pick<T>(cm_spline_forward, cm_spline_forward_f64)(
+          ptr<T>(rc), ptr<T>(r_knots), ptr<T>(coeffs), E, static_cast<int>(r_knots.numel()), static_cast<int>(J),
+          static_cast<float>(r_width), static_cast<float>(r_max), ptr<T>(R), static_cast<T *>(nullptr), stream_of(rc)));
+    });
     if (r.requires_grad()) {
       ctx->saved_data["r_width"] = r_width;
       ctx->saved_data["r_max"] = r_max;
@@ -234,11 +287,15 @@ class CubicSplineAutograd : public torch::autograd::Function<CubicSplineAutograd
     auto saved = ctx->get_saved_variables();
     const Tensor &r = saved[0], &knots = saved[1], &coeffs = saved[2];
     Tensor g = grad_outputs[0].contiguous();
+    need(g, r.scalar_type(), "grad_output");
     Tensor out = torch::empty({r.numel()}, r.options());
-    CM_CALL(cm_spline_backward(fptr(r), fptr(knots), fptr(coeffs), fptr(g), r.numel(), static_cast<int>(knots.numel()),
-                               static_cast<int>(coeffs.size(2)), static_cast<float>(ctx->saved_data["r_width"].toDouble()),
-                               static_cast<float>(ctx->saved_data["r_max"].toDouble()), r.numel() ? out.data_ptr<float>() : nullptr,
-                               stream_of(r)));
+    by_dtype(r.scalar_type(), [&](auto tag) {
+      using T = decltype(tag);
+      CM_CALL(pick<T>(cm_spline_backward, cm_spline_backward_f64)(
+          ptr<T>(r), ptr<T>(knots), ptr<T>(coeffs), ptr<T>(g), r.numel(), static_cast<int>(knots.numel()),
+          static_cast<int>(coeffs.size(2)), static_cast<float>(ctx->saved_data["r_width"].toDouble()),
+          static_cast<float>(ctx->saved_data["r_max"].toDouble()), ptr<T>(out), stream_of(r)));
+    });
     return {out.view(ctx->saved_data["r_sizes"].toIntVector()), Tensor(), Tensor(), Tensor(), Tensor()};
   }
 };
@@ -308,7 +365,7 @@ class ElementalLinearAutograd : public torch::autograd::Function<ElementalLinear
 // ---- symmetric contraction ---------------------------------------------------------------------------------------------
 // Host pass over the packed sparse coupling tables (format of ops/symmetric_contraction.py:91-187): groups the entries
 // (i, j, k, path, value) by the sorted index triple they multiply.  Returns device tensors
-// {mono3, off3, path3, val3, mono2, off2, path2, val2} and whether the structure is the one compiled into the library.
+// {mono3, off3, path3, val3, mono2, off2, path2, val2, val3 (fp64), val2 (fp64)} and whether the structure is the one compiled into the library.
 struct Monomials {
   std::vector<Tensor> dev;
   bool builtin;
@@ -316,7 +373,7 @@ struct Monomials {
 
 template <size_t D>
 void pack_terms(const std::map<std::array<int, D>, std::map<int, double>> &terms, std::vector<int32_t> &mono,
-                std::vector<int32_t> &off, std::vector<int32_t> &path, std::vector<float> &val) {
+                std::vector<int32_t> &off, std::vector<int32_t> &path, std::vector<double> &val) {
   off.push_back(0);
   for (const auto &kv : terms) {
     int32_t word = 0;
@@ -324,7 +381,7 @@ void pack_terms(const std::map<std::array<int, D>, std::map<int, double>> &terms
     mono.push_back(word);
     for (const auto &pv : kv.second) {
       path.push_back(pv.first);
-      val.push_back(static_cast<float>(pv.second));
+      val.push_back(pv.second);
     }
     off.push_back(static_cast<int32_t>(path.size()));
   }
@@ -355,7 +412,7 @@ Monomials monomials_of(const Tensor &U3_num, const Tensor &U3_idx, const Tensor 
         }
       }
     std::vector<int32_t> m3, o3, p3, m2, o2, p2;
-    std::vector<float> w3, w2;
+    std::vector<double> w3, w2;
     pack_terms<3>(t3, m3, o3, p3, w3);
     pack_terms<2>(t2, m2, o2, p2, w2);
     int b3n = 0, b2n = 0;
@@ -364,12 +421,16 @@ Monomials monomials_of(const Tensor &U3_num, const Tensor &U3_idx, const Tensor 
     cm_symcon_builtin_structure(b3.data(), b3n, b2.data(), b2n, nullptr, nullptr);
     const bool builtin = b3 == m3 && b2 == m2;
     auto dev_i = [&](const std::vector<int32_t> &v) { return torch::tensor(v, torch::kInt32).to(U3_idx.device()); };
-    auto dev_f = [&](const std::vector<float> &v) { return torch::tensor(v, torch::kFloat32).to(U3_idx.device()); };
-    return std::vector<Tensor>{dev_i(m3), dev_i(o3), dev_i(p3), dev_f(w3), dev_i(m2), dev_i(o2), dev_i(p2), dev_f(w2),
+    auto dev_f = [&](const std::vector<double> &v, c10::ScalarType dt) {
+      return torch::tensor(v, torch::kFloat64).to(U3_idx.device(), dt);
+    };
+    // values in both precisions: [3] / [7] fp32, [8] / [9] fp64
+    return std::vector<Tensor>{dev_i(m3), dev_i(o3), dev_i(p3), dev_f(w3, torch::kFloat32), dev_i(m2), dev_i(o2), dev_i(p2),
+                               dev_f(w2, torch::kFloat32), dev_f(w3, torch::kFloat64), dev_f(w2, torch::kFloat64),
                                torch::tensor({builtin ? 1 : 0}, torch::kInt32)};
   });
   Monomials m;
-  m.builtin = got[8].item<int>() != 0;
+  m.builtin = got.back().item<int>() != 0;
   got.pop_back();
   m.dev = got;
   return m;
@@ -382,8 +443,10 @@ class SymmetricContractionAutograd : public torch::autograd::Function<SymmetricC
                         Tensor U1_num_nonzero, Tensor U1_index, Tensor W3, Tensor W2, Tensor W1, int64_t W3_size, int64_t W2_size,
                         int64_t W1_size) {
     X = X.contiguous();
-    need(X, torch::kFloat32, "X"), need(atom_types, torch::kInt32, "atom_types");
-    need(W3, torch::kFloat32, "W3"), need(W2, torch::kFloat32, "W2"), need(W1, torch::kFloat32, "W1");
+    const auto dt = float_type_of(X, "X");
+    need(X, dt, "X"), need(atom_types, torch::kInt32, "atom_types");
+    need(W3, dt, "W3"), need(W2, dt, "W2"), need(W1, dt, "W1");
+    const bool f64 = dt == torch::kFloat64;
     TORCH_CHECK(X.dim() == 3 && X.size(1) == 16 && X.size(2) % 32 == 0, "X must be [nnodes, 16, C] with C % 32 == 0");
     const int64_t N = X.size(0), C = X.size(2);
     Monomials mono = monomials_of(U3_num_nonzero, U3_indices, U3_values, U2_num_nonzero, U2_indices, U2_values);
@@ -400,10 +463,13 @@ class SymmetricContractionAutograd : public torch::autograd::Function<SymmetricC
       Tensor w3 = W3.reshape({ne, W3.size(-2), C}).narrow(1, 0, W3_size).contiguous();
       Tensor w2 = W2.reshape({ne, W2.size(-2), C}).narrow(1, 0, W2_size).contiguous();
       Tensor w1 = W1.reshape({ne, W1.size(-2), C}).narrow(1, 0, W1_size).contiguous();
-      CM_CALL(cm_symcon_tables(iptr(d[1]), iptr(d[2]), fptr(d[3]), n3, iptr(d[5]), iptr(d[6]), fptr(d[7]), n2, fptr(w3), fptr(w2),
-                               fptr(w1), static_cast<int>(ne), static_cast<int>(W3_size), static_cast<int>(W2_size),
-                               static_cast<int>(W1_size), static_cast<int>(C), n3 ? T3.data_ptr<float>() : nullptr,
-                               n2 ? T2.data_ptr<float>() : nullptr, T1.data_ptr<float>(), stream_of(X)));
+      by_dtype(dt, [&](auto tag) {
+        using T = decltype(tag);
+        CM_CALL(pick<T>(cm_symcon_tables, cm_symcon_tables_f64)(
+            iptr(d[1]), iptr(d[2]), ptr<T>(d[f64 ? 8 : 3]), n3, iptr(d[5]), iptr(d[6]), ptr<T>(d[f64 ? 9 : 7]), n2, ptr<T>(w3),
+            ptr<T>(w2), ptr<T>(w1), static_cast<int>(ne), static_cast<int>(W3_size), static_cast<int>(W2_size),
+            static_cast<int>(W1_size), static_cast<int>(C), ptr<T>(T3), ptr<T>(T2), ptr<T>(T1), stream_of(X)));
+      });
       return std::vector<Tensor>{T3, T2, T1};
     });
 
@@ -412,10 +478,13 @@ class SymmetricContractionAutograd : public torch::autograd::Function<SymmetricC
     const bool want_grad = X.requires_grad();
     Tensor out = torch::empty({N, C}, X.options());
     Tensor grad = want_grad ? torch::empty({N, 16, C}, X.options()) : Tensor();
-    CM_CALL(cm_symcon_forward(fptr(X), iptr(groups[0]), iptr(groups[1]), mono.builtin ? nullptr : iptr(d[0]), n3,
-                              mono.builtin ? nullptr : iptr(d[4]), n2, fptr(tables[0]), fptr(tables[1]), fptr(tables[2]), N,
-                              static_cast<int>(ne), static_cast<int>(C), N ? out.data_ptr<float>() : nullptr,
-                              want_grad && N ? grad.data_ptr<float>() : nullptr, stream_of(X)));
+    by_dtype(dt, [&](auto tag) {
+      using T = decltype(tag);
+      CM_CALL(pick<T>(cm_symcon_forward, cm_symcon_forward_f64)(
+          ptr<T>(X), iptr(groups[0]), iptr(groups[1]), mono.builtin ? nullptr : iptr(d[0]), n3,
+          mono.builtin ? nullptr : iptr(d[4]), n2, ptr<T>(tables[0]), ptr<T>(tables[1]), ptr<T>(tables[2]), N,
+          static_cast<int>(ne), static_cast<int>(C), ptr<T>(out), ptr<T>(grad), stream_of(X)));
+    });
     if (want_grad) ctx->save_for_backward({grad});
     return out.view({N, 1, C});
   }
@@ -424,8 +493,13 @@ class SymmetricContractionAutograd : public torch::autograd::Function<SymmetricC
     const Tensor grad = ctx->get_saved_variables()[0];
     const int64_t N = grad.size(0), C = grad.size(2);
     Tensor g = grad_outputs[0].contiguous().view({N, C});
+    need(g, grad.scalar_type(), "grad_output");
     Tensor gX = torch::empty_like(grad);
-    CM_CALL(cm_symcon_backward(fptr(grad), fptr(g), N, static_cast<int>(C), N ? gX.data_ptr<float>() : nullptr, stream_of(grad)));
+    by_dtype(grad.scalar_type(), [&](auto tag) {
+      using T = decltype(tag);
+      CM_CALL(pick<T>(cm_symcon_backward, cm_symcon_backward_f64)(ptr<T>(grad), ptr<T>(g), N, static_cast<int>(C), ptr<T>(gX),
+                                                                  stream_of(grad)));
+    });
     variable_list out(17);
     out[0] = gX;
     return out;

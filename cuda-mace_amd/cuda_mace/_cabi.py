@@ -59,6 +59,16 @@ SIGNATURES = {
     "cm_neighbour_list_workspace": (_sz, [_i64, _i64]),
     "cm_neighbour_list_count": (_i32, [_p, _p, _i32, _i32, _i32, _f64, _i64, _i64, _p, _sz, _p, _p, _p]),
     "cm_neighbour_list_fill": (_i32, [_p, _f64, _i64, _i64, _p, _p, _i64, _p, _p, _p, _p, _p]),
+    # fp64 instantiations: same argument lists, floating-point buffers in double
+    "cm_mp_forward_f64": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _p, _p]),
+    "cm_mp_backward_f64": (_i32, [_p] * 8 + [_i64, _i64, _i32] + [_p] * 5),
+    "cm_sh_forward_f64": (_i32, [_p, _i64, _p, _p]),
+    "cm_sh_backward_f64": (_i32, [_p, _p, _i64, _p, _p]),
+    "cm_spline_forward_f64": (_i32, [_p, _p, _p, _i64, _i32, _i32, _f64, _f64, _p, _p, _p]),
+    "cm_spline_backward_f64": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _f64, _f64, _p, _p]),
+    "cm_symcon_tables_f64": (_i32, [_p, _p, _p, _i32, _p, _p, _p, _i32, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _p, _p, _p]),
+    "cm_symcon_forward_f64": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
+    "cm_symcon_backward_f64": (_i32, [_p, _p, _i64, _i32, _p, _p]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():
@@ -93,7 +103,15 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
-F32, I32 = torch.float32, torch.int32
+F32, F64, I32 = torch.float32, torch.float64, torch.int32
+
+
+def _typed(name: str, like: torch.Tensor):
+    """(entry point, dtype) for the precision of `like`: `name` for fp32 tensors, `name`_f64 for fp64 ones (message
+    passing, harmonics, spline and contraction exist in both, as in the reference)."""
+    if like.dtype == F64:
+        return getattr(lib, name + "_f64"), F64
+    return getattr(lib, name), F32
 
 
 # ---- index kernels ---------------------------------------------------------------------------
@@ -120,6 +138,7 @@ def stable_key_sort(keys: torch.Tensor, nkeys: int):
 
 # ---- message passing --------------------------------------------------------------------------
 def mp_forward(X, Y, R, sender, first_occ, nnodes: int) -> torch.Tensor:
+    fn, D = _typed("cm_mp_forward", X)
     C = X.shape[-1]
     E = sender.numel()
     if Y.shape != (16, E):
@@ -128,11 +147,11 @@ def mp_forward(X, Y, R, sender, first_occ, nnodes: int) -> torch.Tensor:
         raise CudaMaceError("radial must hold nedges*4*channels = %d values, got %d" % (E * 4 * C, R.numel()))
     if X.shape[0] != nnodes:
         raise CudaMaceError("X must be [nnodes, channels]")
-    out = torch.empty(nnodes, 16, C, dtype=F32, device=X.device)
+    out = torch.empty(nnodes, 16, C, dtype=D, device=X.device)
     _check(
-        lib.cm_mp_forward(
-            _dev(X, F32, "X"), _dev(Y, F32, "Y"), _dev(R, F32, "radial"), _dev(sender, I32, "sender_list"),
-            _dev(first_occ, I32, "first_occurences"), nnodes, E, C, _dev(out, F32, "out"), _stream(),
+        fn(
+            _dev(X, D, "X"), _dev(Y, D, "Y"), _dev(R, D, "radial"), _dev(sender, I32, "sender_list"),
+            _dev(first_occ, I32, "first_occurences"), nnodes, E, C, _dev(out, D, "out"), _stream(),
         )
     )
     return out
@@ -140,20 +159,21 @@ def mp_forward(X, Y, R, sender, first_occ, nnodes: int) -> torch.Tensor:
 
 def mp_backward(X, Y, R, grad_out, sender, first_occ, sender_perm, sender_offsets, nnodes: int,
                 need_gX: bool = True, need_gY: bool = True, need_gR: bool = True):
+    fn, D = _typed("cm_mp_backward", X)
     C = X.shape[-1]
     E = sender.numel()
     dev = X.device
-    gX = torch.empty(nnodes, C, dtype=F32, device=dev) if need_gX else None
-    gY = torch.empty(16, E, dtype=F32, device=dev) if need_gY else None
-    gR = torch.empty(E, 4, C, dtype=F32, device=dev) if need_gR else None
-    scratch = torch.empty(E, C, dtype=F32, device=dev) if need_gX else None
+    gX = torch.empty(nnodes, C, dtype=D, device=dev) if need_gX else None
+    gY = torch.empty(16, E, dtype=D, device=dev) if need_gY else None
+    gR = torch.empty(E, 4, C, dtype=D, device=dev) if need_gR else None
+    scratch = torch.empty(E, C, dtype=D, device=dev) if need_gX else None
     _check(
-        lib.cm_mp_backward(
-            _dev(X, F32, "X"), _dev(Y, F32, "Y"), _dev(R, F32, "radial"), _dev(grad_out, F32, "grad_out"),
+        fn(
+            _dev(X, D, "X"), _dev(Y, D, "Y"), _dev(R, D, "radial"), _dev(grad_out, D, "grad_out"),
             _dev(sender, I32, "sender_list"), _dev(first_occ, I32, "first_occurences"),
             _dev(sender_perm, I32, "sender_perm") if need_gX else None,
             _dev(sender_offsets, I32, "sender_offsets") if need_gX else None,
-            nnodes, E, C, _dev(gX, F32, "gX"), _dev(gY, F32, "gY"), _dev(gR, F32, "gR"), _dev(scratch, F32, "scratch"), _stream(),
+            nnodes, E, C, _dev(gX, D, "gX"), _dev(gY, D, "gY"), _dev(gR, D, "gR"), _dev(scratch, D, "scratch"), _stream(),
         )
     )
     return gX, gY, gR
@@ -238,21 +258,22 @@ def mp_edge_backward(X, vectors, r_knots, coeffs, r_width: float, r_max: float, 
 
 # ---- spherical harmonics ------------------------------------------------------------------------
 def sh_forward(xyz: torch.Tensor) -> torch.Tensor:
+    fn, D = _typed("cm_sh_forward", xyz)
     E = xyz.shape[0]
-    Y = torch.empty(16, E, dtype=F32, device=xyz.device)
-    _check(lib.cm_sh_forward(_dev(xyz, F32, "xyz"), E, _dev(Y, F32, "Y"), _stream()))
+    Y = torch.empty(16, E, dtype=D, device=xyz.device)
+    _check(fn(_dev(xyz, D, "xyz"), E, _dev(Y, D, "Y"), _stream()))
     return Y
 
 
 def sh_backward(xyz: torch.Tensor, grad_Y: torch.Tensor) -> torch.Tensor:
+    fn, D = _typed("cm_sh_backward", xyz)
     E = xyz.shape[0]
-    g = torch.empty(E, 3, dtype=F32, device=xyz.device)
-    _check(lib.cm_sh_backward(_dev(xyz, F32, "xyz"), _dev(grad_Y, F32, "grad_Y"), E, _dev(g, F32, "grad_xyz"), _stream()))
+    g = torch.empty(E, 3, dtype=D, device=xyz.device)
+    _check(fn(_dev(xyz, D, "xyz"), _dev(grad_Y, D, "grad_Y"), E, _dev(g, D, "grad_xyz"), _stream()))
     return g
 
 
 # ---- edge geometry ------------------------------------------------------------------------------
-F64 = torch.float64
 
 
 def edge_geometry_forward(positions, row_a, row_b, shifts):
@@ -290,30 +311,32 @@ def edge_geometry_backward(positions, row_a, row_b, shifts, a_first_occ, b_perm,
 
 # ---- cubic spline ---------------------------------------------------------------------------------
 def spline_forward(r, r_knots, coeffs, r_width: float, r_max: float, want_deriv: bool = False):
+    fn, D = _typed("cm_spline_forward", r)
     E = r.numel()
     J = coeffs.shape[-1]
     nknots = r_knots.numel()
     if coeffs.shape[0] != nknots - 1 or coeffs.shape[1] != 4:
         raise CudaMaceError("coeffs must be [nknots-1, 4, noutputs]")
-    R = torch.empty(E, J, dtype=F32, device=r.device)
-    dR = torch.empty(E, J, dtype=F32, device=r.device) if want_deriv else None
+    R = torch.empty(E, J, dtype=D, device=r.device)
+    dR = torch.empty(E, J, dtype=D, device=r.device) if want_deriv else None
     _check(
-        lib.cm_spline_forward(
-            _dev(r, F32, "r"), _dev(r_knots, F32, "r_knots"), _dev(coeffs, F32, "coeffs"), E, nknots, J,
-            float(r_width), float(r_max), _dev(R, F32, "R_out"), _dev(dR, F32, "R_deriv"), _stream(),
+        fn(
+            _dev(r, D, "r"), _dev(r_knots, D, "r_knots"), _dev(coeffs, D, "coeffs"), E, nknots, J,
+            float(r_width), float(r_max), _dev(R, D, "R_out"), _dev(dR, D, "R_deriv"), _stream(),
         )
     )
     return (R, dR) if want_deriv else R
 
 
 def spline_backward(r, r_knots, coeffs, grad_R, r_width: float, r_max: float) -> torch.Tensor:
+    fn, D = _typed("cm_spline_backward", r)
     E = r.numel()
     J = coeffs.shape[-1]
-    out = torch.empty(E, dtype=F32, device=r.device)
+    out = torch.empty(E, dtype=D, device=r.device)
     _check(
-        lib.cm_spline_backward(
-            _dev(r, F32, "r"), _dev(r_knots, F32, "r_knots"), _dev(coeffs, F32, "coeffs"), _dev(grad_R, F32, "grad_R"),
-            E, r_knots.numel(), J, float(r_width), float(r_max), _dev(out, F32, "grad_r"), _stream(),
+        fn(
+            _dev(r, D, "r"), _dev(r_knots, D, "r_knots"), _dev(coeffs, D, "coeffs"), _dev(grad_R, D, "grad_R"),
+            E, r_knots.numel(), J, float(r_width), float(r_max), _dev(out, D, "grad_r"), _stream(),
         )
     )
     return out
@@ -358,21 +381,22 @@ def linear(X, W_T, node_perm=None, group_offsets=None, scale=None, zero_last_gro
 
 # ---- symmetric contraction -----------------------------------------------------------------------------
 def symcon_tables(term3_off, term3_path, term3_val, term2_off, term2_path, term2_val, W3, W2, W1):
+    fn, D = _typed("cm_symcon_tables", W3)
     ne, P3, C = W3.shape
     P2 = W2.shape[1]
     P1 = W1.shape[1]
     n3 = term3_off.numel() - 1
     n2 = term2_off.numel() - 1
     dev = W3.device
-    T3 = torch.empty(ne, n3, C, dtype=F32, device=dev)
-    T2 = torch.empty(ne, n2, C, dtype=F32, device=dev)
-    T1 = torch.empty(ne, C, dtype=F32, device=dev)
+    T3 = torch.empty(ne, n3, C, dtype=D, device=dev)
+    T2 = torch.empty(ne, n2, C, dtype=D, device=dev)
+    T1 = torch.empty(ne, C, dtype=D, device=dev)
     _check(
-        lib.cm_symcon_tables(
-            _dev(term3_off, I32, "term3_off"), _dev(term3_path, I32, "term3_path"), _dev(term3_val, F32, "term3_val"), n3,
-            _dev(term2_off, I32, "term2_off"), _dev(term2_path, I32, "term2_path"), _dev(term2_val, F32, "term2_val"), n2,
-            _dev(W3, F32, "W3"), _dev(W2, F32, "W2"), _dev(W1, F32, "W1"), ne, P3, P2, P1, C,
-            _dev(T3, F32, "T3"), _dev(T2, F32, "T2"), _dev(T1, F32, "T1"), _stream(),
+        fn(
+            _dev(term3_off, I32, "term3_off"), _dev(term3_path, I32, "term3_path"), _dev(term3_val, D, "term3_val"), n3,
+            _dev(term2_off, I32, "term2_off"), _dev(term2_path, I32, "term2_path"), _dev(term2_val, D, "term2_val"), n2,
+            _dev(W3, D, "W3"), _dev(W2, D, "W2"), _dev(W1, D, "W1"), ne, P3, P2, P1, C,
+            _dev(T3, D, "T3"), _dev(T2, D, "T2"), _dev(T1, D, "T1"), _stream(),
         )
     )
     return T3, T2, T1
@@ -395,29 +419,31 @@ def symcon_forward(X, node_perm, group_offsets, mono3, mono2, T3, T2, T1, want_g
     """builtin=True: the monomial lists are the ones compiled into the library; the unrolled kernel is used.
     zero_init=False skips clearing the outputs: rows of nodes that are in no group are then undefined (every node is in
     a group when all element indices are in range)."""
+    fn, D = _typed("cm_symcon_forward", X)
     N, sixteen, C = X.shape
     if sixteen != 16:
         raise CudaMaceError("symmetric contraction: X must be [N,16,C]")
     ne = T1.shape[0]
     alloc = torch.zeros if zero_init else torch.empty
-    out = alloc(N, C, dtype=F32, device=X.device)
-    grad = alloc(N, 16, C, dtype=F32, device=X.device) if want_grad else None
+    out = alloc(N, C, dtype=D, device=X.device)
+    grad = alloc(N, 16, C, dtype=D, device=X.device) if want_grad else None
     _check(
-        lib.cm_symcon_forward(
-            _dev(X, F32, "X"), _dev(node_perm, I32, "node_perm"), _dev(group_offsets, I32, "group_offsets"),
+        fn(
+            _dev(X, D, "X"), _dev(node_perm, I32, "node_perm"), _dev(group_offsets, I32, "group_offsets"),
             None if builtin else _dev(mono3, I32, "mono3"), mono3.numel(),
             None if builtin else _dev(mono2, I32, "mono2"), mono2.numel(),
-            _dev(T3, F32, "T3"), _dev(T2, F32, "T2"), _dev(T1, F32, "T1"), N, ne, C,
-            _dev(out, F32, "out"), _dev(grad, F32, "grad"), _stream(),
+            _dev(T3, D, "T3"), _dev(T2, D, "T2"), _dev(T1, D, "T1"), N, ne, C,
+            _dev(out, D, "out"), _dev(grad, D, "grad"), _stream(),
         )
     )
     return out, grad
 
 
 def symcon_backward(grad, grad_out) -> torch.Tensor:
+    fn, D = _typed("cm_symcon_backward", grad)
     N, _, C = grad.shape
     gX = torch.empty_like(grad)
-    _check(lib.cm_symcon_backward(_dev(grad, F32, "grad"), _dev(grad_out, F32, "grad_out"), N, C, _dev(gX, F32, "gX"), _stream()))
+    _check(fn(_dev(grad, D, "grad"), _dev(grad_out, D, "grad_out"), N, C, _dev(gX, D, "gX"), _stream()))
     return gX
 
 

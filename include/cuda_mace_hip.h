@@ -258,6 +258,43 @@ int cm_symcon_backward(const float *grad, const float *grad_out, int64_t nnodes,
                        float *gX, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * fp64 variants.  The reference dispatches message passing, spherical harmonics, the cubic spline and the symmetric
+ * contraction on float and double (AT_DISPATCH_FLOATING_TYPES at
+ * jit_wrappers/src/invariant_message_passing_wrapper.cpp:102 and :189, spherical_harmonics_wrapper.cpp:36 and :105,
+ * cubic_spline_wrapper.cpp:50 and :123, symmetric_contraction_wrapper.cpp:68); its linears are float only
+ * (linear_wrapper.cpp:67).  Each entry point below is the double instantiation of the fp32 one of the same name:
+ * same operands, shapes, NULL conventions and index arguments, every floating-point buffer in double.
+ * cm_spline_*_f64 accept any noutputs > 0.
+ */
+int cm_mp_forward_f64(const double *X, const double *Y, const double *R, const int32_t *sender,
+                      const int32_t *first_occ, int64_t nnodes, int64_t nedges, int channels,
+                      double *out, cm_stream_t stream);
+int cm_mp_backward_f64(const double *X, const double *Y, const double *R, const double *grad_out,
+                       const int32_t *sender, const int32_t *first_occ, const int32_t *sender_perm,
+                       const int32_t *sender_offsets, int64_t nnodes, int64_t nedges, int channels,
+                       double *gX, double *gY, double *gR, double *edge_scratch, cm_stream_t stream);
+int cm_sh_forward_f64(const double *xyz, int64_t nedges, double *Y, cm_stream_t stream);
+int cm_sh_backward_f64(const double *xyz, const double *grad_Y, int64_t nedges, double *grad_xyz,
+                       cm_stream_t stream);
+int cm_spline_forward_f64(const double *r, const double *r_knots, const double *coeffs, int64_t nedges,
+                          int nknots, int noutputs, double r_width, double r_max, double *R_out,
+                          double *R_deriv, cm_stream_t stream);
+int cm_spline_backward_f64(const double *r, const double *r_knots, const double *coeffs,
+                           const double *grad_R, int64_t nedges, int nknots, int noutputs,
+                           double r_width, double r_max, double *grad_r, cm_stream_t stream);
+int cm_symcon_tables_f64(const int32_t *term3_off, const int32_t *term3_path, const double *term3_val,
+                         int n3, const int32_t *term2_off, const int32_t *term2_path,
+                         const double *term2_val, int n2, const double *W3, const double *W2,
+                         const double *W1, int nelements, int P3, int P2, int P1, int channels,
+                         double *T3, double *T2, double *T1, cm_stream_t stream);
+int cm_symcon_forward_f64(const double *X, const int32_t *node_perm, const int32_t *group_offsets,
+                          const int32_t *mono3_ijk, int n3, const int32_t *mono2_ij, int n2,
+                          const double *T3, const double *T2, const double *T1, int64_t nnodes,
+                          int nelements, int channels, double *out, double *grad, cm_stream_t stream);
+int cm_symcon_backward_f64(const double *grad, const double *grad_out, int64_t nnodes, int channels,
+                           double *gX, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Neighbour list on the device: all ordered pairs (i, j, S) with |r_j - r_i + S . cell| < cutoff, (j, S) != (i, 0),
  * sorted lexicographically by (i, j, Sx, Sy, Sz) -- the step before the path.  The reference leaves it to the
  * host: its model consumes data["edge_index"] / ["shifts"] built upstream (models/InvariantMACE.py:297-301) and its
