@@ -1,1 +1,2 @@
+from .ase_calculator import MACECalculator  # noqa: F401
 from .device_calculator import DeviceCalculator  # noqa: F401
