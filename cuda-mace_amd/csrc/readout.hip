@@ -9,7 +9,8 @@
 //   d2[n,c] = scale * sum_j W2a[c, j] * w2b[j] * act'(z_j)                     (= d e[n] / d h2[n, c], stored in fp32)
 //   d e[n] / d h1[n, c] = scale * w1[c]                                        (constant, not stored)
 //
-// and, on request, the [N, 2C] fp64 concatenation of the features that the model returns as "node_feats".  The
+// and, on request, the [N, 2C] fp64 concatenation of the features that the model returns as "node_feats" (row n
+// optionally written to row feats_rows[n], for callers that keep their nodes in another order internally).  The
 // backward is then a scaling of those derivatives by the incoming gradient of e[n].
 //
 // Work split: a workgroup of 256 threads takes 16 nodes; their h2 rows are staged in LDS with coalesced loads and
@@ -30,7 +31,8 @@ constexpr int kLdS = kMaxC + 1;    // padded row stride of the feature tile: the
 __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     const float *__restrict__ h1, const float *__restrict__ h2, const double *__restrict__ w1, const double *__restrict__ W2a,
     const double *__restrict__ w2b, double act_cst, double scale, double shift, int nnodes, int C, int H,
-    double *__restrict__ node_es, float *__restrict__ d2, double *__restrict__ feats64) {
+    double *__restrict__ node_es, float *__restrict__ d2, double *__restrict__ feats64,
+    const int32_t *__restrict__ feats_rows) {
   __shared__ double sW[kMaxC * kLdW];      // W2a [C, H], H padded to 16 columns with zeros
   __shared__ float s2[kNodes * kLdS];
   __shared__ double sD[kNodes * kHidden];  // w2b[j] * act'(z_j) per node
@@ -47,8 +49,11 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     const float a = feats64 ? h1[static_cast<int64_t>(node0 + r) * C + c] : 0.f;
     s2[r * kLdS + c] = b;
     if (feats64) {
-      feats64[static_cast<int64_t>(node0 + r) * (2 * C) + c] = a;
-      feats64[static_cast<int64_t>(node0 + r) * (2 * C) + C + c] = b;
+      const int row = feats_rows ? feats_rows[node0 + r] : node0 + r;
+      if (static_cast<unsigned>(row) < static_cast<unsigned>(nnodes)) {
+        feats64[static_cast<int64_t>(row) * (2 * C) + c] = a;
+        feats64[static_cast<int64_t>(row) * (2 * C) + C + c] = b;
+      }
     }
   }
   __syncthreads();
@@ -96,7 +101,8 @@ __global__ void readout_backward_kernel(const double *__restrict__ g, const doub
 
 extern "C" int cm_readout_forward(const float *h1, const float *h2, const double *w1, const double *W2a, const double *w2b,
                                   double act_cst, double scale, double shift, int64_t nnodes, int channels, int hidden,
-                                  double *node_energies, float *d_h2, double *node_feats64, cm_stream_t stream) {
+                                  double *node_energies, float *d_h2, double *node_feats64, const int32_t *feats_rows,
+                                  cm_stream_t stream) {
   CM_REQUIRE(channels >= 1 && channels <= cm::kMaxC, "cm_readout_forward: channels=%d must be in [1, %d]", channels, cm::kMaxC);
   CM_REQUIRE(hidden >= 1 && hidden <= cm::kHidden, "cm_readout_forward: hidden=%d must be in [1, %d]", hidden, cm::kHidden);
   CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 2, "cm_readout_forward: nnodes out of range");
@@ -104,7 +110,7 @@ extern "C" int cm_readout_forward(const float *h1, const float *h2, const double
   CM_REQUIRE(h1 && h2 && w1 && W2a && w2b && node_energies && d_h2, "cm_readout_forward: NULL pointer");
   hipLaunchKernelGGL(cm::readout_forward_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nnodes, cm::kNodes))),
                      dim3(cm::kNodes * cm::kHidden), 0, cm::as_stream(stream), h1, h2, w1, W2a, w2b, act_cst, scale, shift,
-                     static_cast<int>(nnodes), channels, hidden, node_energies, d_h2, node_feats64);
+                     static_cast<int>(nnodes), channels, hidden, node_energies, d_h2, node_feats64, feats_rows);
   return cm::check_launch("cm_readout_forward");
 }
 

@@ -54,7 +54,7 @@ SIGNATURES = {
     "cm_symcon_forward": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
     "cm_symcon_builtin_structure": (_i32, [_p, _i32, _p, _i32, _p, _p]),
     "cm_symcon_backward": (_i32, [_p, _p, _i64, _i32, _p, _p]),
-    "cm_readout_forward": (_i32, [_p] * 5 + [_f64, _f64, _f64, _i64, _i32, _i32, _p, _p, _p, _p]),
+    "cm_readout_forward": (_i32, [_p] * 5 + [_f64, _f64, _f64, _i64, _i32, _i32, _p, _p, _p, _p, _p]),
     "cm_readout_backward": (_i32, [_p, _p, _p, _f64, _i64, _i32, _p, _p, _p]),
     "cm_neighbour_list_workspace": (_sz, [_i64, _i64]),
     "cm_neighbour_list_count": (_i32, [_p, _p, _i32, _i32, _i32, _f64, _i64, _i64, _p, _sz, _p, _p, _p]),
@@ -486,8 +486,10 @@ def neighbour_list(positions, cell, pbc, cutoff: float, max_cells: int = 0):
 
 
 # ---- readouts -------------------------------------------------------------------------------------
-def readout_forward(h1, h2, w1, W2a, w2b, act_cst: float, scale: float, shift: float, want_feats: bool = True):
-    """(node_energies fp64 [N], d_h2 fp32 [N, C], node_feats fp64 [N, 2C] or None)."""
+def readout_forward(h1, h2, w1, W2a, w2b, act_cst: float, scale: float, shift: float, want_feats: bool = True,
+                    feats_rows=None):
+    """(node_energies fp64 [N], d_h2 fp32 [N, C], node_feats fp64 [N, 2C] or None); feats_rows int32 [N] (a permutation)
+    sends the features of node n to row feats_rows[n]."""
     N, C = h1.shape
     H = W2a.shape[1]
     dev = h1.device
@@ -498,7 +500,7 @@ def readout_forward(h1, h2, w1, W2a, w2b, act_cst: float, scale: float, shift: f
         lib.cm_readout_forward(
             _dev(h1, F32, "h1"), _dev(h2, F32, "h2"), _dev(w1, F64, "w1"), _dev(W2a, F64, "W2a"), _dev(w2b, F64, "w2b"),
             float(act_cst), float(scale), float(shift), N, C, H, _dev(es, F64, "node_energies"), _dev(d2, F32, "d_h2"),
-            _dev(feats, F64, "node_feats"), _stream(),
+            _dev(feats, F64, "node_feats"), _dev(feats_rows, I32, "feats_rows") if want_feats else None, _stream(),
         )
     )
     return es, d2, feats

@@ -28,13 +28,19 @@ from cuda_mace.utils.irreps import Instruction
 
 
 # ---- the few upstream helpers the forward needs ------------------------------------------------------
-def scatter_sum(src: torch.Tensor, index: torch.Tensor, dim: int = -1, dim_size: Optional[int] = None) -> torch.Tensor:
+def scatter_sum(src: torch.Tensor, index: torch.Tensor, dim: int = -1, dim_size: Optional[int] = None,
+                ptr: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Sum of src over equal index values.  With `ptr` (index is sorted and ptr holds the segment boundaries, as for the
+    atoms of a batch of graphs) the sums are taken segment by segment in a fixed order, so that they do not vary from
+    run to run as atomic additions do."""
     dim = dim % src.dim()
     size = list(src.shape)
     size[dim] = int(dim_size) if dim_size is not None else int(index.max()) + 1
     if size[dim] == 1:
         # single graph: a plain reduction, whose summation order does not vary from run to run
         return src.sum(dim=dim, keepdim=True)
+    if ptr is not None and ptr.numel() == size[dim] + 1:
+        return torch.segment_reduce(src, "sum", offsets=ptr, axis=dim)
     out = torch.zeros(size, dtype=src.dtype, device=src.device)
     return out.index_add_(dim, index, src)
 
@@ -268,15 +274,19 @@ class InvariantResidualInteraction(torch.nn.Module):
 
 class OptimizedInvariantMACE(torch.nn.Module):
     def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True,
-                 fused_readout: bool = True, fused_contraction: bool = True):
+                 fused_readout: bool = True, fused_contraction: bool = True, spatial_order_min_atoms: Optional[int] = 8192):
         """fused_radial=True evaluates the spherical harmonics and the radial spline inside the message-passing kernels
         (same numbers; no [16, nedges] or [nedges, 4C] tensors in memory); False keeps the reference's separate
         SphericalHarmonics -> CubicSpline -> message passing steps.  fused_readout=True evaluates both readouts, scale
         and shift in one fp64 kernel per direction when the readout modules have the standard form; False (or any other
         form, or several heads) runs the modules themselves in fp64 as the reference does.  fused_contraction=True runs the
         channel-mixing linear before each symmetric contraction and the contraction as one autograd node whose backward is
-        a single kernel; False keeps the reference's separate Linear / ElementalLinear and SymmetricContraction ops."""
+        a single kernel; False keeps the reference's separate Linear / ElementalLinear and SymmetricContraction ops.
+        spatial_order_min_atoms: from this many atoms on, the model works on a relabelled copy of the graph in which
+        atoms that are close in space have close indices (derived once per edge_index tensor), so that the gathers of
+        sender rows hit in cache; outputs come back in the caller's order.  None switches the relabelling off."""
         super().__init__()
+        self.spatial_order_min_atoms = spatial_order_min_atoms
         self.fused_radial = bool(fused_radial)
         assert int(mace_model.num_interactions) == 2, "exactly two interaction layers are supported"
         self.register_buffer("atomic_numbers", deepcopy(mace_model.atomic_numbers))
@@ -356,9 +366,58 @@ class OptimizedInvariantMACE(torch.nn.Module):
         g = lambda name: getattr(self, "contraction_%s_%d" % (name, i))  # noqa: E731
         return g("mono3"), g("mono2"), g("T3"), g("T2"), g("T1"), self._contraction_builtin[i]
 
+    def _spatial_order(self, data: Dict[str, torch.Tensor]):
+        """Relabelling of one neighbour list: atoms sorted by (graph, 3-D bin of half the cutoff, lexicographic), edges
+        re-sorted by the new (row 0, row 1) labels.  Returns (perm new -> old [N], inverse [N], edge_perm new -> old [E],
+        relabelled edge_index [2, E], relabelled batch [N]).  Any permutation is valid; this one is cheap and keeps
+        neighbours within a few hundred indices of each other."""
+        pos = data["positions"].detach()
+        batch, edge_index = data["batch"], data["edge_index"]
+        n = pos.shape[0]
+        bins = torch.floor((pos - pos.min(dim=0).values) / (0.5 * float(self.r_max))).long()
+        nb = int(bins.max()) + 1
+        key = ((batch * nb + bins[:, 0]) * nb + bins[:, 1]) * nb + bins[:, 2]
+        perm = torch.argsort(key, stable=True)
+        inverse = torch.empty_like(perm)
+        inverse[perm] = torch.arange(n, device=perm.device)
+        row0, row1 = inverse[edge_index[0]], inverse[edge_index[1]]
+        edge_perm = torch.argsort(row0 * n + row1, stable=True)
+        new_edges = torch.stack((row0[edge_perm], row1[edge_perm])).contiguous()
+        return perm, inverse, edge_perm, new_edges, batch[perm].contiguous()
+
     def forward(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
                 compute_virials: bool = False, compute_stress: bool = False,
                 compute_displacement: bool = False) -> Dict[str, Optional[torch.Tensor]]:
+        n = data["positions"].shape[0]
+        if self.spatial_order_min_atoms is None or n < self.spatial_order_min_atoms or training:
+            return self._forward_ordered(data, training, compute_force, compute_virials, compute_stress, compute_displacement)
+        # Same step on the relabelled graph.  Everything that depends only on the neighbour list or the species is
+        # derived once per tensor object; per call the positions are gathered into the new order and forces, node
+        # energies and node features gathered back (fixed-order gathers: results stay reproducible bit for bit).
+        perm, inverse, edge_perm, edge_index, batch = _cached(data["edge_index"], "_cm_spatial_order", None,
+                                                              lambda: self._spatial_order(data))
+        inner = dict(data)
+        inner["positions"] = data["positions"].detach().index_select(0, perm)
+        inner["edge_index"], inner["batch"] = edge_index, batch
+        inner["node_attrs"] = _cached(data["node_attrs"], "_cm_spatial_attrs", perm.data_ptr(),
+                                      lambda: data["node_attrs"].index_select(0, perm))
+        for name in ("shifts", "unit_shifts"):
+            if name in data:
+                t = data[name]
+                inner[name] = _cached(t, "_cm_spatial_rows", edge_perm.data_ptr(), lambda t=t: t.index_select(0, edge_perm))
+        rows = _cached(data["edge_index"], "_cm_spatial_rows32", None, lambda: (perm.int(), inverse))
+        out = self._forward_ordered(inner, training, compute_force, compute_virials, compute_stress, compute_displacement,
+                                    node_rows=rows)
+        for name in ("forces", "node_energy"):  # node_feats is already written in the caller's order
+            if out.get(name) is not None:
+                out[name] = out[name].index_select(0, inverse)
+        return out
+
+    def _forward_ordered(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
+                         compute_virials: bool = False, compute_stress: bool = False, compute_displacement: bool = False,
+                         node_rows=None) -> Dict[str, Optional[torch.Tensor]]:
+        """node_rows = (rows int32 [N], inverse int64 [N]): node n of `data` is node rows[n] of the caller; the
+        returned node_feats is written in the caller's order (every other per-node output stays in the order of `data`)."""
         data["positions"].requires_grad_(True)
         positions = data["positions"]
         node_attrs = data["node_attrs"]
@@ -386,7 +445,7 @@ class OptimizedInvariantMACE(torch.nn.Module):
 
         e0_per_head, node_feats_up = _cached(node_attrs, "_cm_species_only", id(self), species_only)
         node_e0 = _select_head(e0_per_head, zero_heads if node_heads is None else node_heads)
-        e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs)
+        e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
         node_feats = None
 
         # index structures shared by both layers, cached on the caller's tensors so that they are rebuilt only when
@@ -435,12 +494,15 @@ class OptimizedInvariantMACE(torch.nn.Module):
         if fused_readout:
             act_cst, scale, shift = self.readout_constants
             node_inter_es, node_feats_out = ReadoutEnergyAutograd.apply(
-                node_feats_list[0], node_feats_list[1], self.readout_w1, self.readout_W2a, self.readout_w2b, act_cst, scale, shift)
+                node_feats_list[0], node_feats_list[1], self.readout_w1, self.readout_W2a, self.readout_w2b, act_cst, scale, shift,
+                None if node_rows is None else node_rows[0])
         else:
             node_feats_out = torch.cat([f.double() for f in node_feats_list], dim=-1)
+            if node_rows is not None:
+                node_feats_out = node_feats_out.index_select(0, node_rows[1])
             node_inter_es = torch.sum(torch.stack(node_es_list, dim=0), dim=0)
             node_inter_es = self.scale_shift(node_inter_es, zero_heads if node_heads is None else node_heads)
-        inter_e = scatter_sum(src=node_inter_es.double(), index=batch, dim=-1, dim_size=num_graphs)
+        inter_e = scatter_sum(src=node_inter_es.double(), index=batch, dim=-1, dim_size=num_graphs, ptr=data["ptr"])
 
         total_energy = e0 + inter_e
         node_energy = node_e0 + node_inter_es

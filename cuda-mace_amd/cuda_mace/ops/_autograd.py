@@ -204,11 +204,13 @@ class LinearContractionAutograd(torch.autograd.Function):
 
 class ReadoutEnergyAutograd(torch.autograd.Function):
     """(h1, h2 fp32 [N, C]) -> (node energies fp64 [N], node_feats fp64 [N, 2C]): both readouts, scale and shift in one
-    kernel; the derivative with respect to h2 is produced by the same pass and only scaled in the backward."""
+    kernel; the derivative with respect to h2 is produced by the same pass and only scaled in the backward.  feats_rows
+    (int32 permutation, optional) places the features of node n in row feats_rows[n] of node_feats."""
 
     @staticmethod
-    def forward(ctx, h1, h2, w1, W2a, w2b, act_cst, scale, shift):
-        es, d2, feats = cabi.readout_forward(h1.detach().contiguous(), h2.detach().contiguous(), w1, W2a, w2b, act_cst, scale, shift)
+    def forward(ctx, h1, h2, w1, W2a, w2b, act_cst, scale, shift, feats_rows=None):
+        es, d2, feats = cabi.readout_forward(h1.detach().contiguous(), h2.detach().contiguous(), w1, W2a, w2b, act_cst, scale, shift,
+                                             feats_rows=feats_rows)
         ctx.save_for_backward(w1, d2)
         ctx.scale = float(scale)
         ctx.mark_non_differentiable(feats)
@@ -218,7 +220,7 @@ class ReadoutEnergyAutograd(torch.autograd.Function):
     def backward(ctx, grad_es, _grad_feats):
         w1, d2 = ctx.saved_tensors
         g1, g2 = cabi.readout_backward(grad_es.contiguous(), w1, d2, ctx.scale, ctx.needs_input_grad[0], ctx.needs_input_grad[1])
-        return g1, g2, None, None, None, None, None, None
+        return g1, g2, None, None, None, None, None, None, None
 
 
 # ------------------------------------------------------------------------------------------------

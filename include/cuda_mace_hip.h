@@ -332,12 +332,14 @@ int cm_neighbour_list_fill(const double *positions, double cutoff, int64_t nnode
  *   act(z) = act_cst * z * sigmoid(z) (1/sqrt(fan_in) folded into both);
  *   node_energies[n] = scale * (h1[n] . w1 + sum_j w2b[j] act((h2[n] . W2a)_j)) + shift        fp64 [nnodes]
  *   d_h2 fp32 [nnodes, channels] = d node_energies[n] / d h2[n, c]   (d / d h1 is scale * w1, not stored)
- *   node_feats64 fp64 [nnodes, 2 * channels] = [h1 | h2], or NULL.
+ *   node_feats64 fp64 [nnodes, 2 * channels] = [h1 | h2], or NULL; with feats_rows int32 [nnodes] (a permutation; may
+ *   be NULL) the features of node n go to row feats_rows[n].
  * Backward: grad_h1[n, c] = g[n] * scale * w1[c], grad_h2[n, c] = g[n] * d_h2[n, c] (either may be NULL).
  */
 int cm_readout_forward(const float *h1, const float *h2, const double *w1, const double *W2a, const double *w2b,
                        double act_cst, double scale, double shift, int64_t nnodes, int channels, int hidden,
-                       double *node_energies, float *d_h2, double *node_feats64, cm_stream_t stream);
+                       double *node_energies, float *d_h2, double *node_feats64, const int32_t *feats_rows,
+                       cm_stream_t stream);
 int cm_readout_backward(const double *grad_node_energies, const double *w1, const float *d_h2, double scale,
                         int64_t nnodes, int channels, float *grad_h1, float *grad_h2, cm_stream_t stream);
 

@@ -181,3 +181,39 @@ def test_config4_full_size_properties(cabi):
     assert abs(e0 - e1) <= 2e-6 * abs(e0)
     f_rot = a["forces"].detach() @ Q
     assert float((c["forces"].detach() - f_rot).abs().max()) <= 2e-5 * max(fmax, 1.0)
+
+
+def test_spatial_relabelling_is_transparent(cabi):
+    """The model on its internally relabelled graph (atoms sorted by spatial bin, edges re-sorted) returns, in the caller's
+    order, what it returns without the relabelling: a batch of two boxes with virials, against the plain path and the
+    fp64 reference; the relabelled run repeats bit for bit."""
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.utils.synthetic import collate
+
+    systems = [make_system(n, 4, seed=40 + k, density=0.1) for k, n in enumerate((260, 190))]
+    deg = sum(int(d["edge_index"].shape[1]) for d in systems) / sum(int(d["positions"].shape[0]) for d in systems)
+    upstream = SyntheticInvariantMACE(channels=64, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=deg, seed=13)
+    params = upstream.export_params()
+    plain = OptimizedInvariantMACE(upstream, device="cuda", spatial_order_min_atoms=None)
+    ordered = OptimizedInvariantMACE(upstream, device="cuda", spatial_order_min_atoms=0)
+    data = to_device(collate(systems), "cuda")
+    a = plain(dict(data), compute_virials=True, compute_stress=True)
+    b = ordered(dict(data), compute_virials=True, compute_stress=True)
+    perm = data["edge_index"]._cm_spatial_order[1][0]
+    assert not torch.equal(perm, torch.arange(perm.numel(), device="cuda"))  # the relabelling did something
+    scale = float(a["forces"].abs().max())
+    torch.testing.assert_close(b["energy"].detach(), a["energy"].detach(), rtol=1e-7, atol=1e-7)
+    torch.testing.assert_close(b["forces"], a["forces"], rtol=0, atol=2e-6 * scale)
+    torch.testing.assert_close(b["node_energy"].detach(), a["node_energy"].detach(), rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(b["node_feats"].detach(), a["node_feats"].detach(), rtol=1e-5, atol=1e-6 * float(a["node_feats"].abs().max()))
+    torch.testing.assert_close(b["virials"], a["virials"], rtol=1e-5, atol=1e-5 * float(a["virials"].abs().max()))
+    torch.testing.assert_close(b["stress"], a["stress"], rtol=1e-5, atol=1e-5 * float(a["stress"].abs().max()))
+    again = ordered(dict(data), compute_virials=True, compute_stress=True)
+    assert torch.equal(again["forces"], b["forces"]) and torch.equal(again["energy"], b["energy"])
+    start = 0
+    for g, d in enumerate(systems):
+        n = d["positions"].shape[0]
+        ref = M.energy_and_forces(params, d)
+        assert abs(float(b["energy"][g].detach()) - float(ref["energy"])) <= 1e-5 * abs(float(ref["energy"])) + 1e-6
+        assert float((b["forces"][start:start + n].double().cpu() - ref["forces"]).abs().max()) <= 1e-4
+        start += n

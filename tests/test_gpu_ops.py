@@ -376,6 +376,11 @@ def test_readout_forward_backward(cabi, N, C, H, seed):
     es, d2, feats = cabi.readout_forward(dev(h1.float()), dev(h2.float()), dev(w1), dev(W2a), dev(w2b), cst, scale, shift)
     close(es, ref.detach(), 1e-12, 1e-12)  # fp64 arithmetic on identical (fp32-representable) inputs
     assert torch.equal(feats.cpu(), torch.cat([h1, h2], dim=1))
+    # optional row map of the feature output: node n goes to row rows[n]; energies stay in place
+    rows = torch.randperm(N, generator=g).int()
+    es_m, _, feats_m = cabi.readout_forward(dev(h1.float()), dev(h2.float()), dev(w1), dev(W2a), dev(w2b), cst, scale, shift,
+                                            feats_rows=dev(rows))
+    assert torch.equal(es_m, es) and torch.equal(feats_m.cpu()[rows.long()], torch.cat([h1, h2], dim=1))
     g1, g2 = cabi.readout_backward(dev(gn), dev(w1), d2, scale)
     close(g1, a1.grad, 1e-6, 1e-7)
     close(g2, a2.grad, 1e-6, 1e-7)
