@@ -22,8 +22,8 @@ from cuda_mace.ops.linear import ElementalLinear, Linear, ScalarElementalLinear
 from cuda_mace.ops.spherical_harmonics import SphericalHarmonics
 from cuda_mace.ops.symmetric_contraction import SymmetricContraction as CUDAContraction
 from cuda_mace import _cabi as cabi
-from cuda_mace.ops._autograd import (EdgeGeometryAutograd, LinearContractionAutograd, ReadoutEnergyAutograd, _cached, groups_of,
-                                     groups_of_one_hot, monomials_from_packed)
+from cuda_mace.ops._autograd import (EdgeGeometryAutograd, LinearContractionAutograd, ReadoutEnergyAutograd, _cached, _cached_for,
+                                     groups_of, groups_of_one_hot, monomials_from_packed)
 from cuda_mace.utils.irreps import Instruction
 
 
@@ -272,6 +272,10 @@ class InvariantResidualInteraction(torch.nn.Module):
         return self.linear.weights_transposed, self.linear.weights, 1.0 / sqrt(K), False
 
 
+class _WeightsToken:
+    """Identity of one model's (frozen) weights; a cache entry that holds it can never be taken for another model's."""
+
+
 class OptimizedInvariantMACE(torch.nn.Module):
     def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True,
                  fused_readout: bool = True, fused_contraction: bool = True, spatial_order_min_atoms: Optional[int] = 8192):
@@ -287,6 +291,7 @@ class OptimizedInvariantMACE(torch.nn.Module):
         sender rows hit in cache; outputs come back in the caller's order.  None switches the relabelling off."""
         super().__init__()
         self.spatial_order_min_atoms = spatial_order_min_atoms
+        self._weights_token = _WeightsToken()  # what caches of weight-dependent, species-only tensors are keyed on
         self.fused_radial = bool(fused_radial)
         assert int(mace_model.num_interactions) == 2, "exactly two interaction layers are supported"
         self.register_buffer("atomic_numbers", deepcopy(mace_model.atomic_numbers))
@@ -399,12 +404,12 @@ class OptimizedInvariantMACE(torch.nn.Module):
         inner = dict(data)
         inner["positions"] = data["positions"].detach().index_select(0, perm)
         inner["edge_index"], inner["batch"] = edge_index, batch
-        inner["node_attrs"] = _cached(data["node_attrs"], "_cm_spatial_attrs", perm.data_ptr(),
-                                      lambda: data["node_attrs"].index_select(0, perm))
+        inner["node_attrs"] = _cached_for(data["edge_index"], "_cm_spatial_attrs", data["node_attrs"],
+                                          lambda: data["node_attrs"].index_select(0, perm))
         for name in ("shifts", "unit_shifts"):
             if name in data:
                 t = data[name]
-                inner[name] = _cached(t, "_cm_spatial_rows", edge_perm.data_ptr(), lambda t=t: t.index_select(0, edge_perm))
+                inner[name] = _cached_for(data["edge_index"], "_cm_spatial_" + name, t, lambda t=t: t.index_select(0, edge_perm))
         rows = _cached(data["edge_index"], "_cm_spatial_rows32", None, lambda: (perm.int(), inverse))
         out = self._forward_ordered(inner, training, compute_force, compute_virials, compute_stress, compute_displacement,
                                     node_rows=rows)
@@ -443,7 +448,7 @@ class OptimizedInvariantMACE(torch.nn.Module):
                 return (self.atomic_energies_fn(attrs64),
                         self.interactions[0].linear_up(self.node_embedding(attrs64).float()))
 
-        e0_per_head, node_feats_up = _cached(node_attrs, "_cm_species_only", id(self), species_only)
+        e0_per_head, node_feats_up = _cached_for(node_attrs, "_cm_species_only", self._weights_token, species_only)
         node_e0 = _select_head(e0_per_head, zero_heads if node_heads is None else node_heads)
         e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
         node_feats = None

@@ -35,6 +35,19 @@ def _cached(owner: torch.Tensor, slot: str, key, build):
     return val
 
 
+def _cached_for(owner: torch.Tensor, slot: str, other, build):
+    """Value derived from `owner` and `other` (a tensor, or any object that stands for a set of weights), kept on
+    `owner`; rebuilt when either was modified in place or `other` is another object.  The entry holds a reference to
+    `other`, so neither its address nor its id can be recycled under the cache."""
+    hit = owner.__dict__.get(slot)
+    tag = (owner._version, owner.data_ptr(), getattr(other, "_version", 0))
+    if hit is not None and hit[0] is other and hit[1] == tag:
+        return hit[2]
+    val = build()
+    owner.__dict__[slot] = (other, tag, val)
+    return val
+
+
 def csr_of(receiver: torch.Tensor, nnodes: int) -> torch.Tensor:
     return _cached(receiver, "_cm_csr", nnodes, lambda: cabi.first_occurences(receiver, nnodes))
 

@@ -16,7 +16,8 @@ def test_md_like_walk(cabi, use_graph):
     data = to_device(make_system(n, 10, seed=11, density=0.1), "cuda")
     avg = data["edge_index"].shape[1] / n
     model = OptimizedInvariantMACE(SyntheticInvariantMACE(channels=64, atomic_numbers=tuple(range(1, 11)),
-                                                          avg_num_neighbors=avg, seed=12), device="cuda")
+                                                          avg_num_neighbors=avg, seed=12), device="cuda",
+                                   spatial_order_min_atoms=0 if use_graph else None)  # one of the two with relabelling
     calc = DeviceCalculator(model, data["node_attrs"], cutoff=5.0, skin=0.4, pbc=(True, True, True), cell=data["cell"],
                             use_graph=use_graph)
     g = torch.Generator(device="cuda").manual_seed(1)

@@ -5,8 +5,8 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("natoms,channels,periodic", [(21, 64, False), (600, 128, True)])
-def test_graph_replays_equal_eager(cabi, natoms, channels, periodic):
+@pytest.mark.parametrize("natoms,channels,periodic,relabel", [(21, 64, False, False), (600, 128, True, False), (600, 64, True, True)])
+def test_graph_replays_equal_eager(cabi, natoms, channels, periodic, relabel):
     from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
     from cuda_mace.utils.graph import GraphedStep
     from cuda_mace.utils.synthetic import make_system, to_device
@@ -19,7 +19,8 @@ def test_graph_replays_equal_eager(cabi, natoms, channels, periodic):
         numbers = (1, 6, 7, 8)
     avg = data["edge_index"].shape[1] / natoms
     model = OptimizedInvariantMACE(SyntheticInvariantMACE(channels=channels, atomic_numbers=numbers, avg_num_neighbors=avg,
-                                                          seed=4), device="cuda")
+                                                          seed=4), device="cuda",
+                                   spatial_order_min_atoms=0 if relabel else None)  # relabel: the spatially re-ordered graph
     dev = to_device(data, "cuda")
     step = GraphedStep(model, dev)
     g = torch.Generator(device="cuda").manual_seed(0)
