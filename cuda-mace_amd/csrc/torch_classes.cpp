@@ -34,6 +34,15 @@ void *stream_of(const Tensor &t) { return c10::hip::getCurrentHIPStream(t.device
 
 #define CM_CALL(expr) TORCH_CHECK((expr) == 0, cm_last_error())
 
+// Profiler range over one autograd forward or backward, as the reference's PUSH_RANGE / POP_RANGE (include/utils.h:9-21);
+// emitted only when tracing is switched on (see cm_trace_push).
+struct TraceRange {
+  explicit TraceRange(const char *name) { cm_trace_push(name); }
+  ~TraceRange() { cm_trace_pop(); }
+  TraceRange(const TraceRange &) = delete;
+  TraceRange &operator=(const TraceRange &) = delete;
+};
+
 void need(const Tensor &t, c10::ScalarType dtype, const char *name) {
   TORCH_CHECK(t.is_cuda(), name, " must live on the GPU (got a ", t.device(), " tensor)");
   TORCH_CHECK(t.scalar_type() == dtype, name, " must be ", dtype, " (got ", t.scalar_type(), ")");
@@ -176,6 +185,7 @@ class InvariantMessagePassingTPAutograd : public torch::autograd::Function<Invar
  public:
   static Tensor forward(AutogradContext *ctx, Tensor X, Tensor Y, Tensor radial, Tensor sender_list, Tensor receiver_list,
                         int64_t nnodes) {
+    TraceRange range("cuda_mace:message_passing forward");
     X = X.contiguous(), Y = Y.contiguous();
     Tensor R = radial.contiguous();
     const auto dt = float_type_of(X, "X");
@@ -201,6 +211,7 @@ class InvariantMessagePassingTPAutograd : public torch::autograd::Function<Invar
   }
 
   static variable_list backward(AutogradContext *ctx, variable_list grad_outputs) {
+    TraceRange range("cuda_mace:message_passing backward");
     auto saved = ctx->get_saved_variables();
     const Tensor &X = saved[0], &Y = saved[1], &R = saved[2], &sender = saved[3], &first_occ = saved[4];
     const int64_t nnodes = ctx->saved_data["nnodes"].toInt();
@@ -232,6 +243,7 @@ class InvariantMessagePassingTPAutograd : public torch::autograd::Function<Invar
 class SphericalHarmonicsAutograd : public torch::autograd::Function<SphericalHarmonicsAutograd> {
  public:
   static Tensor forward(AutogradContext *ctx, Tensor xyz) {
+    TraceRange range("cuda_mace:spherical_harmonics forward");
     xyz = xyz.contiguous();
     const auto dt = float_type_of(xyz, "xyz");
     need(xyz, dt, "xyz");
@@ -245,6 +257,7 @@ class SphericalHarmonicsAutograd : public torch::autograd::Function<SphericalHar
     return Y;
   }
   static variable_list backward(AutogradContext *ctx, variable_list grad_outputs) {
+    TraceRange range("cuda_mace:spherical_harmonics backward");
     const Tensor xyz = ctx->get_saved_variables()[0];
     Tensor g = grad_outputs[0].contiguous();
     need(g, xyz.scalar_type(), "grad_output");
@@ -261,6 +274,7 @@ class SphericalHarmonicsAutograd : public torch::autograd::Function<SphericalHar
 class CubicSplineAutograd : public torch::autograd::Function<CubicSplineAutograd> {
  public:
   static Tensor forward(AutogradContext *ctx, Tensor r, Tensor r_knots, Tensor coeffs, double r_width, double r_max) {
+    TraceRange range("cuda_mace:cubic_spline forward");
     Tensor rc = r.contiguous().view({-1});
     const auto dt = float_type_of(rc, "r");
     need(rc, dt, "r"), need(r_knots, dt, "r_knots"), need(coeffs, dt, "coeffs");
@@ -284,6 +298,7 @@ class CubicSplineAutograd : public torch::autograd::Function<CubicSplineAutograd
     return R;
   }
   static variable_list backward(AutogradContext *ctx, variable_list grad_outputs) {
+    TraceRange range("cuda_mace:cubic_spline backward");
     auto saved = ctx->get_saved_variables();
     const Tensor &r = saved[0], &knots = saved[1], &coeffs = saved[2];
     Tensor g = grad_outputs[0].contiguous();
@@ -320,6 +335,7 @@ Tensor run_linear(const Tensor &X, const Tensor &WT, const Tensor &perm, const T
 class LinearAutograd : public torch::autograd::Function<LinearAutograd> {
  public:
   static Tensor forward(AutogradContext *ctx, Tensor X, Tensor W, Tensor W_T) {
+    TraceRange range("cuda_mace:linear forward");
     X = X.contiguous();
     need(X, torch::kFloat32, "X"), need(W, torch::kFloat32, "W"), need(W_T, torch::kFloat32, "W_T");
     TORCH_CHECK(X.dim() == 3 && X.size(1) == 16, "X must be [nnodes, 16, K]");
@@ -331,6 +347,7 @@ class LinearAutograd : public torch::autograd::Function<LinearAutograd> {
     return run_linear(X, W_T, Tensor(), Tensor(), false, scale);
   }
   static variable_list backward(AutogradContext *ctx, variable_list grad_outputs) {
+    TraceRange range("cuda_mace:linear backward");
     const Tensor W = ctx->get_saved_variables()[0];
     // dX = scale * g . W^T: the operand the kernel wants is the transpose of W^T, i.e. W itself
     Tensor dX = run_linear(grad_outputs[0].contiguous(), W, Tensor(), Tensor(), false,
@@ -342,6 +359,7 @@ class LinearAutograd : public torch::autograd::Function<LinearAutograd> {
 class ElementalLinearAutograd : public torch::autograd::Function<ElementalLinearAutograd> {
  public:
   static Tensor forward(AutogradContext *ctx, Tensor X, Tensor W, Tensor W_T, Tensor one_hot) {
+    TraceRange range("cuda_mace:elemental_linear forward");
     X = X.contiguous();
     need(X, torch::kFloat32, "X"), need(W, torch::kFloat32, "W"), need(W_T, torch::kFloat32, "W_T");
     TORCH_CHECK((X.dim() == 3 && X.size(1) == 16) || X.dim() == 2, "X must be [nnodes, 16, K] or [nnodes, K]");
@@ -355,6 +373,7 @@ class ElementalLinearAutograd : public torch::autograd::Function<ElementalLinear
     return run_linear(X, W_T, groups[0], groups[1], true, scale);
   }
   static variable_list backward(AutogradContext *ctx, variable_list grad_outputs) {
+    TraceRange range("cuda_mace:elemental_linear backward");
     auto saved = ctx->get_saved_variables();
     Tensor dX = run_linear(grad_outputs[0].contiguous(), saved[0], saved[1], saved[2], true,
                            static_cast<float>(ctx->saved_data["scale"].toDouble()));
@@ -442,6 +461,7 @@ class SymmetricContractionAutograd : public torch::autograd::Function<SymmetricC
                         Tensor U3_indices, Tensor U3_values, Tensor U2_num_nonzero, Tensor U2_indices, Tensor U2_values,
                         Tensor U1_num_nonzero, Tensor U1_index, Tensor W3, Tensor W2, Tensor W1, int64_t W3_size, int64_t W2_size,
                         int64_t W1_size) {
+    TraceRange range("cuda_mace:symmetric_contraction forward");
     X = X.contiguous();
     const auto dt = float_type_of(X, "X");
     need(X, dt, "X"), need(atom_types, torch::kInt32, "atom_types");
@@ -490,6 +510,7 @@ class SymmetricContractionAutograd : public torch::autograd::Function<SymmetricC
   }
 
   static variable_list backward(AutogradContext *ctx, variable_list grad_outputs) {
+    TraceRange range("cuda_mace:symmetric_contraction backward");
     const Tensor grad = ctx->get_saved_variables()[0];
     const int64_t N = grad.size(0), C = grad.size(2);
     Tensor g = grad_outputs[0].contiguous().view({N, C});

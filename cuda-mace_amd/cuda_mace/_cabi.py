@@ -34,6 +34,9 @@ SIGNATURES = {
     "cm_abi_version": (_i32, []),
     "cm_last_error": (ctypes.c_char_p, []),
     "cm_channels_supported": (_i32, [_i32]),
+    "cm_trace_enabled": (_i32, []),
+    "cm_trace_push": (None, [ctypes.c_char_p]),
+    "cm_trace_pop": (None, []),
     "cm_first_occurences": (_i32, [_p, _i64, _i64, _p, _p]),
     "cm_stable_key_sort_workspace": (_sz, [_i64, _i64]),
     "cm_stable_key_sort": (_i32, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),

@@ -11,6 +11,8 @@ instead of once per call.
 """
 from __future__ import annotations
 
+import functools
+
 import numpy as np
 import torch
 
@@ -22,6 +24,31 @@ F32, I32 = torch.float32, torch.int32
 def _require(cond, msg):
     if not cond:
         raise RuntimeError(msg)
+
+
+_TRACE = bool(cabi.lib.cm_trace_enabled())  # decided once: CUDA_MACE_TRACE must be set before the import
+
+
+def _traced(name: str):
+    """Profiler range around an autograd forward / backward (the reference's PUSH_RANGE / POP_RANGE, include/utils.h:9-21);
+    the function is returned unchanged when tracing is off."""
+
+    def decorate(fn):
+        if not _TRACE:
+            return fn
+        label = ("cuda_mace:" + name).encode()
+
+        @functools.wraps(fn)
+        def wrapper(*args, **kwargs):
+            cabi.lib.cm_trace_push(label)
+            try:
+                return fn(*args, **kwargs)
+            finally:
+                cabi.lib.cm_trace_pop()
+
+        return wrapper
+
+    return decorate
 
 
 def _cached(owner: torch.Tensor, slot: str, key, build):
@@ -81,6 +108,7 @@ class InvariantMessagePassingSplineTPAutograd(torch.autograd.Function):
     Differentiable in X, Y and the edge lengths r."""
 
     @staticmethod
+    @_traced("message_passing_spline forward")
     def forward(ctx, X, Y, r, r_knots, coeffs, r_width, r_max, sender_list, receiver_list, nnodes):
         _require(X.dtype == F32 and Y.dtype == F32 and r.dtype == F32 and coeffs.dtype == F32 and r_knots.dtype == F32,
                  "fused message passing: fp32 tensors expected")
@@ -96,6 +124,7 @@ class InvariantMessagePassingSplineTPAutograd(torch.autograd.Function):
         return out
 
     @staticmethod
+    @_traced("message_passing_spline backward")
     def backward(ctx, grad_out):
         X, Y, r, r_knots, coeffs, sender, first_occ = ctx.saved_tensors
         need_x, need_y, need_r = ctx.needs_input_grad[:3]
@@ -116,6 +145,7 @@ class InvariantMessagePassingEdgeTPAutograd(torch.autograd.Function):
     (vectors, |vectors|); differentiable in X and the vectors."""
 
     @staticmethod
+    @_traced("message_passing_edges forward")
     def forward(ctx, X, vectors, r_knots, coeffs, r_width, r_max, sender_list, receiver_list, nnodes):
         _require(X.dtype == F32 and vectors.dtype == F32 and coeffs.dtype == F32 and r_knots.dtype == F32,
                  "edge message passing: fp32 tensors expected")
@@ -131,6 +161,7 @@ class InvariantMessagePassingEdgeTPAutograd(torch.autograd.Function):
         return out
 
     @staticmethod
+    @_traced("message_passing_edges backward")
     def backward(ctx, grad_out):
         X, vectors, r_knots, coeffs, sender, first_occ = ctx.saved_tensors
         need_x, need_v = ctx.needs_input_grad[:2]
@@ -150,6 +181,7 @@ class EdgeGeometryAutograd(torch.autograd.Function):
     and the sorted view of row_b (the same index structures message passing uses), in fp64, without atomics."""
 
     @staticmethod
+    @_traced("edge_geometry forward")
     def forward(ctx, positions, shifts, row_a, row_b):
         _require(row_a.dtype == I32 and row_b.dtype == I32, "edge geometry: int32 edge lists expected")
         _require(positions.dim() == 2 and positions.shape[1] == 3, "edge geometry: positions must be [nnodes, 3]")
@@ -162,6 +194,7 @@ class EdgeGeometryAutograd(torch.autograd.Function):
         return vec, length
 
     @staticmethod
+    @_traced("edge_geometry backward")
     def backward(ctx, grad_vec, grad_len):
         if grad_vec is None and grad_len is None:
             return None, None, None, None
@@ -194,6 +227,7 @@ class LinearContractionAutograd(torch.autograd.Function):
     tables = (mono3, mono2, T3, T2, T1, builtin)."""
 
     @staticmethod
+    @_traced("linear_contraction forward")
     def forward(ctx, X, W_T, W, scale, lin_groups, sym_groups, tables):
         mono3, mono2, T3, T2, T1, builtin = tables
         lp, lo = lin_groups if lin_groups is not None else (None, None)
@@ -207,6 +241,7 @@ class LinearContractionAutograd(torch.autograd.Function):
         return out
 
     @staticmethod
+    @_traced("linear_contraction backward")
     def backward(ctx, grad_out):
         grad, W = ctx.saved_tensors
         lp, lo = ctx.lin_groups if ctx.lin_groups is not None else (None, None)
@@ -221,6 +256,7 @@ class ReadoutEnergyAutograd(torch.autograd.Function):
     (int32 permutation, optional) places the features of node n in row feats_rows[n] of node_feats."""
 
     @staticmethod
+    @_traced("readout forward")
     def forward(ctx, h1, h2, w1, W2a, w2b, act_cst, scale, shift, feats_rows=None):
         es, d2, feats = cabi.readout_forward(h1.detach().contiguous(), h2.detach().contiguous(), w1, W2a, w2b, act_cst, scale, shift,
                                              feats_rows=feats_rows)
@@ -230,6 +266,7 @@ class ReadoutEnergyAutograd(torch.autograd.Function):
         return es, feats
 
     @staticmethod
+    @_traced("readout backward")
     def backward(ctx, grad_es, _grad_feats):
         w1, d2 = ctx.saved_tensors
         g1, g2 = cabi.readout_backward(grad_es.contiguous(), w1, d2, ctx.scale, ctx.needs_input_grad[0], ctx.needs_input_grad[1])

@@ -36,6 +36,16 @@ const char *cm_last_error(void);
 int cm_channels_supported(int channels);
 
 /* ---------------------------------------------------------------------------------------------
+ * Profiler ranges.  The reference opens an NVTX range named "cuda_mace" around every autograd forward and backward
+ * (PUSH_RANGE / POP_RANGE, include/utils.h:9-21; e.g. src/linear.cpp:15, :24).  Here the ranges are ROCTx ranges,
+ * emitted only when the environment variable CUDA_MACE_TRACE is set to a non-zero value at the first call; the
+ * marker library is looked up at run time.  cm_trace_push / cm_trace_pop do nothing otherwise.
+ */
+int cm_trace_enabled(void);
+void cm_trace_push(const char *name);
+void cm_trace_pop(void);
+
+/* ---------------------------------------------------------------------------------------------
  * CSR offsets of a non-decreasing receiver list.
  * Replaces jit_calculate_first_occurences (jit_wrappers/src/invariant_message_passing_wrapper.cpp:19-70)
  * and calculate_first_occurences_kernel_ptr (cuda/src/invariant_message_passing_impl.cu:8-72).

@@ -52,3 +52,27 @@ def test_binding_rejects_host_tensors():
 
     with pytest.raises(RuntimeError, match="GPU"):
         _cabi.sh_forward(torch.zeros(4, 3))
+
+
+def test_profiler_ranges_are_off_unless_asked_for():
+    """cm_trace_* do nothing by default; with CUDA_MACE_TRACE=1 the marker library is found at run time and push / pop
+    can be called without a profiler attached.  The switch is read once per process, hence the child processes."""
+    import subprocess
+    import sys
+
+    code = (
+        "import ctypes; lib = ctypes.CDLL(%r); lib.cm_trace_push.argtypes = [ctypes.c_char_p]; lib.cm_trace_push.restype = None;"
+        "lib.cm_trace_pop.restype = None; lib.cm_trace_push(b'cuda_mace:test'); lib.cm_trace_pop(); print(lib.cm_trace_enabled())" % LIB
+    )
+    seen = {}
+    for value in (None, "0", "1"):
+        env = {k: v for k, v in os.environ.items() if k != "CUDA_MACE_TRACE"}
+        if value is not None:
+            env["CUDA_MACE_TRACE"] = value
+        res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120)
+        assert res.returncode == 0, res.stderr
+        seen[value] = int(res.stdout.split()[-1])
+    assert seen[None] == 0 and seen["0"] == 0
+    have_markers = any(os.path.exists(os.path.join(d, n)) for d in ("/opt/rocm/lib", "/opt/rocm/lib64")
+                       for n in ("librocprofiler-sdk-roctx.so", "libroctx64.so"))
+    assert seen["1"] == (1 if have_markers else 0)
