@@ -32,6 +32,7 @@ MEASURED_TRAFFIC = {
     "mp_backward_edge_kernel<128,true,true,false>": 6331300000,
     "mp_spline_forward_kernel<128,true>": 776800000,
     "mp_spline_backward_edge_kernel<128,true,true,true,false>": 818300000,
+    "linear_kernel<4,false>": 412100000,
 }
 
 
@@ -50,8 +51,8 @@ def mp_algorithmic_bytes(N, E, C):
 
 def isolated_ops(args, torch, cabi, make_system, reps=3):
     """A reference copy (reads and writes `copy_bytes` each) followed by the message-passing kernels (tabulated radial
-    weights, and fully fused from the edge vectors) on random operands at the benchmark shape; prints one line per
-    kernel with its average duration."""
+    weights, and fully fused from the edge vectors) and the channel-mixing linear on random operands at the benchmark
+    shape; prints one line per kernel with its average duration."""
     import numpy as np
 
     N, C = args.atoms, args.channels
@@ -70,6 +71,7 @@ def isolated_ops(args, torch, cabi, make_system, reps=3):
     knots = torch.tensor(kn, dtype=torch.float32, device="cuda")
     coeffs = torch.randn(255, 4, 4 * C, device="cuda", generator=g)
     fo = cabi.first_occurences(rcv, N)
+    WT = torch.randn(4, C, C, device="cuda", generator=g)
     copy_bytes = 1 << 30
     src = torch.empty(copy_bytes // 4, dtype=torch.float32, device="cuda").normal_(generator=g)
     dst = torch.empty_like(src)
@@ -83,6 +85,8 @@ def isolated_ops(args, torch, cabi, make_system, reps=3):
          lambda: cabi.mp_edge_forward(X, vec, knots, coeffs, float(h), 5.0, snd, fo, N)),
         ("mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb,
          lambda: cabi.mp_edge_backward(X, vec, knots, coeffs, float(h), 5.0, G, snd, fo, None, None, N, need_gX=False)),
+        # channel-mixing linear [N,16,C] x [C,C] per l: reads X and the four weight blocks, writes OUT
+        ("linear_kernel<%d,false>" % (C // 32), 4 * (32 * N * C + 4 * C * C), lambda: cabi.linear(G, WT)),
     ]
     print("# isolated ops at N=%d E=%d C=%d" % (N, E, C), flush=True)
     for name, nbytes, fn in cases:
@@ -243,7 +247,8 @@ def main():
             flops = 32 * N * C * C
             tf = flops / (t_lin * 1e-3) / 1e12
             others.append({"kernel": "linear_kernel<%d,false>" % (C // 32), "bound": "mfma", "achieved": round(tf, 1),
-                           "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4), "traffic": None,
+                           "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
+                           "traffic": MEASURED_TRAFFIC.get("linear_kernel<%d,false>" % (C // 32)) if default_workload else None,
                            "algorithmic_flops_per_launch": flops, "avg_launch_ms": round(t_lin, 4),
                            "launches_timed": len(events["linear"]),
                            "note": "fp32-equivalent flops of the [N,16,C] x [C,C] channel mixing against the fp32 matrix "
