@@ -250,6 +250,23 @@ class LinearContractionAutograd(torch.autograd.Function):
         return gX, None, None, None, None, None, None
 
 
+class ScalarLinearAutograd(torch.autograd.Function):
+    """Y = X . W for scalar features X [N, K] on the MFMA linear kernel (one component per node); W_T [N', K] and
+    W [K, N'] are the two orientations of the same weights (forward uses W_T, the backward W)."""
+
+    @staticmethod
+    @_traced("scalar_linear forward")
+    def forward(ctx, X, W_T, W):
+        ctx.save_for_backward(W)
+        return cabi.linear(X.contiguous(), W_T, scale=1.0)
+
+    @staticmethod
+    @_traced("scalar_linear backward")
+    def backward(ctx, grad):
+        (W,) = ctx.saved_tensors
+        return cabi.linear(grad.contiguous(), W, scale=1.0), None, None
+
+
 class ReadoutEnergyAutograd(torch.autograd.Function):
     """(h1, h2 fp32 [N, C]) -> (node energies fp64 [N], node_feats fp64 [N, 2C]): both readouts, scale and shift in one
     kernel; the derivative with respect to h2 is produced by the same pass and only scaled in the backward.  feats_rows
