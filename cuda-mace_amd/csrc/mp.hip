@@ -202,7 +202,7 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
             stv_stream(gp + 3 * C, x * q3);
           }
           if constexpr (WANT_GX) {
-            stv(gXe + e * C + V * cl, r0 * q0 + r1 * q1 + r2 * q2 + r3 * q3);
+            stv_stream(gXe + e * C + V * cl, r0 * q0 + r1 * q1 + r2 * q2 + r3 * q3);
           }
         }
       }
@@ -265,19 +265,20 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
   const int k1 = offsets[node + 1];
   vec acc = zerov<vec>();
   if (active) {
-    // four independent row gathers in flight per slot; the summation order stays fixed
+    // four independent row gathers in flight per slot; the summation order stays fixed.  Every row is read exactly
+    // once: streamed loads
     int k = k0 + slot;
     for (; k + 3 * K::EPW < k1; k += 4 * K::EPW) {
       const int ea = perm[k], eb = perm[k + K::EPW], ec = perm[k + 2 * K::EPW], ed = perm[k + 3 * K::EPW];
-      const vec va = static_cast<unsigned>(ea) < static_cast<uint64_t>(nedges) ? ldv<vec>(gXe + static_cast<int64_t>(ea) * C + V * cl) : zerov<vec>();
-      const vec vb = static_cast<unsigned>(eb) < static_cast<uint64_t>(nedges) ? ldv<vec>(gXe + static_cast<int64_t>(eb) * C + V * cl) : zerov<vec>();
-      const vec vc = static_cast<unsigned>(ec) < static_cast<uint64_t>(nedges) ? ldv<vec>(gXe + static_cast<int64_t>(ec) * C + V * cl) : zerov<vec>();
-      const vec vd = static_cast<unsigned>(ed) < static_cast<uint64_t>(nedges) ? ldv<vec>(gXe + static_cast<int64_t>(ed) * C + V * cl) : zerov<vec>();
+      const vec va = static_cast<unsigned>(ea) < static_cast<uint64_t>(nedges) ? ldv_stream<vec>(gXe + static_cast<int64_t>(ea) * C + V * cl) : zerov<vec>();
+      const vec vb = static_cast<unsigned>(eb) < static_cast<uint64_t>(nedges) ? ldv_stream<vec>(gXe + static_cast<int64_t>(eb) * C + V * cl) : zerov<vec>();
+      const vec vc = static_cast<unsigned>(ec) < static_cast<uint64_t>(nedges) ? ldv_stream<vec>(gXe + static_cast<int64_t>(ec) * C + V * cl) : zerov<vec>();
+      const vec vd = static_cast<unsigned>(ed) < static_cast<uint64_t>(nedges) ? ldv_stream<vec>(gXe + static_cast<int64_t>(ed) * C + V * cl) : zerov<vec>();
       acc += (va + vb) + (vc + vd);
     }
     for (; k < k1; k += K::EPW) {
       const int e = perm[k];
-      if (static_cast<unsigned>(e) < static_cast<uint64_t>(nedges)) acc += ldv<vec>(gXe + static_cast<int64_t>(e) * C + V * cl);
+      if (static_cast<unsigned>(e) < static_cast<uint64_t>(nedges)) acc += ldv_stream<vec>(gXe + static_cast<int64_t>(e) * C + V * cl);
     }
   }
 #pragma unroll
