@@ -102,7 +102,15 @@ def _dev(t: Optional[torch.Tensor], dtype: torch.dtype, name: str) -> Optional[i
     return t.data_ptr() if t.numel() > 0 else None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_get_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream() -> int:
+    """Handle of torch's current HIP stream on the current device (the raw query: this runs once per kernel launch and
+    the public accessor costs ten times as much on the host)."""
+    if _raw_stream is not None and _get_device is not None:
+        return _raw_stream(_get_device())
     return torch.cuda.current_stream().cuda_stream
 
 
