@@ -386,6 +386,7 @@ class OptimizedInvariantMACE(torch.nn.Module):
         batch, edge_index = data["batch"], data["edge_index"]
         n = pos.shape[0]
         bins = torch.floor((pos - pos.min(dim=0).values) / (0.5 * float(self.r_max))).long()
+        bins.clamp_(max=(1 << 16) - 1)  # 48 bits for the bin, the rest for the graph index: the key cannot overflow
         nb = int(bins.max()) + 1
         key = ((batch * nb + bins[:, 0]) * nb + bins[:, 1]) * nb + bins[:, 2]
         perm = torch.argsort(key, stable=True)
