@@ -67,21 +67,36 @@ def get_symmetric_displacement(positions, unit_shifts, cell, edge_index, num_gra
     return positions, shifts, displacement, cell
 
 
+_CONSTANTS: Dict[tuple, torch.Tensor] = {}
+
+
+def _constant(value: float, shape, dtype, device) -> torch.Tensor:
+    """A tensor filled with `value`, made once per (value, shape, dtype, device) and never written again: saves a fill
+    kernel per step for seeds and all-zero outputs."""
+    key = (float(value), tuple(shape), dtype, device)
+    hit = _CONSTANTS.get(key)
+    if hit is None:
+        hit = _CONSTANTS[key] = torch.full(tuple(shape), float(value), dtype=dtype, device=device)
+    return hit
+
+
 def get_outputs(energy, positions, displacement, cell, training=False, compute_force=True, compute_virials=False,
                 compute_stress=False):
-    """forces = -dE/dpositions; virials = -dE/ddisplacement; stress = -virials / volume."""
+    """forces = -dE/dpositions; virials = -dE/ddisplacement; stress = -virials / volume.  The backward pass is seeded with
+    -1 (a constant tensor kept per device), so that it delivers forces and virials themselves and no negation runs."""
     forces = virials = stress = None
-    grad_outputs = [torch.ones_like(energy)]
+    grad_outputs = [_constant(-1.0, energy.shape, energy.dtype, energy.device)]
     want_virials = compute_virials or compute_stress
     if compute_force and want_virials:
-        gp, gd = torch.autograd.grad([energy], [positions, displacement], grad_outputs=grad_outputs,
-                                     retain_graph=training, create_graph=training, allow_unused=True)
-        forces = -gp
-        virials = -gd if gd is not None else torch.zeros_like(displacement)
+        forces, virials = torch.autograd.grad([energy], [positions, displacement], grad_outputs=grad_outputs,
+                                              retain_graph=training, create_graph=training, allow_unused=True)
+        if virials is None:
+            virials = torch.zeros_like(displacement)
     elif compute_force:
-        (gp,) = torch.autograd.grad([energy], [positions], grad_outputs=grad_outputs, retain_graph=training,
-                                    create_graph=training, allow_unused=True)
-        forces = -gp if gp is not None else torch.zeros_like(positions)
+        (forces,) = torch.autograd.grad([energy], [positions], grad_outputs=grad_outputs, retain_graph=training,
+                                        create_graph=training, allow_unused=True)
+    if compute_force and forces is None:
+        forces = torch.zeros_like(positions)
     if compute_stress and virials is not None and cell is not None:
         cell3 = cell.view(-1, 3, 3)
         volume = torch.linalg.det(cell3).abs().view(-1, 1, 1)
@@ -440,7 +455,7 @@ class OptimizedInvariantMACE(torch.nn.Module):
         shifts = data["shifts"]
         cell = data.get("cell")
 
-        displacement = torch.zeros((num_graphs, 3, 3), dtype=positions.dtype, device=positions.device)
+        displacement = _constant(0.0, (num_graphs, 3, 3), positions.dtype, positions.device)  # replaced below when strained
         if compute_virials or compute_stress or compute_displacement:
             positions, shifts, displacement, cell = get_symmetric_displacement(
                 positions=positions, unit_shifts=data["unit_shifts"], cell=cell, edge_index=data["edge_index"],
@@ -457,7 +472,11 @@ class OptimizedInvariantMACE(torch.nn.Module):
 
         e0_per_head, node_feats_up = _cached_for(node_attrs, "_cm_species_only", self._weights_token, species_only)
         node_e0 = _select_head(e0_per_head, zero_heads if node_heads is None else node_heads)
-        e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
+        if num_graphs == 1 and node_heads is None:
+            # one graph: the sum of the atomic reference energies is a function of the species tensor alone, too
+            e0 = _cached_for(node_attrs, "_cm_e0_sum", self._weights_token, lambda: node_e0.sum(dim=0, keepdim=True))
+        else:
+            e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
         node_feats = None
 
         # index structures shared by both layers, cached on the caller's tensors so that they are rebuilt only when
