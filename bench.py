@@ -233,6 +233,13 @@ def main():
                               "come from the 2 MB spline table in L2 (16 loads of 16 B per lane and edge, texture-address "
                               "units ~80% busy): bounded by L1 delivery, not HBM; see roofline_other_kernels for the "
                               "HBM-bound message passing with tabulated R[E,4,C] and for the matrix-core linear",
+                         binding_resource={
+                             "resource": "vector-memory (L1) delivery: 17 loads of 16 B per lane and edge",
+                             "bytes": 68 * E * C, "achieved_GB/s": round(68 * E * C / (t_fwd * 1e-3) / 1e9, 1),
+                             "peak_GB/s": round(256 * 64 * 2.4, 1) * 1.0,
+                             "frac": round(68 * E * C / (t_fwd * 1e-3) / 1e9 / (256 * 64 * 2.4), 4),
+                             "meaning": "bytes the kernel pulls through the per-CU vector-memory path (coefficient table in "
+                                        "L2, sender rows) against 256 CUs x 64 B/clk x 2.4 GHz"},
                          unfused_equivalent={
                              "bytes": fwd_b + sh_f + spline_f,
                              "GB/s": round((fwd_b + sh_f + spline_f) / (t_fwd * 1e-3) / 1e9, 1),
