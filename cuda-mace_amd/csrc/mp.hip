@@ -59,7 +59,7 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
     const float *__restrict__ X, const float *__restrict__ Y, const float *__restrict__ R,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes,
     int64_t nedges, float *__restrict__ out) {
-  using K = Cfg<C>;
+  using K = Cfg<C, true>;
   using vec = typename K::vec;
   constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
@@ -87,13 +87,13 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
       for (int j = slot; j < cnt; j += K::EPW) {
         const int64_t e = base + j;
         const int s = sS[j];
-        const float *rp = R + e * (4 * C) + V * cl;
-        vec r0 = ldv_stream<vec>(rp);
-        vec r1 = ldv_stream<vec>(rp + C);
-        vec r2 = ldv_stream<vec>(rp + 2 * C);
-        vec r3 = ldv_stream<vec>(rp + 3 * C);
+        const float *rp = R + e * (4 * C) + K::off(cl);
+        vec r0 = K::ld_stream(rp);
+        vec r1 = K::ld_stream(rp + C);
+        vec r2 = K::ld_stream(rp + 2 * C);
+        vec r3 = K::ld_stream(rp + 3 * C);
         vec x = zerov<vec>();
-        if (static_cast<unsigned>(s) < static_cast<unsigned>(nnodes)) x = ldv<vec>(X + static_cast<int64_t>(s) * C + V * cl);
+        if (static_cast<unsigned>(s) < static_cast<unsigned>(nnodes)) x = K::ld(X + static_cast<int64_t>(s) * C + K::off(cl));
         const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
         const f4 ya = yp[0], yb = yp[1], yc = yp[2], yd = yp[3];
         const vec t0 = x * r0, t1 = x * r1, t2 = x * r2, t3 = x * r3;
@@ -125,9 +125,9 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
   }
   if (slot == 0 && active) {
     // streamed out (non-temporal): measured 5 % faster than regular stores, which compete with the R stream for L2
-    float *op = out + static_cast<int64_t>(node) * (16 * C) + V * cl;
+    float *op = out + static_cast<int64_t>(node) * (16 * C) + K::off(cl);
 #pragma unroll
-    for (int m = 0; m < 16; ++m) stv_stream(op + m * C, acc[m]);
+    for (int m = 0; m < 16; ++m) K::st_stream(op + m * C, acc[m]);
   }
 }
 
@@ -158,9 +158,9 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
 
   vec g[16];
   {
-    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + V * cl;
+    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + K::off(cl);
 #pragma unroll
-    for (int m = 0; m < 16; ++m) g[m] = active ? ldv<vec>(gp + m * C) : zerov<vec>();
+    for (int m = 0; m < 16; ++m) g[m] = active ? K::ld(gp + m * C) : zerov<vec>();
   }
   // which m this lane ends up holding after slot_reduce16
   const int myrev = ((cl & 1) << 3) | ((cl & 2) << 1) | ((cl & 4) >> 1) | ((cl & 8) >> 3);
@@ -176,12 +176,12 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
       const int s = sS[j];
       vec r0 = zerov<vec>(), r1 = zerov<vec>(), r2 = zerov<vec>(), r3 = zerov<vec>(), x = zerov<vec>();
       if (active) {
-        const float *rp = R + e * (4 * C) + V * cl;
-        r0 = ldv_stream<vec>(rp);
-        r1 = ldv_stream<vec>(rp + C);
-        r2 = ldv_stream<vec>(rp + 2 * C);
-        r3 = ldv_stream<vec>(rp + 3 * C);
-        if (static_cast<unsigned>(s) < static_cast<unsigned>(nnodes)) x = ldv<vec>(X + static_cast<int64_t>(s) * C + V * cl);
+        const float *rp = R + e * (4 * C) + K::off(cl);
+        r0 = K::ld_stream(rp);
+        r1 = K::ld_stream(rp + C);
+        r2 = K::ld_stream(rp + 2 * C);
+        r3 = K::ld_stream(rp + 3 * C);
+        if (static_cast<unsigned>(s) < static_cast<unsigned>(nnodes)) x = K::ld(X + static_cast<int64_t>(s) * C + K::off(cl));
       }
       const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
       const f4 ya = yp[0], yb = yp[1], yc = yp[2], yd = yp[3];
@@ -195,14 +195,14 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
                       yd.z * g[14] + yd.w * g[15];
         if (active) {
           if constexpr (WANT_GR) {
-            float *gp = gR + e * (4 * C) + V * cl;
-            stv_stream(gp, x * q0);
-            stv_stream(gp + C, x * q1);
-            stv_stream(gp + 2 * C, x * q2);
-            stv_stream(gp + 3 * C, x * q3);
+            float *gp = gR + e * (4 * C) + K::off(cl);
+            K::st_stream(gp, x * q0);
+            K::st_stream(gp + C, x * q1);
+            K::st_stream(gp + 2 * C, x * q2);
+            K::st_stream(gp + 3 * C, x * q3);
           }
           if constexpr (WANT_GX) {
-            stv_stream(gXe + e * C + V * cl, r0 * q0 + r1 * q1 + r2 * q2 + r3 * q3);
+            K::st_stream(gXe + e * C + K::off(cl), r0 * q0 + r1 * q1 + r2 * q2 + r3 * q3);
           }
         }
       }
@@ -270,20 +270,20 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
     int k = k0 + slot;
     for (; k + 3 * K::EPW < k1; k += 4 * K::EPW) {
       const int ea = perm[k], eb = perm[k + K::EPW], ec = perm[k + 2 * K::EPW], ed = perm[k + 3 * K::EPW];
-      const vec va = static_cast<unsigned>(ea) < static_cast<uint64_t>(nedges) ? ldv_stream<vec>(gXe + static_cast<int64_t>(ea) * C + V * cl) : zerov<vec>();
-      const vec vb = static_cast<unsigned>(eb) < static_cast<uint64_t>(nedges) ? ldv_stream<vec>(gXe + static_cast<int64_t>(eb) * C + V * cl) : zerov<vec>();
-      const vec vc = static_cast<unsigned>(ec) < static_cast<uint64_t>(nedges) ? ldv_stream<vec>(gXe + static_cast<int64_t>(ec) * C + V * cl) : zerov<vec>();
-      const vec vd = static_cast<unsigned>(ed) < static_cast<uint64_t>(nedges) ? ldv_stream<vec>(gXe + static_cast<int64_t>(ed) * C + V * cl) : zerov<vec>();
+      const vec va = static_cast<unsigned>(ea) < static_cast<uint64_t>(nedges) ? K::ld_stream(gXe + static_cast<int64_t>(ea) * C + K::off(cl)) : zerov<vec>();
+      const vec vb = static_cast<unsigned>(eb) < static_cast<uint64_t>(nedges) ? K::ld_stream(gXe + static_cast<int64_t>(eb) * C + K::off(cl)) : zerov<vec>();
+      const vec vc = static_cast<unsigned>(ec) < static_cast<uint64_t>(nedges) ? K::ld_stream(gXe + static_cast<int64_t>(ec) * C + K::off(cl)) : zerov<vec>();
+      const vec vd = static_cast<unsigned>(ed) < static_cast<uint64_t>(nedges) ? K::ld_stream(gXe + static_cast<int64_t>(ed) * C + K::off(cl)) : zerov<vec>();
       acc += (va + vb) + (vc + vd);
     }
     for (; k < k1; k += K::EPW) {
       const int e = perm[k];
-      if (static_cast<unsigned>(e) < static_cast<uint64_t>(nedges)) acc += ldv_stream<vec>(gXe + static_cast<int64_t>(e) * C + V * cl);
+      if (static_cast<unsigned>(e) < static_cast<uint64_t>(nedges)) acc += K::ld_stream(gXe + static_cast<int64_t>(e) * C + K::off(cl));
     }
   }
 #pragma unroll
   for (int off = kWave / 2; off >= K::SW; off >>= 1) acc += shfl_downv(acc, off);
-  if (slot == 0 && active) stv(gX + static_cast<int64_t>(node) * C + V * cl, acc);
+  if (slot == 0 && active) K::st(gX + static_cast<int64_t>(node) * C + K::off(cl), acc);
 }
 
 template <int C>

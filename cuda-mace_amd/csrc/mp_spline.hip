@@ -113,7 +113,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
                                                                  const int32_t *__restrict__ sender,
                                                                  const int32_t *__restrict__ first_occ, int nnodes,
                                                                  int64_t nedges, float *__restrict__ out) {
-  using K = Cfg<C>;
+  using K = Cfg<C, true>;
   using vec = typename K::vec;
   constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
         const int s = sS[j];
         const int idx = sIdx[j];
         const float xr = sXr[j];
-        const vec x = ldv<vec>(X + (static_cast<unsigned>(s) * C + unsigned(V) * cl));
+        const vec x = K::ld(X + (static_cast<unsigned>(s) * C + unsigned(K::off(cl))));
         float y[16];
         {
           const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
@@ -157,15 +157,15 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
             y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
           }
         }
-        const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(V) * cl;  // 32-bit offset from the uniform table base
+        const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(K::off(cl));  // 32-bit offset from the uniform table base
         const float *__restrict__ tab = sp.coeffs;
         auto per_l = [&](auto lc) {
           constexpr int L = decltype(lc)::value;
           // addressed from the middle of the interval's 16C-float row: all 16 pieces lie within +-8C floats of it, which
           // up to C = 128 fits the signed immediate offset of a load, so one address serves them all
           const float *mid = tab + (co + 8 * C);
-          const vec a = ldv<vec>(mid + (L * C - 8 * C)), b = ldv<vec>(mid + (L * C - 4 * C)), c = ldv<vec>(mid + L * C),
-                    d = ldv<vec>(mid + (L * C + 4 * C));
+          const vec a = K::ld(mid + (L * C - 8 * C)), b = K::ld(mid + (L * C - 4 * C)), c = K::ld(mid + L * C),
+                    d = K::ld(mid + (L * C + 4 * C));
           const vec t = x * (a + xr * (b + xr * (c + xr * d)));
 #pragma unroll
           for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) acc[m] += y[m] * t;
@@ -184,9 +184,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_k
     for (int m = 0; m < 16; ++m) acc[m] += shfl_downv(acc[m], off);
   }
   if (slot == 0 && active) {
-    float *op = out + static_cast<int64_t>(node) * (16 * C) + V * cl;
+    float *op = out + static_cast<int64_t>(node) * (16 * C) + K::off(cl);
 #pragma unroll
-    for (int m = 0; m < 16; ++m) stv(op + m * C, acc[m]);
+    for (int m = 0; m < 16; ++m) K::st(op + m * C, acc[m]);
   }
 }
 
@@ -221,9 +221,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
 
   vec g[16];
   {
-    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + V * cl;
+    const float *gp = G + static_cast<int64_t>(node) * (16 * C) + K::off(cl);
 #pragma unroll
-    for (int m = 0; m < 16; ++m) g[m] = active ? ldv_stream<vec>(gp + m * C) : zerov<vec>();  // read once
+    for (int m = 0; m < 16; ++m) g[m] = active ? K::ld_stream(gp + m * C) : zerov<vec>();  // read once
   }
 
   for (int base = e0; base < e1; base += kChunk) {
@@ -244,18 +244,18 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
       const int s = sS[j];
       const int idx = sIdx[j];
       xr = sXr[j];
-      x = ldv<vec>(X + (static_cast<unsigned>(s) * C + unsigned(V) * cla));
-      const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(V) * cla;
+      x = K::ld(X + (static_cast<unsigned>(s) * C + unsigned(K::off(cla))));
+      const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(K::off(cla));
       const float *__restrict__ tab = sp.coeffs;
 #pragma unroll
       for (int L = 0; L < 4; ++L) {
         // addressed from the middle of the interval's 16C-float row (offsets within +-8C floats: one address and
         // immediate offsets, up to C = 128)
         const float *mid = tab + (co + 8 * C);
-        ca[L] = ldv<vec>(mid + (L * C - 8 * C));
-        cb[L] = ldv<vec>(mid + (L * C - 4 * C));
-        cc[L] = ldv<vec>(mid + L * C);
-        cd[L] = ldv<vec>(mid + (L * C + 4 * C));
+        ca[L] = K::ld(mid + (L * C - 8 * C));
+        cb[L] = K::ld(mid + (L * C - 4 * C));
+        cc[L] = K::ld(mid + L * C);
+        cd[L] = K::ld(mid + (L * C + 4 * C));
       }
     };
     if (slot < nlive) fetch(slot);
@@ -299,7 +299,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
 
       if constexpr (WANT_GX) {
         // streamed out: 666 MB at the headline size, read once by the sender pass (measured 2 % on the whole step)
-        if (active) stv_stream(gXe + static_cast<int64_t>(base + sOrig[j]) * C + V * cl, gxe);
+        if (active) K::st_stream(gXe + static_cast<int64_t>(base + sOrig[j]) * C + K::off(cl), gxe);
       }
       if constexpr (WANT_GR) {
         const float tot = slot_sum<K::SW>(grv);
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
     if constexpr (WANT_GX) {
       // rows of edges that are not live: zero, the sender pass sums every row
       for (int k = slot; k < cnt; k += K::EPW)
-        if (!((live_mask >> k) & 1ull) && active) stv(gXe + static_cast<int64_t>(base + k) * C + V * cl, zerov<vec>());
+        if (!((live_mask >> k) & 1ull) && active) K::st(gXe + static_cast<int64_t>(base + k) * C + K::off(cl), zerov<vec>());
     }
     if constexpr (WANT_GY || WANT_GR) {
       __syncthreads();
