@@ -80,8 +80,29 @@ struct VecOf<3> {
   using type = f3;
 };
 
+// Five- and seven-wide variants for 160 and 224 channels on 32 lanes (strided channel ownership only: there is no
+// 20- or 28-byte access).
+typedef float f5 __attribute__((ext_vector_type(5)));
+typedef float f7 __attribute__((ext_vector_type(7)));
+template <>
+struct VecOf<5> {
+  using type = f5;
+};
+template <>
+struct VecOf<7> {
+  using type = f7;
+};
+
 template <class T>
 __device__ __forceinline__ T zerov();
+template <>
+__device__ __forceinline__ f5 zerov<f5>() {
+  return f5{0.f, 0.f, 0.f, 0.f, 0.f};
+}
+template <>
+__device__ __forceinline__ f7 zerov<f7>() {
+  return f7{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+}
 template <>
 __device__ __forceinline__ f4 zerov<f4>() {
   return zero4();
@@ -139,6 +160,18 @@ __device__ __forceinline__ f4 shfl_down4(f4 v, int delta) {
 __device__ __forceinline__ f4 shfl_downv(f4 v, int delta) { return shfl_down4(v, delta); }
 __device__ __forceinline__ f3 shfl_downv(f3 v, int delta) {
   return f3{__shfl_down(v.x, delta), __shfl_down(v.y, delta), __shfl_down(v.z, delta)};
+}
+__device__ __forceinline__ f5 shfl_downv(f5 v, int delta) {
+  f5 r;
+#pragma unroll
+  for (int i = 0; i < 5; ++i) r[i] = __shfl_down(v[i], delta);
+  return r;
+}
+__device__ __forceinline__ f7 shfl_downv(f7 v, int delta) {
+  f7 r;
+#pragma unroll
+  for (int i = 0; i < 7; ++i) r[i] = __shfl_down(v[i], delta);
+  return r;
 }
 
 }  // namespace cm

@@ -17,8 +17,9 @@ constexpr int pow2ceil(int v) {
 template <int C, bool STRIDED = false>
 struct Cfg {
   // channels per lane: four (one 16-byte access per row), except where three fill the lanes exactly (96 -> 32 lanes,
-  // 192 -> 64 lanes) and four would leave a quarter of them idle
-  static constexpr int V = (C == 96 || C == 192) ? 3 : 4;
+  // 192 -> 64 lanes) and four would leave a quarter of them idle; kernels that own strided channels (see below) also
+  // run 160 and 224 channels on 32 full lanes, five and seven channels each
+  static constexpr int V = (C == 96 || C == 192) ? 3 : (STRIDED && C == 160) ? 5 : (STRIDED && C == 224) ? 7 : 4;
   static constexpr int LPE = C / V;          // lanes that carry one edge
   static constexpr int SW = pow2ceil(LPE);   // slot width in lanes (power of two)
   static constexpr int EPW = kWave / SW;     // edges in flight per wave
@@ -26,43 +27,49 @@ struct Cfg {
   static_assert(C % 32 == 0 && C >= 32 && C <= 256 && C % V == 0, "channel count");
 
   // Which channels a lane owns.  Contiguous: V cl .. V cl + V - 1 (one 16-byte access per row for V = 4, a 12-byte one
-  // for V = 3).  STRIDED (V = 3 only): cl, cl + LPE, cl + 2 LPE, so that each of the three dword accesses of a wave
+  // for V = 3).  STRIDED (V != 4): cl, cl + LPE, cl + 2 LPE, ..., so that each of the V dword accesses of a wave
   // covers a contiguous run of the row: a 12-byte access per lane costs the vector-memory path as much as a 16-byte
   // one, which the kernels that are bound by that path (the forward ones) feel (measured 15 % at 96 and 192 channels),
   // while the backward kernels, bound by instruction issue, are 3 % faster with the single wider access.  Rows in memory
   // are plain channel order either way, so every kernel chooses for itself.  off(cl) is the first channel of lane cl,
   // ES the distance between the lane's channels.
-  static constexpr bool kStrided = STRIDED && V == 3;
+  static constexpr bool kStrided = STRIDED && V != 4;
   static constexpr int ES = kStrided ? LPE : 1;
   __device__ static __forceinline__ int off(int cl) { return kStrided ? cl : V * cl; }
   __device__ static __forceinline__ vec ld(const float *p) {
-    if constexpr (V == 3)
-      return f3{p[0], p[ES], p[2 * ES]};
-    else
+    if constexpr (V == 4) {
       return ld4(p);
+    } else {
+      vec r;
+#pragma unroll
+      for (int i = 0; i < V; ++i) r[i] = p[i * ES];
+      return r;
+    }
   }
   __device__ static __forceinline__ vec ld_stream(const float *p) {
-    if constexpr (V == 3)
-      return f3{__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + ES), __builtin_nontemporal_load(p + 2 * ES)};
-    else
+    if constexpr (V == 4) {
       return ld4_stream(p);
+    } else {
+      vec r;
+#pragma unroll
+      for (int i = 0; i < V; ++i) r[i] = __builtin_nontemporal_load(p + i * ES);
+      return r;
+    }
   }
   __device__ static __forceinline__ void st(float *p, vec v) {
-    if constexpr (V == 3) {
-      p[0] = v.x;
-      p[ES] = v.y;
-      p[2 * ES] = v.z;
-    } else {
+    if constexpr (V == 4) {
       st4(p, v);
+    } else {
+#pragma unroll
+      for (int i = 0; i < V; ++i) p[i * ES] = v[i];
     }
   }
   __device__ static __forceinline__ void st_stream(float *p, vec v) {
-    if constexpr (V == 3) {
-      __builtin_nontemporal_store(v.x, p);
-      __builtin_nontemporal_store(v.y, p + ES);
-      __builtin_nontemporal_store(v.z, p + 2 * ES);
-    } else {
+    if constexpr (V == 4) {
       st4_stream(p, v);
+    } else {
+#pragma unroll
+      for (int i = 0; i < V; ++i) __builtin_nontemporal_store(v[i], p + i * ES);
     }
   }
 };

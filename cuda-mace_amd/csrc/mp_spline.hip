@@ -108,7 +108,7 @@ struct MRange {
 // forward
 // -----------------------------------------------------------------------------------------------
 template <int C, bool FROM_VEC>
-__global__ __launch_bounds__(kWave, CM_FUSED_FWD_WAVES) void mp_spline_forward_kernel(const float *__restrict__ X,
+__global__ __launch_bounds__(kWave, (Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVES)) void mp_spline_forward_kernel(const float *__restrict__ X,
                                                                  const float *__restrict__ Y, Spline sp,
                                                                  const int32_t *__restrict__ sender,
                                                                  const int32_t *__restrict__ first_occ, int nnodes,
