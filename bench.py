@@ -123,7 +123,8 @@ def main():
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU; the hot path has no multi-GPU part (see DESIGN.md, sharding note). "
+        print("bench.py: this build runs on ONE GPU; the hot path has no multi-GPU part (it would shard by receiver node range "
+              "with one halo exchange per layer). "
               "Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
