@@ -61,7 +61,6 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
     int64_t nedges, float *__restrict__ out) {
   using K = Cfg<C, true>;
   using vec = typename K::vec;
-  constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
 
@@ -142,7 +141,6 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
     float *__restrict__ gR, float *__restrict__ gXe) {
   using K = Cfg<C>;
   using vec = typename K::vec;
-  constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
   __shared__ float sGY[16 * kChunk];  // [m][edge]
@@ -255,7 +253,6 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
     const int32_t *__restrict__ offsets, int nnodes, int64_t nedges, float *__restrict__ gX) {
   using K = Cfg<C>;
   using vec = typename K::vec;
-  constexpr int V = K::V;
   const int node = blockIdx.x;
   const int lane = threadIdx.x;
   const int slot = lane / K::SW;

@@ -115,7 +115,6 @@ __global__ __launch_bounds__(kWave, (Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVE
                                                                  int64_t nedges, float *__restrict__ out) {
   using K = Cfg<C, true>;
   using vec = typename K::vec;
-  constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
   __shared__ int sIdx[kChunk];
@@ -200,7 +199,6 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
     float *__restrict__ gY, float *__restrict__ g_r, float *__restrict__ gXe) {
   using K = Cfg<C>;
   using vec = typename K::vec;
-  constexpr int V = K::V;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
   __shared__ int sS[kChunk];
   __shared__ int sIdx[kChunk];
