@@ -160,9 +160,6 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
 #pragma unroll
     for (int m = 0; m < 16; ++m) g[m] = active ? K::ld(gp + m * C) : zerov<vec>();
   }
-  // which m this lane ends up holding after slot_reduce16
-  const int myrev = ((cl & 1) << 3) | ((cl & 2) << 1) | ((cl & 4) >> 1) | ((cl & 8) >> 3);
-
   for (int base = e0; base < e1; base += kChunk) {
     const int cnt = min(kChunk, e1 - base);
     __syncthreads();
@@ -224,13 +221,7 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
         p[14] = dotv(g[14], t3);
         p[15] = dotv(g[15], t3);
         slot_reduce16<K::SW>(p, cl);
-        if constexpr (K::SW >= 16) {
-          if (cl < 16) sGY[myrev * kChunk + j] = p[0];
-        } else {
-          const int m0 = (((cl & 1) << 2) | (cl & 2) | ((cl & 4) >> 2)) * 2;
-          sGY[m0 * kChunk + j] = p[0];
-          sGY[(m0 + 1) * kChunk + j] = p[1];
-        }
+        store_reduced16<K::SW>(p, cl, j, sGY);
       }
     }
     if constexpr (WANT_GY) {

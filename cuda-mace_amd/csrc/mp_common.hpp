@@ -102,14 +102,72 @@ __device__ __forceinline__ float dpp_move(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
 }
 
-// Sums p[m] over the SW lanes of a slot.  Butterfly with halving: after the exchange over lane
-// bit b each lane keeps half of its values, so 16 values cost 8+4+2+1 exchanges instead of 16*4.
-// The 12 exchanges over lane bits 0 and 1 stay inside a quad and go through DPP; the rest through ds_bpermute.
-// Returns, in every lane, the total for m = bitrev4(cl & 15) (SW >= 16), or for SW == 8 the two
-// totals m = bitrev3(cl) * 2 + {0, 1} in p[0], p[1].
+// Sums p[m] over the SW lanes of a slot.  Butterfly with halving: after the exchange over one lane bit each lane keeps
+// half of its values, so 16 values cost 8+4+2+1 exchanges instead of 16*4.
+//
+// SW >= 32: the two widest stages run over lane bits 3 and 2 as DPP adds whose write is masked by bank (a bank is four
+// consecutive lanes of a row of 16, so those two bits select banks): "lanes with the bit clear take p[k] + partner's
+// p[k], lanes with the bit set take p[h+k] + partner's p[h+k]" is two instructions per pair and needs no select
+// (written as inline assembly because the masked form keeps the destination's other lanes, which the DPP builtin
+// cannot express; the s_nop covers the two wait states a DPP read needs after a VALU write of the same register).
+// The stage over lane bit 4 swaps rows of 16 lanes between the two registers of a pair (v_permlane16_swap) and adds;
+// lane bit 0 goes through a quad permutation with selects, and lane bit 1 (and bit 5 for 64-lane slots) is a plain
+// sum.  Every lane ends with the total for m = reduced_index16(cl) in p[0].
+//
+// SW == 16 / 8: the stages over lane bits 0 and 1 stay inside a quad and go through DPP; the rest through
+// ds_bpermute.  Result: m = bitrev4(cl) in p[0] (SW == 16), or the two totals m = bitrev3(cl) * 2 + {0, 1} in p[0], p[1].
 template <int SW>
 __device__ __forceinline__ void slot_reduce16(float (&p)[16], int cl) {
   static_assert(SW >= 8, "slot width");
+  if constexpr (SW >= 32) {
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_add_f32_dpp %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %1, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %2, %2, %2 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %3, %3, %3 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %4, %4, %4 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %5, %5, %5 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %6, %6, %6 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %7, %7, %7 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %0, %8, %8 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %1, %9, %9 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %2, %10, %10 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %3, %11, %11 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %4, %12, %12 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %5, %13, %13 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %6, %14, %14 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        "v_add_f32_dpp %7, %15, %15 row_ror:8 row_mask:0xf bank_mask:0xc\n\t"
+        // lane bit 2: lanes of banks 0 and 2 read four lanes up (rotate right by 12), banks 1 and 3 four lanes down
+        "v_add_f32_dpp %0, %0, %0 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %1, %1, %1 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %2, %2, %2 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %3, %3, %3 row_ror:12 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %0, %4, %4 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %1, %5, %5 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %2, %6, %6 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "v_add_f32_dpp %3, %7, %7 row_ror:4 row_mask:0xf bank_mask:0xa\n\t"
+        "s_nop 0"  // with the wait state the compiler adds after the block: two before a lane-crossing read of %3
+        : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3]), "+v"(p[4]), "+v"(p[5]), "+v"(p[6]), "+v"(p[7])
+        : "v"(p[8]), "v"(p[9]), "v"(p[10]), "v"(p[11]), "v"(p[12]), "v"(p[13]), "v"(p[14]), "v"(p[15]));
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      // first result: row 0 of p[k] over row 0 of p[2+k]; second: row 1 of p[k] over row 1 of p[2+k]
+      const auto sw = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, p[k]), __builtin_bit_cast(unsigned, p[2 + k]),
+                                                       false, false);
+      const unsigned first = sw[0], second = sw[1];  // element-wise copies first: a bit_cast straight from sw[1] reads sw[0]
+      p[k] = __uint_as_float(first) + __uint_as_float(second);
+    }
+    {
+      const bool hi = cl & 1;
+      const float keep = hi ? p[1] : p[0];
+      const float send = hi ? p[0] : p[1];
+      p[0] = keep + dpp_move<0xB1>(send);
+    }
+    p[0] += dpp_move<0x4E>(p[0]);
+    if constexpr (SW >= 64) p[0] += __shfl_xor(p[0], 32);
+    return;
+  }
   {
     const bool hi = cl & 1;
 #pragma unroll
@@ -143,8 +201,6 @@ __device__ __forceinline__ void slot_reduce16(float (&p)[16], int cl) {
     const float send = hi ? p[0] : p[1];
     p[0] = keep + __shfl_xor(send, 8);
   }
-  if constexpr (SW >= 32) p[0] += __shfl_xor(p[0], 16);
-  if constexpr (SW >= 64) p[0] += __shfl_xor(p[0], 32);
 }
 
 // Plain sum of one value over the SW lanes of a slot; every lane gets the total.  Inside a row of 16 lanes: quad sums,
@@ -165,16 +221,20 @@ __device__ __forceinline__ float slot_sum(float v) {
   return v;
 }
 
-// Which m a lane (position cl in its slot) holds after slot_reduce16, SW >= 16.
+// Which m a lane (position cl in its slot) holds after slot_reduce16.
+template <int SW>
 __device__ __forceinline__ int reduced_index16(int cl) {
+  if constexpr (SW >= 32) return (cl & 12) | ((cl >> 3) & 2) | (cl & 1);  // lane bits 3, 2, 4, 0
   return ((cl & 1) << 3) | ((cl & 2) << 1) | ((cl & 4) >> 1) | ((cl & 8) >> 3);
 }
 
 // Writes the reduced gY values of edge j into the LDS tile sGY[m][kChunk].
 template <int SW>
 __device__ __forceinline__ void store_reduced16(const float (&p)[16], int cl, int j, float *sGY) {
-  if constexpr (SW >= 16) {
-    if (cl < 16) sGY[reduced_index16(cl) * kChunk + j] = p[0];
+  if constexpr (SW >= 32) {
+    if ((cl & ~29) == 0) sGY[reduced_index16<SW>(cl) * kChunk + j] = p[0];  // one lane per m: lane bits 1 and 5 clear
+  } else if constexpr (SW == 16) {
+    sGY[reduced_index16<SW>(cl) * kChunk + j] = p[0];
   } else {
     const int m0 = (((cl & 1) << 2) | (cl & 2) | ((cl & 4) >> 2)) * 2;
     sGY[m0 * kChunk + j] = p[0];

@@ -236,13 +236,17 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
     // The loop is rotated: the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
     // arithmetic of the current one, so they travel while the cross-lane reductions (a chain of dependent lane
     // exchanges) run.
-    vec x, ca[4], cb[4], cc[4], cd[4];
-    float xr;
-    auto fetch = [&](int j) {
+    // Two operand sets used in turn (the loop body is written out twice), so that the set being loaded is never copied
+    // into the set being consumed.
+    struct Operands {
+      vec x, ca[4], cb[4], cc[4], cd[4];
+      float xr;
+    };
+    auto fetch = [&](Operands &o, int j) {
       const int s = sS[j];
       const int idx = sIdx[j];
-      xr = sXr[j];
-      x = K::ld(X + (static_cast<unsigned>(s) * C + unsigned(K::off(cla))));
+      o.xr = sXr[j];
+      o.x = K::ld(X + (static_cast<unsigned>(s) * C + unsigned(K::off(cla))));
       const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(K::off(cla));
       const float *__restrict__ tab = sp.coeffs;
 #pragma unroll
@@ -250,14 +254,13 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
         // addressed from the middle of the interval's 16C-float row (offsets within +-8C floats: one address and
         // immediate offsets, up to C = 128)
         const float *mid = tab + (co + 8 * C);
-        ca[L] = K::ld(mid + (L * C - 8 * C));
-        cb[L] = K::ld(mid + (L * C - 4 * C));
-        cc[L] = K::ld(mid + L * C);
-        cd[L] = K::ld(mid + (L * C + 4 * C));
+        o.ca[L] = K::ld(mid + (L * C - 8 * C));
+        o.cb[L] = K::ld(mid + (L * C - 4 * C));
+        o.cc[L] = K::ld(mid + L * C);
+        o.cd[L] = K::ld(mid + (L * C + 4 * C));
       }
     };
-    if (slot < nlive) fetch(slot);
-    for (int j = slot; j < nlive; j += K::EPW) {
+    auto edge = [&](const Operands &o, int j, Operands &next) {
       float y[16];
       {
         const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
@@ -267,19 +270,20 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
           y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
         }
       }
+      const float xr = o.xr;
       const float xr2 = 2.f * xr, xr3 = 3.f * xr * xr;
       float p[16];
       vec gxe = zerov<vec>();
       vec grq = zerov<vec>();
       auto per_l = [&](auto lc) {
         constexpr int L = decltype(lc)::value;
-        const vec a = ca[L], b = cb[L], c = cc[L], d = cd[L];
+        const vec a = o.ca[L], b = o.cb[L], c = o.cc[L], d = o.cd[L];
         const vec rl = a + xr * (b + xr * (c + xr * d));
         vec q = zerov<vec>();
 #pragma unroll
         for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) q += y[m] * g[m];
         if constexpr (WANT_GY) {
-          const vec t = x * rl;
+          const vec t = o.x * rl;
 #pragma unroll
           for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) p[m] = dotv(g[m], t);
         }
@@ -291,14 +295,18 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
       per_l(std::integral_constant<int, 2>{});
       per_l(std::integral_constant<int, 3>{});
       float grv = 0.f;
-      if constexpr (WANT_GR) grv = hsumv(x * grq);
-
-      if (j + K::EPW < nlive) fetch(j + K::EPW);
+      if constexpr (WANT_GR) grv = hsumv(o.x * grq);
 
       if constexpr (WANT_GX) {
-        // streamed out: 666 MB at the headline size, read once by the sender pass (measured 2 % on the whole step)
+        // streamed out: 666 MB at the headline size, read once by the sender pass (measured 2 % on the whole step).
+        // Issued before the loads of the next edge: memory operations retire in issue order, so a store that is
+        // younger than those loads would have to be complete wherever the loop waits for all of them.
         if (active) K::st_stream(gXe + static_cast<int64_t>(base + sOrig[j]) * C + K::off(cl), gxe);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the instruction scheduler from sinking the store below the loads
       }
+      // Unconditional (the last edge of a slot fetches itself again): loads under a branch would make every later wait
+      // assume that they were not issued, i.e. wait for all but the oldest few of them.
+      fetch(next, j + K::EPW < nlive ? j + K::EPW : j);
       if constexpr (WANT_GR) {
         const float tot = slot_sum<K::SW>(grv);
         if (cl == 0) sGr[j] = tot;
@@ -307,6 +315,13 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
         slot_reduce16<K::SW>(p, cl);
         store_reduced16<K::SW>(p, cl, j, sGY);
       }
+    };
+    Operands opa, opb;
+    if (slot < nlive) fetch(opa, slot);
+    for (int j = slot; j < nlive; j += 2 * K::EPW) {
+      edge(opa, j, opb);
+      if (j + K::EPW >= nlive) break;
+      edge(opb, j + K::EPW, opa);
     }
     if constexpr (WANT_GX) {
       // rows of edges that are not live: zero, the sender pass sums every row
