@@ -23,6 +23,7 @@
 // its memory traffic allows.
 #include <algorithm>
 #include <cmath>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -220,11 +221,264 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
   }
 }
 
+// -----------------------------------------------------------------------------------------------
+// Variant with the feature rows on a ring of raw fp32 chunks in LDS, filled by direct global -> LDS loads.
+//
+// What bounds the kernel above is the amount of X that a workgroup has in flight: one 16 KB chunk, and only while it
+// multiplies the previous one.  Here the X chunks never pass through registers: each wave fetches the 32 rows it
+// multiplies itself, 16 bytes per lane, straight into a three-stage ring (global_load_lds_dwordx4), so one or two chunks
+// are in flight at all times; it splits its rows into the bf16 pieces as it feeds the matrix cores (every row is split
+// once, by its own wave, so this costs what the staging pass did, and the staged piece planes of X with their LDS
+// writes and re-reads go away).  The weights take the old road (registers -> pieces -> LDS planes), one chunk ahead.
+//
+// Vector-memory operations retire in issue order and one counter covers them all.  The compiler would wait for "all
+// of them" wherever it sees a load under a branch or a direct-to-LDS load that may alias a later LDS read, which
+// would drain the ring at every chunk.  So every vector-memory operation of the main loop is issued from inline assembly,
+// unseen by the compiler, in a fixed order, and waited for explicitly:
+//     iteration c:   barrier | wait: all but the 4 loads of X chunk c+1 | weights c -> planes | issue weights c+1
+//                    (and scales c+1), then X chunk c+2 | barrier | multiply chunk c
+// The assembly statements that wait also carry the loaded registers as read-write operands, which keeps every use
+// behind the wait.  M0 (the LDS address of a direct load) is written inside those statements; nothing else in this
+// kernel uses it.
+//
+// LDS layout of a ring stage: row r of the tile at r * 128 bytes, its eight 16-byte pieces at positions
+// piece ^ (r & 7), so that the 32 rows a wave reads at the same piece index fall on different banks (a direct load
+// writes lane i at base + 16 i: the layout is chosen through which piece each lane fetches).
+// -----------------------------------------------------------------------------------------------
+constexpr int kStages = 3;
+constexpr int kStageBytes = kTileNodes * kKC * 4;
+
+__device__ __forceinline__ void dma16(const float *src, unsigned lds_byte_address) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(src), "s"(lds_byte_address) : "memory");
+}
+__device__ __forceinline__ void ldg16(f4 &dst, const float *src) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src) : "memory");
+}
+__device__ __forceinline__ void after_wait(f4 &v) { asm volatile("" : "+v"(v)); }
+
+// two workgroups per compute unit (two waves per SIMD) wherever LDS allows it: 256 registers per lane
+template <int NT, bool SCALED>
+__global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_kernel(const float *__restrict__ X, const float *__restrict__ WT,
+                                                                    const int32_t *__restrict__ node_perm,
+                                                                    const int32_t *__restrict__ group_offsets, int nnodes,
+                                                                    int ngroups, int zero_last_group, int ncomp, int K,
+                                                                    float scale, const float *__restrict__ row_scale,
+                                                                    float *__restrict__ OUT) {
+  constexpr int NOUT = 32 * NT;
+  __shared__ __attribute__((aligned(16))) float sRaw[kStages * kTileNodes * kKC];
+  __shared__ __attribute__((aligned(16))) __bf16 sBp[3 * NOUT * kLdH];
+  __shared__ int sNode[kTileNodes];
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int m = blockIdx.x % ncomp;
+  const int l = ncomp == 1 ? 0 : l_of_m(m);
+  const int nblocks = ncomp == 1 ? 1 : 4;
+
+  int tile = blockIdx.x / ncomp;
+  int g = 0, pos0 = 0, gend = nnodes;
+  if (group_offsets) {
+    bool found = false;
+    for (g = 0; g < ngroups; ++g) {
+      const int lo = group_offsets[g], hi = group_offsets[g + 1];
+      const int tiles = (hi - lo + kTileNodes - 1) / kTileNodes;
+      if (tile < tiles) {
+        pos0 = lo + tile * kTileNodes;
+        gend = hi;
+        found = true;
+        break;
+      }
+      tile -= tiles;
+    }
+    if (!found) return;
+  } else {
+    pos0 = tile * kTileNodes;
+    if (pos0 >= nnodes) return;
+  }
+  const int nrows = min(kTileNodes, gend - pos0);
+
+  if (tid < kTileNodes) {
+    int node = -1;
+    if (tid < nrows) {
+      node = node_perm ? node_perm[pos0 + tid] : pos0 + tid;
+      if (static_cast<unsigned>(node) >= static_cast<unsigned>(nnodes)) node = -1;
+    }
+    sNode[tid] = node;
+  }
+  __syncthreads();
+
+  if (zero_last_group && g == ngroups - 1) {
+    for (int i = tid; i < kTileNodes * NOUT; i += kWaves * kWave) {
+      const int node = sNode[i / NOUT];
+      if (node >= 0) OUT[(static_cast<int64_t>(node) * ncomp + m) * NOUT + i % NOUT] = 0.f;
+    }
+    return;
+  }
+  const float *Wg = WT + (static_cast<int64_t>(g) * nblocks + l) * NOUT * K;  // [NOUT, K]
+
+  v16f acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+
+  // weights: staging map as in the kernel above (8 threads x 16 bytes per row of the chunk, 32 rows per pass)
+  constexpr int kTPR = kKC / 4;
+  constexpr int kRPP = kWaves * kWave / kTPR;
+  static_assert(kRPP == 32 && NOUT % kRPP == 0, "staging map");
+  const int srow = tid / kTPR;
+  const int scol = (tid % kTPR) * 4;
+  const float *wsrc = Wg + static_cast<int64_t>(srow) * K + scol;  // + 32 i K for pass i, + kc
+  // matrix-core operand map
+  const int mrow = lane % 32;
+  const int half = lane / 32;
+
+  // X: one direct load covers 8 rows x 128 bytes; a wave issues four per chunk, for its own 32 rows.  Rows beyond the
+  // tile fetch row 0 of X (their products are never stored).
+  const int drow = lane / 8;
+  const int dpiece = (lane & 7) ^ drow;
+  const float *xsrc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int node = sNode[32 * wave + 8 * i + drow];
+    xsrc[i] = X + (static_cast<int64_t>(node >= 0 ? node : 0) * ncomp + m) * K + 4 * dpiece;
+  }
+  const unsigned raw_base = static_cast<unsigned>(reinterpret_cast<uintptr_t>(sRaw)) + static_cast<unsigned>(wave) * (32 * kKC * 4);
+  auto issue_x = [&](int kc, int stage) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16(xsrc[i] + kc, raw_base + static_cast<unsigned>(stage) * kStageBytes + i * (8 * kKC * 4));
+  };
+  // the wave's own A fragments: 8 consecutive k of row 32 wave + mrow, i.e. pieces ks/4 + 2 half and the next one
+  const float *araw = sRaw + (32 * wave + mrow) * kKC;
+  const int swz = mrow & 7;
+
+  f4 pb[NT];
+  f4 sc[2][4];
+  const float *ssrc = nullptr;
+  if constexpr (SCALED) {
+    const int node = sNode[32 * wave + mrow];
+    ssrc = row_scale + static_cast<int64_t>(node >= 0 ? node : 0) * K + 8 * half;
+  }
+  auto issue_w = [&](int kc, auto par) {
+    constexpr int P = decltype(par)::value;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) ldg16(pb[i], wsrc + static_cast<int64_t>(kRPP * i) * K + kc);
+    if constexpr (SCALED) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) ldg16(sc[P][q], ssrc + kc + 16 * (q / 2) + 4 * (q % 2));
+    }
+  };
+
+  const int nch = K / kKC;
+  issue_w(0, std::integral_constant<int, 0>{});
+  issue_x(0, 0);
+  if (nch > 1) issue_x(kKC, 1);
+
+  auto iteration = [&](int c, int stage, auto par) {
+    constexpr int P = decltype(par)::value;
+    const int kc = c * kKC;
+    // every wave has finished multiplying chunk c - 1: the weight planes and ring stage (c + 2) % 3 are free
+    asm volatile("s_barrier" ::: "memory");
+    // weights (and scales) of chunk c and X chunk c have landed; the four loads of X chunk c + 1 may still be out
+    if (c + 1 < nch)
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < NT; ++i) after_wait(pb[i]);
+    if constexpr (SCALED) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) after_wait(sc[P][q]);
+    }
+#pragma unroll
+    for (int i = 0; i < NT; ++i) {
+      bf16x4 h, md, lw;
+      split3(pb[i], h, md, lw);
+      const int at = (kRPP * i + srow) * kLdH + scol;
+      *reinterpret_cast<bf16x4 *>(sBp + at) = h;
+      *reinterpret_cast<bf16x4 *>(sBp + NOUT * kLdH + at) = md;
+      *reinterpret_cast<bf16x4 *>(sBp + 2 * NOUT * kLdH + at) = lw;
+    }
+    if (c + 1 < nch) issue_w(kc + kKC, std::integral_constant<int, 1 - P>{});
+    if (c + 2 < nch) issue_x(kc + 2 * kKC, stage >= 1 ? stage - 1 : 2);  // (stage + 2) % 3
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // weight planes written
+
+    const float *ast = araw + stage * (kTileNodes * kKC);
+#pragma unroll
+    for (int ks = 0; ks < kKC; ks += 16) {
+      const int piece = ks / 4 + 2 * half;
+      f4 r0 = *reinterpret_cast<const f4 *>(ast + 4 * (piece ^ swz));
+      f4 r1 = *reinterpret_cast<const f4 *>(ast + 4 * ((piece + 1) ^ swz));
+      if constexpr (SCALED) {
+        r0 *= sc[P][2 * (ks / 16)];
+        r1 *= sc[P][2 * (ks / 16) + 1];
+      }
+      bf16x4 h0, m0, l0, h1, m1, l1;
+      split3(r0, h0, m0, l0);
+      split3(r1, h1, m1, l1);
+      bf16x8 a[3], b[NT][3];
+      a[0] = __builtin_shufflevector(h0, h1, 0, 1, 2, 3, 4, 5, 6, 7);
+      a[1] = __builtin_shufflevector(m0, m1, 0, 1, 2, 3, 4, 5, 6, 7);
+      a[2] = __builtin_shufflevector(l0, l1, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int p = 0; p < 3; ++p)
+          b[t][p] = *reinterpret_cast<const bf16x8 *>(sBp + p * NOUT * kLdH + (32 * t + mrow) * kLdH + ks + 8 * half);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], b[t][0], acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][2], acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[t][1], acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[t][0], acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][1], acc[t], 0, 0, 0);
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][0], acc[t], 0, 0, 0);
+    }
+  };
+  int stage = 0;
+  for (int c = 0; c < nch; c += 2) {
+    iteration(c, stage, std::integral_constant<int, 0>{});
+    stage = stage == 2 ? 0 : stage + 1;
+    if (c + 1 >= nch) break;
+    iteration(c + 1, stage, std::integral_constant<int, 1>{});
+    stage = stage == 2 ? 0 : stage + 1;
+  }
+
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
+    const int node = sNode[row];
+    if (node >= 0) {
+      float *op = OUT + (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+    }
+  }
+}
+
 template <int NT>
 int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
            int zero_last_group, int ncomp, int K, float scale, const float *row_scale, float *OUT, hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
   const dim3 grid(static_cast<unsigned>(tiles * ncomp)), block(kWaves * kWave);
+  // The ring variant wherever it runs two workgroups per compute unit or the plain one does not either (Nout up to 128,
+  // and 224 / 256), and K has more than one chunk to overlap; measured at 25 000 nodes: 108 vs 119-127 us at 128
+  // columns, 76 vs 80-83 at 96, equal at 64, 224 and 256, slower at 32 (one chunk), 160 and 192 (one workgroup per CU).
+  constexpr bool kRing = NT == 2 || NT == 3 || NT == 4 || NT >= 7;
+  if (kRing && K > kKC) {
+    if (row_scale)
+      hipLaunchKernelGGL((linear_ring_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                         zero_last_group, ncomp, K, scale, row_scale, OUT);
+    else
+      hipLaunchKernelGGL((linear_ring_kernel<NT, false>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                         zero_last_group, ncomp, K, scale, row_scale, OUT);
+    return check_launch("cm_linear");
+  }
   if (row_scale)
     hipLaunchKernelGGL((linear_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
                        zero_last_group, ncomp, K, scale, row_scale, OUT);
