@@ -280,12 +280,15 @@ class ReadoutEnergyAutograd(torch.autograd.Function):
         ctx.save_for_backward(w1, d2)
         ctx.scale = float(scale)
         ctx.mark_non_differentiable(feats)
+        ctx.set_materialize_grads(False)  # no [N, 2C] tensor of zeros is made for the gradient of feats in every backward
         return es, feats
 
     @staticmethod
     @_traced("readout backward")
     def backward(ctx, grad_es, _grad_feats):
         w1, d2 = ctx.saved_tensors
+        if grad_es is None:
+            return (None,) * 9
         g1, g2 = cabi.readout_backward(grad_es.contiguous(), w1, d2, ctx.scale, ctx.needs_input_grad[0], ctx.needs_input_grad[1])
         return g1, g2, None, None, None, None, None, None, None
 
