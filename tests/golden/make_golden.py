@@ -123,7 +123,7 @@ def ops_outputs(d):
 
 
 def model_case():
-    """BASELINE config 1: the 21-atom {H, C, N, O} cluster in an 8 A cube, 64 channels, weights from seed 0."""
+    """Benchmark configuration 1: the 21-atom {H, C, N, O} cluster in an 8 A cube, 64 channels, weights from seed 0."""
     from cuda_mace.models import SyntheticInvariantMACE
     from cuda_mace.utils.synthetic import make_system
 

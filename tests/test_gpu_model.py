@@ -1,7 +1,7 @@
 """End-to-end parity on the GPU: OptimizedInvariantMACE (fp32 HIP kernels, splined radial functions) against
 the fp64 CPU reference model on the same seeded weights and structures.
 
-Bar (BASELINE north_star): energy within 1e-5 relative, forces within 1e-4 eV/A max-abs.
+Bar: energy within 1e-5 relative, forces within 1e-4 eV/A max-abs.
 """
 import numpy as np
 import pytest
@@ -46,7 +46,7 @@ def _compare(params, model, data):
 
 
 def test_cluster_config1(cabi):
-    """BASELINE config 1: 21-atom non-periodic cluster in an 8 A cube, {H, C, N, O}, 64 channels."""
+    """Benchmark configuration 1: 21-atom non-periodic cluster in an 8 A cube, {H, C, N, O}, 64 channels."""
     _say("model c1: 21-atom cluster, C=64")
     data = make_system(21, 4, seed=0, density=None, cluster_box=8.0)
     params, model = _build(64, (1, 6, 7, 8), data, seed=0)
@@ -137,7 +137,7 @@ def test_batch_of_graphs(cabi):
 
 
 def test_config3_full_size_against_reference(cabi):
-    """BASELINE config 3 at its real size (5 000 atoms, 96 channels, 10 elements): energy and forces against the fp64
+    """Benchmark configuration 3 at its real size (5 000 atoms, 96 channels, 10 elements): energy and forces against the fp64
     reference evaluated in edge chunks."""
     _say("model c3: 5000-atom periodic box, C=96")
     data = make_system(5000, 10, seed=0, density=0.1)
@@ -152,7 +152,7 @@ def test_config3_full_size_against_reference(cabi):
 
 
 def test_config4_full_size_properties(cabi):
-    """BASELINE config 4 at its real size (25 000 atoms, 128 channels), where the fp64 reference is out of reach: forces
+    """Benchmark configuration 4 at its real size (25 000 atoms, 128 channels), where the fp64 reference is out of reach: forces
     sum to zero, two evaluations agree bit for bit, and rotating the whole periodic system (positions, cell, shifts)
     leaves the energy unchanged and rotates the forces."""
     _say("model c4: 25000-atom periodic box, C=128")
@@ -220,7 +220,7 @@ def test_spatial_relabelling_is_transparent(cabi):
 
 
 def test_config5_full_size_properties(cabi):
-    """BASELINE config 5 at its real size (100 000 atoms, 192 channels, 5.2 M edges; three channels per lane in the
+    """Benchmark configuration 5 at its real size (100 000 atoms, 192 channels, 5.2 M edges; three channels per lane in the
     message-passing kernels): forces sum to zero, two evaluations agree bit for bit, and moving every atom by the same
     vector (the edge vectors change only by rounding) leaves energy and forces unchanged."""
     _say("model c5: 100000-atom periodic box, C=192")

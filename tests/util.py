@@ -1,4 +1,4 @@
-"""Seeded synthetic inputs shared by the tests (shapes of BASELINE config 2 and smaller)."""
+"""Seeded synthetic inputs shared by the tests (shapes of benchmark configuration 2, the isolated message-passing op at 4096 nodes, and smaller)."""
 import numpy as np
 import torch
 
