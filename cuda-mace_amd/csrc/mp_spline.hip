@@ -56,46 +56,61 @@ __device__ __forceinline__ void locate(const Spline &sp, float re, int &idx, flo
   }
 }
 
-// Stages the chunk's LIVE edges -- those inside the cutoff whose sender index is valid -- densely, in their original
-// order: sender, Y (as [edge][16]), knot interval, offset inside it, and the position of the edge in the chunk.  Returns
-// their number (the same in every lane); my_live tells a lane whether the edge base + lane is one of them.  Edges
-// beyond the cutoff (a neighbour list with a skin has many) cost nothing after this point.  FROM_VEC: Y and the length
-// come from the edge vector; otherwise from the Y and r arrays.
-template <bool FROM_VEC>
+// Stages up to kChunk LIVE edges of a node -- those inside the cutoff whose sender index is valid -- densely, in their
+// original order: sender, Y (as [edge][16]), knot interval, offset inside it, and the position of the edge counted from
+// `first` (the value of `base` on entry).  Raw edges are read kChunk at a time until kChunk live ones are staged or the
+// node's edges are used up, so a neighbour list with a skin (a quarter of its pairs beyond the cutoff) fills the chunk
+// all the same, and the edges beyond the cutoff cost nothing after this point.  `base` advances past every raw edge that
+// was consumed; `dead(pass_base, consumed, live_mask, lane_is_dead)` is called once per pass for the consumed edges that
+// are not live (the backward writes their zeros there).  Returns the number of staged edges (the same in every lane).
+// FROM_VEC: Y and the length come from the edge vector; otherwise from the Y and r arrays.
+template <bool FROM_VEC, class DeadFn>
 __device__ __forceinline__ int stage_edges(const float *__restrict__ Y, const int32_t *__restrict__ sender, const Spline &sp,
-                                           int nnodes, int64_t nedges, int base, int cnt, int lane, float *sY, int *sS,
-                                           int *sIdx, float *sXr, int *sOrig, bool &my_live, unsigned long long &live_mask) {
-  int s = -1, idx = -1;
-  float x = 0.f;
-  float y[16];
+                                           int nnodes, int64_t nedges, int &base, int e1, int lane, float *sY, int *sS,
+                                           int *sIdx, float *sXr, int *sOrig, DeadFn dead) {
+  const int first = base;
+  int nlive = 0;
+  while (nlive < kChunk && base < e1) {
+    const int cnt = min(kChunk, e1 - base);
+    int s = -1, idx = -1;
+    float x = 0.f;
+    float y[16];
 #pragma unroll
-  for (int m = 0; m < 16; ++m) y[m] = 0.f;
-  if (lane < cnt) {
-    const int64_t e = base + lane;
-    s = sender[e];
-    if constexpr (FROM_VEC) {
-      const float v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
-      locate(sp, sqrtf(v0 * v0 + v1 * v1 + v2 * v2), idx, x);
-      sh::eval(sh::direction(v0, v1, v2), y);
-    } else {
-      locate(sp, sp.r[e], idx, x);
+    for (int m = 0; m < 16; ++m) y[m] = 0.f;
+    if (lane < cnt) {
+      const int64_t e = base + lane;
+      s = sender[e];
+      if constexpr (FROM_VEC) {
+        const float v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
+        locate(sp, sqrtf(v0 * v0 + v1 * v1 + v2 * v2), idx, x);
+        sh::eval(sh::direction(v0, v1, v2), y);
+      } else {
+        locate(sp, sp.r[e], idx, x);
 #pragma unroll
-      for (int m = 0; m < 16; ++m) y[m] = Y[m * nedges + e];
+        for (int m = 0; m < 16; ++m) y[m] = Y[m * nedges + e];
+      }
     }
-  }
-  my_live = lane < cnt && idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
-  live_mask = __ballot(my_live);
-  if (my_live) {
-    const int pos = __popcll(live_mask & ((1ull << lane) - 1ull));
-    sS[pos] = s;
-    sIdx[pos] = idx;
-    sXr[pos] = x;
-    sOrig[pos] = lane;
+    const bool live = lane < cnt && idx >= 0 && static_cast<unsigned>(s) < static_cast<unsigned>(nnodes);
+    const unsigned long long live_mask = __ballot(live);
+    const int pos = nlive + __popcll(live_mask & ((1ull << lane) - 1ull));
+    const int nlive_pass = __popcll(live_mask);
+    // raw edges consumed by this pass: all of them, or those up to the live edge that fills the last place
+    int consumed = cnt;
+    if (nlive + nlive_pass > kChunk) consumed = __ffsll(static_cast<long long>(__ballot(live && pos == kChunk - 1)));
+    if (live && pos < kChunk) {
+      sS[pos] = s;
+      sIdx[pos] = idx;
+      sXr[pos] = x;
+      sOrig[pos] = base - first + lane;
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-      *reinterpret_cast<f4 *>(sY + pos * 16 + 4 * q) = f4{y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]};
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<f4 *>(sY + pos * 16 + 4 * q) = f4{y[4 * q], y[4 * q + 1], y[4 * q + 2], y[4 * q + 3]};
+    }
+    dead(base, consumed, live_mask, lane < consumed && !live);
+    nlive = min(kChunk, nlive + nlive_pass);
+    base += consumed;
   }
-  return __popcll(live_mask);
+  return nlive;
 }
 
 template <int L>
@@ -133,13 +148,10 @@ __global__ __launch_bounds__(kWave, (Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVE
 #pragma unroll
   for (int m = 0; m < 16; ++m) acc[m] = zerov<vec>();
 
-  for (int base = e0; base < e1; base += kChunk) {
-    const int cnt = min(kChunk, e1 - base);
+  for (int base = e0; base < e1;) {
     __syncthreads();
-    bool my_live;
-    unsigned long long live_mask;
-    const int nlive = stage_edges<FROM_VEC>(Y, sender, sp, nnodes, nedges, base, cnt, lane, sY, sS, sIdx, sXr, sOrig, my_live,
-                                            live_mask);
+    const int nlive = stage_edges<FROM_VEC>(Y, sender, sp, nnodes, nedges, base, e1, lane, sY, sS, sIdx, sXr, sOrig,
+                                            [](int, int, unsigned long long, bool) {});
     __syncthreads();
     if (active) {
       for (int j = slot; j < nlive; j += K::EPW) {
@@ -224,13 +236,33 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
     for (int m = 0; m < 16; ++m) g[m] = active ? K::ld_stream(gp + m * C) : zerov<vec>();  // read once
   }
 
-  for (int base = e0; base < e1; base += kChunk) {
-    const int cnt = min(kChunk, e1 - base);
+  for (int cursor = e0; cursor < e1;) {
+    const int base = cursor;  // sOrig counts from here
     __syncthreads();
-    bool my_live;
-    unsigned long long live_mask;
-    const int nlive = stage_edges<FROM_VEC>(Y, sender, sp, nnodes, nedges, base, cnt, lane, sY, sS, sIdx, sXr, sOrig, my_live,
-                                            live_mask);
+    // consumed edges that are not live: their outputs are zeros (the sender pass sums every row of gXe)
+    auto dead = [&](int pass_base, int consumed, unsigned long long live_mask, bool lane_is_dead) {
+      if constexpr (WANT_GX) {
+        for (int k = slot; k < consumed; k += K::EPW)
+          if (!((live_mask >> k) & 1ull) && active) K::st(gXe + static_cast<int64_t>(pass_base + k) * C + K::off(cl), zerov<vec>());
+      }
+      if constexpr (WANT_GY || WANT_GR) {
+        if (lane_is_dead) {
+          const int64_t e = pass_base + lane;
+          if constexpr (FROM_VEC) {
+            gY[3 * e + 0] = 0.f;
+            gY[3 * e + 1] = 0.f;
+            gY[3 * e + 2] = 0.f;
+          } else {
+            if constexpr (WANT_GY) {
+#pragma unroll
+              for (int m = 0; m < 16; ++m) gY[m * nedges + e] = 0.f;
+            }
+            if constexpr (WANT_GR) g_r[e] = 0.f;
+          }
+        }
+      }
+    };
+    const int nlive = stage_edges<FROM_VEC>(Y, sender, sp, nnodes, nedges, cursor, e1, lane, sY, sS, sIdx, sXr, sOrig, dead);
     __syncthreads();
     // Every lane of a slot takes part in the reductions, so the loop bound is slot-uniform; only live edges are staged.
     // The loop is rotated: the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
@@ -323,28 +355,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
       if (j + K::EPW >= nlive) break;
       edge(opb, j + K::EPW, opa);
     }
-    if constexpr (WANT_GX) {
-      // rows of edges that are not live: zero, the sender pass sums every row
-      for (int k = slot; k < cnt; k += K::EPW)
-        if (!((live_mask >> k) & 1ull) && active) K::st(gXe + static_cast<int64_t>(base + k) * C + K::off(cl), zerov<vec>());
-    }
     if constexpr (WANT_GY || WANT_GR) {
       __syncthreads();
-      // lane k < nlive finishes the k-th live edge; lanes whose own edge is not live write its zeros
-      if (lane < cnt && !my_live) {
-        const int64_t e = base + lane;
-        if constexpr (FROM_VEC) {
-          gY[3 * e + 0] = 0.f;
-          gY[3 * e + 1] = 0.f;
-          gY[3 * e + 2] = 0.f;
-        } else {
-          if constexpr (WANT_GY) {
-#pragma unroll
-            for (int m = 0; m < 16; ++m) gY[m * nedges + e] = 0.f;
-          }
-          if constexpr (WANT_GR) g_r[e] = 0.f;
-        }
-      }
+      // lane k < nlive finishes the k-th staged edge
       if (lane < nlive) {
         const int64_t e = base + sOrig[lane];
         if constexpr (FROM_VEC) {

@@ -102,11 +102,14 @@ def test_mp_spline_forward_backward(cabi, case):
     assert no_x[0] is None and torch.equal(no_x[1], gY) and torch.equal(no_x[2], gr)
 
 
-def test_edges_beyond_cutoff_and_invalid_senders_cost_nothing_and_contribute_nothing(cabi):
+@pytest.mark.parametrize("degree", [70, 200])
+def test_edges_beyond_cutoff_and_invalid_senders_cost_nothing_and_contribute_nothing(cabi, degree):
     """A list with a wide skin (most edges beyond r_max) and a few out-of-range sender indices: those edges add nothing
-    to the output and get exactly zero gradients; the rest matches the oracle evaluated on the live edges alone."""
+    to the output and get exactly zero gradients; the rest matches the oracle evaluated on the live edges alone.  The
+    kernels stage 64 live edges at a time out of as many raw ones as that takes: 70 raw edges per node fill one chunk from
+    two reads, 200 make chunks that end in the middle of a read."""
     nnodes, C, seed = 90, 128, 11
-    snd, rcv = random_graph(nnodes, 70, seed)
+    snd, rcv = random_graph(nnodes, degree, seed)
     E = snd.numel()
     X, _, _, G = mp_inputs(nnodes, E, C, seed)
     g = torch.Generator().manual_seed(seed)
