@@ -60,7 +60,7 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
                                                                const int32_t *__restrict__ group_offsets, int nnodes,
                                                                int ngroups, int zero_last_group, int ncomp, int K,
                                                                float scale, const float *__restrict__ row_scale,
-                                                               float *__restrict__ OUT) {
+                                                               const float *residual, float *OUT) {
   constexpr int NOUT = 32 * NT;
   // three bf16 planes per operand: plane p of X at sAp + p * kTileNodes * kLdH, of the weights at sBp + p * NOUT * kLdH
   // (77 KB at Nout = 192, 92 KB at 256: beyond 64 KB, within the 160 KB of a gfx950 compute unit)
@@ -214,9 +214,16 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
     const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
     const int node = sNode[row];
     if (node >= 0) {
-      float *op = OUT + (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
+      const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
+      float *op = OUT + at;
+      if (residual) {  // may be OUT itself: every element is read and written by the same lane
+        const float *rp = residual + at;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+        for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale + rp[32 * t];
+      } else {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+      }
     }
   }
 }
@@ -263,7 +270,7 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
                                                                     const int32_t *__restrict__ group_offsets, int nnodes,
                                                                     int ngroups, int zero_last_group, int ncomp, int K,
                                                                     float scale, const float *__restrict__ row_scale,
-                                                                    float *__restrict__ OUT) {
+                                                                    const float *residual, float *OUT) {
   constexpr int NOUT = 32 * NT;
   __shared__ __attribute__((aligned(16))) float sRaw[kStages * kTileNodes * kKC];
   __shared__ __attribute__((aligned(16))) __bf16 sBp[3 * NOUT * kLdH];
@@ -454,16 +461,24 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
     const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
     const int node = sNode[row];
     if (node >= 0) {
-      float *op = OUT + (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
+      const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
+      float *op = OUT + at;
+      if (residual) {  // may be OUT itself: every element is read and written by the same lane
+        const float *rp = residual + at;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+        for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale + rp[32 * t];
+      } else {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+      }
     }
   }
 }
 
 template <int NT>
 int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
-           int zero_last_group, int ncomp, int K, float scale, const float *row_scale, float *OUT, hipStream_t st) {
+           int zero_last_group, int ncomp, int K, float scale, const float *row_scale, const float *residual, float *OUT,
+           hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
   const dim3 grid(static_cast<unsigned>(tiles * ncomp)), block(kWaves * kWave);
   // The ring variant wherever it runs two workgroups per compute unit or the plain one does not either (Nout up to 128,
@@ -473,18 +488,18 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
   if (kRing && K > kKC) {
     if (row_scale)
       hipLaunchKernelGGL((linear_ring_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
-                         zero_last_group, ncomp, K, scale, row_scale, OUT);
+                         zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
     else
       hipLaunchKernelGGL((linear_ring_kernel<NT, false>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
-                         zero_last_group, ncomp, K, scale, row_scale, OUT);
+                         zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
     return check_launch("cm_linear");
   }
   if (row_scale)
     hipLaunchKernelGGL((linear_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
-                       zero_last_group, ncomp, K, scale, row_scale, OUT);
+                       zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
   else
     hipLaunchKernelGGL((linear_kernel<NT, false>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
-                       zero_last_group, ncomp, K, scale, row_scale, OUT);
+                       zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
   return check_launch("cm_linear");
 }
 
@@ -493,7 +508,7 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
 
 extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_perm, const int32_t *group_offsets,
                          int64_t nnodes, int ngroups, int zero_last_group, int ncomp, int K, int Nout, float scale,
-                         const float *row_scale, float *OUT, cm_stream_t stream) {
+                         const float *row_scale, const float *residual, float *OUT, cm_stream_t stream) {
   CM_REQUIRE(ncomp == 1 || ncomp == 16, "cm_linear: ncomp=%d must be 1 or 16", ncomp);
   CM_REQUIRE(!zero_last_group || (group_offsets != nullptr && ngroups >= 2),
              "cm_linear: a zero group needs node_perm / group_offsets and at least one weight group before it");
@@ -507,14 +522,14 @@ extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_p
   CM_REQUIRE(X && W_T && OUT, "cm_linear: NULL pointer");
   hipStream_t st = cm::as_stream(stream);
   switch (Nout / 32) {
-    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
-    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
-    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
-    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
-    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
-    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
-    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
-    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, OUT, st);
+    case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
+    case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
+    case 3: return cm::launch<3>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
+    case 4: return cm::launch<4>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
+    case 5: return cm::launch<5>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
+    case 6: return cm::launch<6>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
+    case 7: return cm::launch<7>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
+    case 8: return cm::launch<8>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
   }
   return CM_EINVAL;
 }

@@ -327,7 +327,7 @@ Tensor run_linear(const Tensor &X, const Tensor &WT, const Tensor &perm, const T
   const bool grouped = perm.defined();
   CM_CALL(cm_linear(fptr(X), fptr(WT), grouped ? iptr(perm) : nullptr, grouped ? iptr(off) : nullptr, N,
                     static_cast<int>(ngroups + (zero_last_group ? 1 : 0)), zero_last_group ? 1 : 0, scalar ? 1 : 16,
-                    static_cast<int>(K), static_cast<int>(Nout), scale, nullptr, N ? out.data_ptr<float>() : nullptr,
+                    static_cast<int>(K), static_cast<int>(Nout), scale, nullptr, nullptr, N ? out.data_ptr<float>() : nullptr,
                     stream_of(X)));
   return out;
 }

@@ -52,7 +52,7 @@ SIGNATURES = {
     "cm_sh_backward": (_i32, [_p, _p, _i64, _p, _p]),
     "cm_spline_forward": (_i32, [_p, _p, _p, _i64, _i32, _i32, _f32, _f32, _p, _p, _p]),
     "cm_spline_backward": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _f32, _f32, _p, _p]),
-    "cm_linear": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _i32, _f32, _p, _p, _p]),
+    "cm_linear": (_i32, [_p, _p, _p, _p, _i64, _i32, _i32, _i32, _i32, _i32, _f32, _p, _p, _p, _p]),
     "cm_symcon_tables": (_i32, [_p, _p, _p, _i32, _p, _p, _p, _i32, _p, _p, _p, _i32, _i32, _i32, _i32, _i32, _p, _p, _p, _p]),
     "cm_symcon_forward": (_i32, [_p, _p, _p, _p, _i32, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
     "cm_symcon_builtin_structure": (_i32, [_p, _i32, _p, _i32, _p, _p]),
@@ -355,11 +355,12 @@ def spline_backward(r, r_knots, coeffs, grad_R, r_width: float, r_max: float) ->
 
 # ---- linears ------------------------------------------------------------------------------------------
 def linear(X, W_T, node_perm=None, group_offsets=None, scale=None, zero_last_group: bool = False,
-           row_scale=None) -> torch.Tensor:
+           row_scale=None, residual=None) -> torch.Tensor:
     """X [N,16,K] with W_T [(ngroups,)4,N',K], or scalar features X [N,K] with W_T [(ngroups,)N',K] (transposed weight
     blocks); scale defaults to 1/sqrt(K).  Grouped calls pass the node grouping; with zero_last_group the grouping has
     one more group than W_T, whose rows come out as zeros.  Rows of nodes in no group are left unwritten.
-    row_scale [N,K]: X[n,m,k] is multiplied by row_scale[n,k] on the way in."""
+    row_scale [N,K]: X[n,m,k] is multiplied by row_scale[n,k] on the way in.  residual (shape of the result): added to
+    the written rows."""
     scalar = X.dim() == 2
     if scalar:
         if W_T.dim() == 2:
@@ -379,12 +380,14 @@ def linear(X, W_T, node_perm=None, group_offsets=None, scale=None, zero_last_gro
     if row_scale is not None and tuple(row_scale.shape) != (N, K):
         raise CudaMaceError("linear: row_scale must be [N, K]")
     OUT = torch.empty((N, Nout) if scalar else (N, 16, Nout), dtype=F32, device=X.device)
+    if residual is not None and tuple(residual.shape) != tuple(OUT.shape):
+        raise CudaMaceError("linear: residual must have the shape of the result, %s" % (tuple(OUT.shape),))
     _check(
         lib.cm_linear(
             _dev(X, F32, "X"), _dev(W_T, F32, "W_T"), _dev(node_perm, I32, "node_perm"),
             _dev(group_offsets, I32, "group_offsets"), N, ngroups + (1 if zero_last_group else 0), int(zero_last_group), ncomp,
             K, Nout, float(scale) if scale is not None else 1.0 / float(K) ** 0.5, _dev(row_scale, F32, "row_scale"),
-            _dev(OUT, F32, "OUT"), _stream(),
+            _dev(residual, F32, "residual"), _dev(OUT, F32, "OUT"), _stream(),
         )
     )
     return OUT

@@ -166,11 +166,16 @@ class linear_matmul(torch.nn.Module):
         # widths the MFMA linear kernel takes (multiples of 32 up to 256); anything else goes to torch.matmul as in the reference
         self.on_kernel = all(w % 32 == 0 and 32 <= w <= 256 for w in (n_in, n_out))
 
-    def forward(self, x):
+    def forward(self, x, residual=None):
+        """residual (optional, shape of the result): added to the product, in the kernel's epilogue where the kernel runs."""
         if self.on_kernel and x.is_cuda and x.dtype == torch.float32 and x.dim() == 2:
             # same fp32-equivalent GEMM as the per-l linears; a third faster than the library GEMM at these sizes
-            return ScalarLinearAutograd.apply(x, self.weights_transposed, self.weights)
-        return torch.matmul(x, self.weights)
+            if residual is not None and residual.dtype == torch.float32 and residual.shape == (x.shape[0], self.weights.shape[1]):
+                return ScalarLinearAutograd.apply(x, self.weights_transposed, self.weights, residual)
+            y = ScalarLinearAutograd.apply(x, self.weights_transposed, self.weights, None)
+        else:
+            y = torch.matmul(x, self.weights)
+        return y if residual is None else y + residual
 
 
 def element_linear_to_cuda(skip_tp):
@@ -512,9 +517,8 @@ class OptimizedInvariantMACE(torch.nn.Module):
                 contracted = LinearContractionAutograd.apply(
                     node_feats, W_T, W, scale, groups_of_one_hot(node_attrs32) if per_element else None,
                     groups_of(atom_types, ne), self._contraction_tables(layer))
-                node_feats = product.linear(contracted)  # fp32 [N, C]
-                if sc is not None and getattr(product, "use_sc", True):
-                    node_feats = node_feats + sc
+                # fp32 [N, C]; the skip connection is added in the linear kernel's epilogue
+                node_feats = product.linear(contracted, sc if sc is not None and getattr(product, "use_sc", True) else None)
             else:
                 node_feats = product(node_feats=node_feats, sc=sc, node_attrs=atom_types)  # fp32 [N, C]
             node_feats_list.append(node_feats)

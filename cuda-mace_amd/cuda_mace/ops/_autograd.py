@@ -251,20 +251,22 @@ class LinearContractionAutograd(torch.autograd.Function):
 
 
 class ScalarLinearAutograd(torch.autograd.Function):
-    """Y = X . W for scalar features X [N, K] on the MFMA linear kernel (one component per node); W_T [N', K] and
-    W [K, N'] are the two orientations of the same weights (forward uses W_T, the backward W)."""
+    """Y = X . W (+ residual) for scalar features X [N, K] on the MFMA linear kernel (one component per node); W_T [N', K]
+    and W [K, N'] are the two orientations of the same weights (forward uses W_T, the backward W).  The optional
+    residual [N, N'] is added in the kernel's epilogue; its gradient is the incoming one."""
 
     @staticmethod
     @_traced("scalar_linear forward")
-    def forward(ctx, X, W_T, W):
+    def forward(ctx, X, W_T, W, residual):  # always four arguments (residual may be None): backward returns four
         ctx.save_for_backward(W)
-        return cabi.linear(X.contiguous(), W_T, scale=1.0)
+        return cabi.linear(X.contiguous(), W_T, scale=1.0, residual=None if residual is None else residual.contiguous())
 
     @staticmethod
     @_traced("scalar_linear backward")
     def backward(ctx, grad):
         (W,) = ctx.saved_tensors
-        return cabi.linear(grad.contiguous(), W, scale=1.0), None, None
+        gX = cabi.linear(grad.contiguous(), W, scale=1.0) if ctx.needs_input_grad[0] else None
+        return gX, None, None, (grad if ctx.needs_input_grad[3] else None)
 
 
 class ReadoutEnergyAutograd(torch.autograd.Function):

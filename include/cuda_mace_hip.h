@@ -219,11 +219,14 @@ int cm_spline_backward(const float *r, const float *r_knots, const float *coeffs
  *   That is the backward of the symmetric contraction (gX[n, m, k] = grad_out[n, k] * grad[n, m, k],
  *   cuda/src/symmetric_contraction_impl.cu:198-234) folded into the backward of the linear layer that precedes
  *   the contraction: pass grad as X and grad_out as row_scale, and no [nnodes, 16, K] product is written.
+ *   residual fp32 [nnodes, ncomp, Nout] or NULL: when given, it is added to the written rows (OUT = scale X W +
+ *   residual; the model's "linear of the product plus skip connection", models/InvariantMACE.py:41-53 followed by the
+ *   product block's addition of sc, in one pass).  residual may be OUT itself (in-place accumulation).
  */
 int cm_linear(const float *X, const float *W_T, const int32_t *node_perm,
               const int32_t *group_offsets, int64_t nnodes, int ngroups, int zero_last_group,
-              int ncomp, int K, int Nout, float scale, const float *row_scale, float *OUT,
-              cm_stream_t stream);
+              int ncomp, int K, int Nout, float scale, const float *row_scale, const float *residual,
+              float *OUT, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Symmetric contraction, correlation 3, scalar (L = 0) output, with its analytic gradient.

@@ -398,3 +398,19 @@ def test_linear_row_scale(cabi):
     ref = O.linear(X * S[:, None, :], W)
     got = cabi.linear(X.float().to(DEV), W.transpose(-1, -2).contiguous().float().to(DEV), row_scale=S.float().to(DEV))
     close(got, ref, 1e-5, 2e-6)
+
+
+@pytest.mark.parametrize("K,Nout", [(128, 128), (64, 160), (32, 96)])
+def test_linear_residual(cabi, K, Nout):
+    """residual is added to the written rows, for 16-component and scalar features (both kernel variants: 128 and 96
+    columns run on the LDS-ring kernel when K has more than one chunk, 160 columns and K = 32 on the plain one)."""
+    g = torch.Generator().manual_seed(5)
+    N = 333
+    X = torch.randn(N, 16, K, generator=g, dtype=torch.float64).float().double()
+    R = torch.randn(N, 16, Nout, generator=g, dtype=torch.float64).float().double()
+    W = torch.randn(4, K, Nout, generator=g, dtype=torch.float64).float().double()
+    got = cabi.linear(X.float().to(DEV), W.transpose(-1, -2).contiguous().float().to(DEV), residual=R.float().to(DEV))
+    close(got, O.linear(X, W) + R, 1e-5, 2e-6)
+    Xs, Rs, Ws = X[:, 0].contiguous(), R[:, 0].contiguous(), W[0]
+    got = cabi.linear(Xs.float().to(DEV), Ws.t().contiguous().float().to(DEV), scale=1.0, residual=Rs.float().to(DEV))
+    close(got, Xs @ Ws + Rs, 1e-5, 2e-6)
