@@ -46,8 +46,8 @@ SIGNATURES = {
     "cm_mp_spline_backward": (_i32, [_p] * 5 + [_i32, _f32, _f32] + [_p] * 5 + [_i64, _i64, _i32] + [_p] * 5),
     "cm_mp_edge_forward": (_i32, [_p] * 4 + [_i32, _f32, _f32, _p, _p, _i64, _i64, _i32, _p, _p]),
     "cm_mp_edge_backward": (_i32, [_p] * 4 + [_i32, _f32, _f32] + [_p] * 5 + [_i64, _i64, _i32] + [_p] * 4),
-    "cm_edge_geometry_forward": (_i32, [_p, _p, _p, _p, _i64, _i64, _p, _p, _p]),
-    "cm_edge_geometry_backward": (_i32, [_p] * 9 + [_i64, _i64, _p, _p, _p]),
+    "cm_edge_geometry_forward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _p, _p, _p]),
+    "cm_edge_geometry_backward": (_i32, [_p] * 10 + [_i64, _i64, _p, _p, _p]),
     "cm_sh_forward": (_i32, [_p, _i64, _p, _p]),
     "cm_sh_backward": (_i32, [_p, _p, _i64, _p, _p]),
     "cm_spline_forward": (_i32, [_p, _p, _p, _i64, _i32, _i32, _f32, _f32, _p, _p, _p]),
@@ -287,7 +287,8 @@ def sh_backward(xyz: torch.Tensor, grad_Y: torch.Tensor) -> torch.Tensor:
 # ---- edge geometry ------------------------------------------------------------------------------
 
 
-def edge_geometry_forward(positions, row_a, row_b, shifts):
+def edge_geometry_forward(positions, row_a, row_b, shifts, node_rows=None):
+    """node_rows int32 [N] (optional): atom n of the edge lists is row node_rows[n] of positions."""
     E = row_a.numel()
     dev = positions.device
     vec = torch.empty(E, 3, dtype=F32, device=dev)
@@ -295,14 +296,15 @@ def edge_geometry_forward(positions, row_a, row_b, shifts):
     _check(
         lib.cm_edge_geometry_forward(
             _dev(positions, F64, "positions"), _dev(row_a, I32, "row_a"), _dev(row_b, I32, "row_b"),
-            _dev(shifts, F64, "shifts"), positions.shape[0], E, _dev(vec, F32, "vectors"), _dev(length, F32, "lengths"), _stream(),
+            _dev(shifts, F64, "shifts"), _dev(node_rows, I32, "node_rows"), positions.shape[0], E, _dev(vec, F32, "vectors"),
+            _dev(length, F32, "lengths"), _stream(),
         )
     )
     return vec, length
 
 
 def edge_geometry_backward(positions, row_a, row_b, shifts, a_first_occ, b_perm, b_offsets, grad_vectors, grad_lengths,
-                           need_positions: bool = True, need_shifts: bool = False):
+                           need_positions: bool = True, need_shifts: bool = False, node_rows=None):
     E = row_a.numel()
     N = positions.shape[0]
     dev = positions.device
@@ -311,7 +313,8 @@ def edge_geometry_backward(positions, row_a, row_b, shifts, a_first_occ, b_perm,
     _check(
         lib.cm_edge_geometry_backward(
             _dev(positions, F64, "positions"), _dev(row_a, I32, "row_a"), _dev(row_b, I32, "row_b"),
-            _dev(shifts, F64, "shifts"), _dev(a_first_occ, I32, "a_first_occ"), _dev(b_perm, I32, "b_perm"),
+            _dev(shifts, F64, "shifts"), _dev(node_rows, I32, "node_rows"), _dev(a_first_occ, I32, "a_first_occ"),
+            _dev(b_perm, I32, "b_perm"),
             _dev(b_offsets, I32, "b_offsets"), _dev(grad_vectors, F32, "grad_vectors"),
             _dev(grad_lengths, F32, "grad_lengths"), N, E, _dev(gpos, F64, "grad_positions"),
             _dev(gshift, F64, "grad_shifts"), _stream(),

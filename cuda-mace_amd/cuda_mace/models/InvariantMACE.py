@@ -429,7 +429,10 @@ class OptimizedInvariantMACE(torch.nn.Module):
         perm, inverse, edge_perm, edge_index, batch = _cached(data["edge_index"], "_cm_spatial_order", None,
                                                               lambda: self._spatial_order(data))
         inner = dict(data)
-        inner["positions"] = data["positions"].detach().index_select(0, perm)
+        # Without strain the positions stay in the caller's order: the geometry kernels read them (and write the forces)
+        # through the row map.  The strain path transforms positions per graph and works on a gathered copy.
+        direct = not (compute_virials or compute_stress or compute_displacement)
+        inner["positions"] = data["positions"].detach() if direct else data["positions"].detach().index_select(0, perm)
         inner["edge_index"], inner["batch"] = edge_index, batch
         inner["node_attrs"] = _cached_for(data["edge_index"], "_cm_spatial_attrs", data["node_attrs"],
                                           lambda: data["node_attrs"].index_select(0, perm))
@@ -439,17 +442,19 @@ class OptimizedInvariantMACE(torch.nn.Module):
                 inner[name] = _cached_for(data["edge_index"], "_cm_spatial_" + name, t, lambda t=t: t.index_select(0, edge_perm))
         rows = _cached(data["edge_index"], "_cm_spatial_rows32", None, lambda: (perm.int(), inverse))
         out = self._forward_ordered(inner, training, compute_force, compute_virials, compute_stress, compute_displacement,
-                                    node_rows=rows)
-        for name in ("forces", "node_energy"):  # node_feats is already written in the caller's order
+                                    node_rows=rows, positions_in_caller_order=direct)
+        # node_feats is already written in the caller's order, and so are the forces on the direct path
+        for name in ("node_energy",) if direct else ("forces", "node_energy"):
             if out.get(name) is not None:
                 out[name] = out[name].index_select(0, inverse)
         return out
 
     def _forward_ordered(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
                          compute_virials: bool = False, compute_stress: bool = False, compute_displacement: bool = False,
-                         node_rows=None) -> Dict[str, Optional[torch.Tensor]]:
+                         node_rows=None, positions_in_caller_order: bool = False) -> Dict[str, Optional[torch.Tensor]]:
         """node_rows = (rows int32 [N], inverse int64 [N]): node n of `data` is node rows[n] of the caller; the
-        returned node_feats is written in the caller's order (every other per-node output stays in the order of `data`)."""
+        returned node_feats is written in the caller's order (every other per-node output stays in the order of `data`).
+        positions_in_caller_order: data["positions"] (and hence the forces) are rows of the caller, read through rows."""
         data["positions"].requires_grad_(True)
         positions = data["positions"]
         node_attrs = data["node_attrs"]
@@ -494,7 +499,8 @@ class OptimizedInvariantMACE(torch.nn.Module):
                                            lambda: (node_attrs.detach().float(), node_attrs.detach().argmax(dim=-1).int()))
 
         # vectors = positions[edge_index[1]] - positions[edge_index[0]] + shifts in fp64, rounded once to fp32
-        vectors32, lengths32 = EdgeGeometryAutograd.apply(positions, shifts, receiver, sender)
+        vectors32, lengths32 = EdgeGeometryAutograd.apply(positions, shifts, receiver, sender,
+                                                          node_rows[0] if positions_in_caller_order else None)
         # fused mode: the message-passing kernels take the vectors themselves and evaluate the harmonics per edge
         edge_attrs = None if self.fused_radial else self.spherical_harmonics.forward(vectors32)
 

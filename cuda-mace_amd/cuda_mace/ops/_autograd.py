@@ -175,20 +175,24 @@ class InvariantMessagePassingEdgeTPAutograd(torch.autograd.Function):
 
 # ------------------------------------------------------------------------------------------------
 class EdgeGeometryAutograd(torch.autograd.Function):
-    """(positions [N,3], shifts [E,3], row_a int32 [E] non-decreasing, row_b int32 [E]) -> (vectors fp32 [E,3],
-    lengths fp32 [E]) with vectors = positions[row_b] - positions[row_a] + shifts evaluated in fp64.
+    """(positions [N,3], shifts [E,3], row_a int32 [E] non-decreasing, row_b int32 [E], node_rows int32 [N] or None) ->
+    (vectors fp32 [E,3], lengths fp32 [E]) with vectors = positions[row_b] - positions[row_a] + shifts evaluated in fp64.
+    With node_rows, atom n of the edge lists is row node_rows[n] of positions (and of its gradient).
     Differentiable in positions and shifts; the backward scatters edge gradients to atoms over the CSR of row_a
     and the sorted view of row_b (the same index structures message passing uses), in fp64, without atomics."""
 
     @staticmethod
     @_traced("edge_geometry forward")
-    def forward(ctx, positions, shifts, row_a, row_b):
+    def forward(ctx, positions, shifts, row_a, row_b, node_rows):
         _require(row_a.dtype == I32 and row_b.dtype == I32, "edge geometry: int32 edge lists expected")
         _require(positions.dim() == 2 and positions.shape[1] == 3, "edge geometry: positions must be [nnodes, 3]")
+        _require(node_rows is None or (node_rows.dtype == I32 and node_rows.numel() == positions.shape[0]),
+                 "edge geometry: node_rows must be int32 [nnodes]")
         pos64 = positions.detach().double().contiguous()
         sh64 = shifts.detach().double().contiguous()
-        vec, length = cabi.edge_geometry_forward(pos64, row_a, row_b, sh64)
+        vec, length = cabi.edge_geometry_forward(pos64, row_a, row_b, sh64, node_rows)
         ctx.save_for_backward(pos64, sh64, row_a, row_b)
+        ctx.node_rows = node_rows
         ctx.dtypes = (positions.dtype, shifts.dtype)
         ctx.set_materialize_grads(False)  # an unused output arrives as None in backward, not as zeros
         return vec, length
@@ -197,7 +201,7 @@ class EdgeGeometryAutograd(torch.autograd.Function):
     @_traced("edge_geometry backward")
     def backward(ctx, grad_vec, grad_len):
         if grad_vec is None and grad_len is None:
-            return None, None, None, None
+            return None, None, None, None, None
         pos64, sh64, row_a, row_b = ctx.saved_tensors
         need_pos, need_shift = ctx.needs_input_grad[:2]
         nnodes = pos64.shape[0]
@@ -206,12 +210,12 @@ class EdgeGeometryAutograd(torch.autograd.Function):
         gv = grad_vec.contiguous() if grad_vec is not None else None
         gl = grad_len.contiguous() if grad_len is not None else None
         gpos, gshift = cabi.edge_geometry_backward(pos64, row_a, row_b, sh64, first_occ, perm, off, gv, gl,
-                                                   need_positions=need_pos, need_shifts=need_shift)
+                                                   need_positions=need_pos, need_shifts=need_shift, node_rows=ctx.node_rows)
         if gpos is not None:
             gpos = gpos.to(ctx.dtypes[0])
         if gshift is not None:
             gshift = gshift.to(ctx.dtypes[1])
-        return gpos, gshift, None, None
+        return gpos, gshift, None, None, None
 
 
 class LinearContractionAutograd(torch.autograd.Function):

@@ -169,13 +169,15 @@ int cm_sh_backward(const float *xyz, const float *grad_Y, int64_t nedges, float 
  *   grad_positions[n] = sum_{e: row_b[e] = n} g - sum_{e: row_a[e] = n} g   (fp64 [nnodes, 3], may be NULL)
  *   grad_shifts[e] = g                                                     (fp64 [nedges, 3], may be NULL)
  *   a_first_occ = cm_first_occurences(row_a); b_perm / b_offsets = cm_stable_key_sort(row_b, nedges, nnodes).
+ *   node_rows int32 [nnodes] or NULL: when given, atom n of the edge lists is row node_rows[n] of positions and of
+ *   grad_positions (a permutation), so a caller that relabels its atoms keeps positions and forces in its own order.
  */
 int cm_edge_geometry_forward(const double *positions, const int32_t *row_a, const int32_t *row_b,
-                             const double *shifts, int64_t nnodes, int64_t nedges, float *vectors,
-                             float *lengths, cm_stream_t stream);
+                             const double *shifts, const int32_t *node_rows, int64_t nnodes, int64_t nedges,
+                             float *vectors, float *lengths, cm_stream_t stream);
 int cm_edge_geometry_backward(const double *positions, const int32_t *row_a, const int32_t *row_b,
-                              const double *shifts, const int32_t *a_first_occ, const int32_t *b_perm,
-                              const int32_t *b_offsets, const float *grad_vectors,
+                              const double *shifts, const int32_t *node_rows, const int32_t *a_first_occ,
+                              const int32_t *b_perm, const int32_t *b_offsets, const float *grad_vectors,
                               const float *grad_lengths, int64_t nnodes, int64_t nedges,
                               double *grad_positions, double *grad_shifts, cm_stream_t stream);
 

@@ -356,6 +356,16 @@ def test_edge_geometry(cabi, nnodes, avg, iso, seed):
     vec2, _ = O.edge_geometry(pos, row_a, row_b, shifts)
     (vec2 * gv.float().double()).sum().backward()
     close(only_vec, pos.grad, 1e-12, 1e-13)
+    # row map: the same positions stored in a permuted order give bit-identical vectors, and the position gradient
+    # comes out in that order
+    rows = torch.randperm(nnodes, generator=g).int()
+    stored = torch.empty_like(pos.detach())
+    stored[rows.long()] = pos.detach()  # atom n sits in row rows[n]
+    vec_m, len_m = cabi.edge_geometry_forward(d(stored), d(row_a), d(row_b), d(shifts), node_rows=d(rows))
+    assert torch.equal(vec_m, vec) and torch.equal(len_m, length)
+    gpos_m, _ = cabi.edge_geometry_backward(d(stored), d(row_a), d(row_b), d(shifts), fo, perm, off, d(gv).float(), d(gl).float(),
+                                            need_positions=True, node_rows=d(rows))
+    assert torch.equal(gpos_m[d(rows).long()], gpos)
 
 
 # ---- readouts ---------------------------------------------------------------------------------------------
