@@ -238,12 +238,48 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
 // -----------------------------------------------------------------------------------------------
 // backward, sender pass: gX[n, :] = sum over the edges sent by n of the per-edge contributions
 // -----------------------------------------------------------------------------------------------
-template <int C>
+// LIVE: 0 = every row of gXe is read; 1 / 2 = only rows of edges within r_max, by the edge vector / the edge length
+// (the spline-fused edge pass writes no others).
+//
+// A slot (the lanes that carry one row) takes four edges per iteration.  Three loads depend on each other per edge --
+// its index from the sender-sorted view, its vector or length (LIVE), its row -- so the loop is pipelined over
+// iterations: iteration i issues the rows of batch i, the vectors of batch i + 1 and the indices of batch i + 2
+// together and uses what iteration i - 1 issued: one memory latency per iteration instead of three.  Every load is
+// unconditional: an edge that is not to be read (beyond the list's end, beyond the cutoff, out of range) loads the row
+// of the slot's last good edge again, a cache hit, and its value is dropped by a select.  The loads are issued from
+// inline assembly and waited for once per iteration by an explicit wait, with the loaded registers passed through the
+// waiting statement so that no use can move above it: left to itself the compiler sinks each load to its first use in
+// the next iteration and waits for it there, which puts the three latencies back in a row.  Registers that are still
+// being loaded are never copied; the batches change roles after the wait.  The summation order is fixed.
+__device__ __forceinline__ void issue_load(int &dst, const int32_t *p) {
+  asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load(float &dst, const float *p) {
+  asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load(f3 &dst, const float *p) {
+  asm volatile("global_load_dwordx3 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load_stream(float &dst, const float *p) {
+  asm volatile("global_load_dword %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void issue_load_stream(f4 &dst, const float *p) {
+  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
+}
+template <class T>
+__device__ __forceinline__ void arrived(T &v) {
+  asm volatile("" : "+v"(v));
+}
+
+template <int C, int LIVE>
 __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
     const float *__restrict__ gXe, const int32_t *__restrict__ perm,
-    const int32_t *__restrict__ offsets, int nnodes, int64_t nedges, float *__restrict__ gX) {
+    const int32_t *__restrict__ offsets, int nnodes, int64_t nedges, const float *__restrict__ live_by, float r_max,
+    float *__restrict__ gX) {
   using K = Cfg<C>;
   using vec = typename K::vec;
+  constexpr int B = 4;            // edges per slot and iteration
+  constexpr int STEP = B * K::EPW;
   const int node = blockIdx.x;
   const int lane = threadIdx.x;
   const int slot = lane / K::SW;
@@ -252,22 +288,120 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
   const int k0 = offsets[node];
   const int k1 = offsets[node + 1];
   vec acc = zerov<vec>();
-  if (active) {
-    // four independent row gathers in flight per slot; the summation order stays fixed.  Every row is read exactly
-    // once: streamed loads
+  if (active && k0 < k1 && nedges > 0) {
+    const int klast = k1 - 1;
+    const int emax = static_cast<int>(nedges - 1);
+    int e_cur[B], e_nxt[B], e_aft[B];   // indices of batches i, i + 1 (arrived) and i + 2 (being loaded)
+    f3 lv_cur[B], lv_nxt[B];    // LIVE 1: vectors of batch i (arrived) and i + 1 (being loaded)
+    float lr_cur[B], lr_nxt[B];  // LIVE 2: lengths of the same
+    f4 rows4[B];                        // rows of the previous batch (four channels per lane: one 16-byte load)
+    float rowsf[B][K::V];               // the same for the other channel counts per lane (dword loads)
+    bool take[B];
+    auto issue_indices = [&](int kk, int (&e)[B]) {
+#pragma unroll
+      for (int j = 0; j < B; ++j) issue_load(e[j], perm + min(kk + j * K::EPW, klast));
+    };
+    auto issue_live = [&](const int (&e)[B]) {  // into lv_nxt / lr_nxt
+      if constexpr (LIVE != 0) {
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+          const int ec = min(max(e[j], 0), emax);
+          if constexpr (LIVE == 1) issue_load(lv_nxt[j], live_by + 3 * static_cast<int64_t>(ec));
+          else issue_load(lr_nxt[j], live_by + ec);
+        }
+      }
+    };
+    auto issue_rows = [&](const int (&e)[B]) {
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        const float *p = gXe + static_cast<int64_t>(e[j]) * C + K::off(cl);
+        if constexpr (K::V == 4) {
+          issue_load_stream(rows4[j], p);
+        } else {
+#pragma unroll
+          for (int q = 0; q < K::V; ++q) issue_load_stream(rowsf[j][q], p + q * K::ES);
+        }
+      }
+    };
+    auto wait_all = [&](auto &...regs) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      (arrived(regs), ...);
+    };
+    auto arrived_rows = [&]() {
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        if constexpr (K::V == 4) {
+          arrived(rows4[j]);
+        } else {
+#pragma unroll
+          for (int q = 0; q < K::V; ++q) arrived(rowsf[j][q]);
+        }
+      }
+    };
+    auto row = [&](int j) -> vec {  // the row if it is to be taken, zeros otherwise
+      vec r;
+      if constexpr (K::V == 4) {
+        r = rows4[j];
+      } else {
+#pragma unroll
+        for (int q = 0; q < K::V; ++q) r[q] = rowsf[j][q];
+      }
+      return take[j] ? r : zerov<vec>();
+    };
+
     int k = k0 + slot;
-    for (; k + 3 * K::EPW < k1; k += 4 * K::EPW) {
-      const int ea = perm[k], eb = perm[k + K::EPW], ec = perm[k + 2 * K::EPW], ed = perm[k + 3 * K::EPW];
-      const vec va = static_cast<unsigned>(ea) < static_cast<uint64_t>(nedges) ? K::ld_stream(gXe + static_cast<int64_t>(ea) * C + K::off(cl)) : zerov<vec>();
-      const vec vb = static_cast<unsigned>(eb) < static_cast<uint64_t>(nedges) ? K::ld_stream(gXe + static_cast<int64_t>(eb) * C + K::off(cl)) : zerov<vec>();
-      const vec vc = static_cast<unsigned>(ec) < static_cast<uint64_t>(nedges) ? K::ld_stream(gXe + static_cast<int64_t>(ec) * C + K::off(cl)) : zerov<vec>();
-      const vec vd = static_cast<unsigned>(ed) < static_cast<uint64_t>(nedges) ? K::ld_stream(gXe + static_cast<int64_t>(ed) * C + K::off(cl)) : zerov<vec>();
-      acc += (va + vb) + (vc + vd);
+    // prologue: indices of batches 0 and 1, then the vectors of batch 0
+    issue_indices(k, e_cur);
+    issue_indices(k + STEP, e_nxt);
+    wait_all(e_cur[0], e_cur[1], e_cur[2], e_cur[3], e_nxt[0], e_nxt[1], e_nxt[2], e_nxt[3]);
+    issue_live(e_cur);  // lands in lv_nxt / lr_nxt: the loop's first act is to move it to the current set
+    int good = min(max(e_cur[0], 0), emax);  // a row that may always be read
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      rows4[j] = zero4();
+#pragma unroll
+      for (int q = 0; q < K::V; ++q) rowsf[j][q] = 0.f;
+      take[j] = false;
+      e_aft[j] = e_nxt[j];
     }
-    for (; k < k1; k += K::EPW) {
-      const int e = perm[k];
-      if (static_cast<unsigned>(e) < static_cast<uint64_t>(nedges)) acc += K::ld_stream(gXe + static_cast<int64_t>(e) * C + K::off(cl));
+    // shift the roles once so that the loop head finds batch 0 in e_nxt / lv_nxt and batch 1 in e_aft
+#pragma unroll
+    for (int j = 0; j < B; ++j) e_nxt[j] = e_cur[j];
+    for (; k < k1; k += STEP) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      arrived_rows();
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        arrived(e_aft[j]);
+        if constexpr (LIVE == 1) arrived(lv_nxt[j]);
+        if constexpr (LIVE == 2) arrived(lr_nxt[j]);
+      }
+      // everything has arrived: rows of the previous batch, vectors of this one, indices of the next one
+      acc += (row(0) + row(1)) + (row(2) + row(3));
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        e_cur[j] = e_nxt[j];
+        e_nxt[j] = e_aft[j];
+        if constexpr (LIVE == 1) lv_cur[j] = lv_nxt[j];
+        if constexpr (LIVE == 2) lr_cur[j] = lr_nxt[j];
+      }
+#pragma unroll
+      for (int j = 0; j < B; ++j) {
+        bool ok = (k + j * K::EPW < k1) & (static_cast<unsigned>(e_cur[j]) <= static_cast<unsigned>(emax));
+        if constexpr (LIVE == 1) ok = ok & (edge_length(lv_cur[j].x, lv_cur[j].y, lv_cur[j].z) <= r_max);
+        if constexpr (LIVE == 2) ok = ok & (lr_cur[j] <= r_max);
+        take[j] = ok;
+        good = ok ? e_cur[j] : good;
+        e_cur[j] = ok ? e_cur[j] : good;
+      }
+      // issue: rows of this batch, vectors of the next, indices of the one after
+      issue_rows(e_cur);
+      issue_live(e_nxt);
+      issue_indices(k + 2 * STEP, e_aft);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    arrived_rows();
+    acc += (row(0) + row(1)) + (row(2) + row(3));
   }
 #pragma unroll
   for (int off = kWave / 2; off >= K::SW; off >>= 1) acc += shfl_downv(acc, off);
@@ -314,18 +448,27 @@ int launch_backward(const float *X, const float *Y, const float *R, const float 
 
 template <int C>
 int launch_sender(const float *gXe, const int32_t *perm, const int32_t *offsets, int64_t nnodes, int64_t nedges,
-                  float *gX, hipStream_t st) {
-  hipLaunchKernelGGL(mp_backward_sender_kernel<C>, dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st, gXe, perm,
-                     offsets, static_cast<int>(nnodes), nedges, gX);
+                  float *gX, hipStream_t st, const float *live_vec, const float *live_r, float r_max) {
+  const dim3 grid(static_cast<unsigned>(nnodes)), block(kWave);
+  if (live_vec)
+    hipLaunchKernelGGL((mp_backward_sender_kernel<C, 1>), grid, block, 0, st, gXe, perm, offsets, static_cast<int>(nnodes), nedges,
+                       live_vec, r_max, gX);
+  else if (live_r)
+    hipLaunchKernelGGL((mp_backward_sender_kernel<C, 2>), grid, block, 0, st, gXe, perm, offsets, static_cast<int>(nnodes), nedges,
+                       live_r, r_max, gX);
+  else
+    hipLaunchKernelGGL((mp_backward_sender_kernel<C, 0>), grid, block, 0, st, gXe, perm, offsets, static_cast<int>(nnodes), nedges,
+                       static_cast<const float *>(nullptr), 0.f, gX);
   return check_launch("cm_mp_backward (sender pass)");
 }
 
 }  // namespace
 
 int mp::launch_sender_pass(int channels, const float *gXe, const int32_t *perm, const int32_t *offsets, int64_t nnodes,
-                           int64_t nedges, float *gX, hipStream_t st) {
+                           int64_t nedges, float *gX, hipStream_t st, const float *live_vec, const float *live_r,
+                           float r_max) {
   int rc = CM_EINVAL;
-  CM_DISPATCH_C(channels, rc = launch_sender<C_>(gXe, perm, offsets, nnodes, nedges, gX, st));
+  CM_DISPATCH_C(channels, rc = launch_sender<C_>(gXe, perm, offsets, nnodes, nedges, gX, st, live_vec, live_r, r_max));
   return rc;
 }
 

@@ -242,9 +242,19 @@ __device__ __forceinline__ void store_reduced16(const float (&p)[16], int cl, in
   }
 }
 
-// Sender pass of the backward, shared by both variants (defined in mp.hip).
+// Length of an edge vector as the spline-fused kernels take it.  The edge pass decides by it which rows of the per-edge
+// scratch it writes and the sender pass which rows it reads, so both must get the same bits: the operations are spelled
+// out (no contraction left to the compiler).
+__device__ __forceinline__ float edge_length(float v0, float v1, float v2) {
+  return sqrtf(fmaf(v2, v2, fmaf(v1, v1, v0 * v0)));
+}
+
+// Sender pass of the backward, shared by both variants (defined in mp.hip).  With live_vec (edge vectors [E, 3]) or
+// live_r (edge lengths [E]) given, only the rows of edges within r_max are read: the spline-fused edge pass writes no
+// others.
 int launch_sender_pass(int channels, const float *gXe, const int32_t *perm, const int32_t *offsets, int64_t nnodes,
-                       int64_t nedges, float *gX, hipStream_t st);
+                       int64_t nedges, float *gX, hipStream_t st, const float *live_vec = nullptr,
+                       const float *live_r = nullptr, float r_max = 0.f);
 
 }  // namespace mp
 }  // namespace cm

@@ -82,7 +82,7 @@ __device__ __forceinline__ int stage_edges(const float *__restrict__ Y, const in
       s = sender[e];
       if constexpr (FROM_VEC) {
         const float v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
-        locate(sp, sqrtf(v0 * v0 + v1 * v1 + v2 * v2), idx, x);
+        locate(sp, edge_length(v0, v1, v2), idx, x);
         sh::eval(sh::direction(v0, v1, v2), y);
       } else {
         locate(sp, sp.r[e], idx, x);
@@ -239,12 +239,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   for (int cursor = e0; cursor < e1;) {
     const int base = cursor;  // sOrig counts from here
     __syncthreads();
-    // consumed edges that are not live: their outputs are zeros (the sender pass sums every row of gXe)
-    auto dead = [&](int pass_base, int consumed, unsigned long long live_mask, bool lane_is_dead) {
-      if constexpr (WANT_GX) {
-        for (int k = slot; k < consumed; k += K::EPW)
-          if (!((live_mask >> k) & 1ull) && active) K::st(gXe + static_cast<int64_t>(pass_base + k) * C + K::off(cl), zerov<vec>());
-      }
+    // consumed edges that are not live: their gradients are zeros (their rows of gXe stay unwritten: the sender pass
+    // reads the rows of live edges only)
+    auto dead = [&](int pass_base, int, unsigned long long, bool lane_is_dead) {
       if constexpr (WANT_GY || WANT_GR) {
         if (lane_is_dead) {
           const int64_t e = pass_base + lane;
@@ -426,7 +423,8 @@ int launch_backward(const float *X, const float *Y, const Spline &sp, const floa
   }
   int rc = check_launch(FROM_VEC ? "cm_mp_edge_backward (edge pass)" : "cm_mp_spline_backward (edge pass)");
   if (rc != CM_OK) return rc;
-  if (gX) rc = mp::launch_sender_pass(C, gXe, perm, offsets, nnodes, nedges, gX, st);
+  if (gX) rc = mp::launch_sender_pass(C, gXe, perm, offsets, nnodes, nedges, gX, st, FROM_VEC ? sp.vec : nullptr,
+                                      FROM_VEC ? nullptr : sp.r, sp.r_max);
   return rc;
 }
 
