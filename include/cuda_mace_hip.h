@@ -113,6 +113,8 @@ int cm_mp_backward(const float *X, const float *Y, const float *R, const float *
  * cuda/src/invariant_message_passing_impl.cu:74-399) so that R[nedges, 4, channels], dR/dr and grad_R are
  * never written to or read from HBM.  The backward returns grad_r[e] = sum_j grad_R[e, j] * dR/dr[e, j]
  * directly (may be NULL), next to gY and gX as in cm_mp_backward.
+ * Edges with r[e] > r_max (the skin of a Verlet list) and edges whose sender index is out of range contribute nothing
+ * and get zero gradients; their rows of edge_scratch are neither written nor read.
  */
 int cm_mp_spline_forward(const float *X, const float *Y, const float *r, const float *r_knots,
                          const float *coeffs, int nknots, float r_width, float r_max,
