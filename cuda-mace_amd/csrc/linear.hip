@@ -456,20 +456,50 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
     stage = stage == 2 ? 0 : stage + 1;
   }
 
+  if constexpr (NT <= 4) {
+    // Output through LDS, so that rows leave as 16-byte stores (a lane's accumulators are one column of 16 rows: stored
+    // directly they are 64 four-byte stores per lane).  Every wave is past its last multiply after the barrier, so the
+    // ring and the weight planes are free: each wave lays its 32 x Nout block out row-major in its own piece of them.
+    asm volatile("s_barrier" ::: "memory");
+    constexpr int TILE = 32 * NOUT;  // floats per wave
+    static_assert(4 * TILE <= kStages * kTileNodes * kKC || (3 * TILE <= kStages * kTileNodes * kKC && TILE * 4 <= 3 * NOUT * kLdH * 2),
+                  "output staging does not fit the ring and the weight planes");
+    float *tile = (4 * TILE <= kStages * kTileNodes * kKC || wave < 3) ? sRaw + wave * TILE : reinterpret_cast<float *>(sBp);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
-    const int node = sNode[row];
-    if (node >= 0) {
-      const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
-      float *op = OUT + at;
-      if (residual) {  // may be OUT itself: every element is read and written by the same lane
-        const float *rp = residual + at;
+    for (int r = 0; r < 16; ++r) {
+      const int row = 8 * (r / 4) + 4 * half + (r % 4);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale + rp[32 * t];
-      } else {
+      for (int t = 0; t < NT; ++t) tile[row * NOUT + 32 * t + mrow] = acc[t][r] * scale;
+    }
+    constexpr int PPR = NOUT / 4;  // 16-byte pieces per row
 #pragma unroll
-        for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+    for (int i = 0; i < TILE / 4 / kWave; ++i) {
+      const int q = i * kWave + lane;
+      const int row = q / PPR, col = 4 * (q % PPR);
+      const int node = sNode[32 * wave + row];
+      if (node >= 0) {
+        const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + col;
+        f4 v = *reinterpret_cast<const f4 *>(tile + row * NOUT + col);
+        if (residual) v += ld4(residual + at);  // may be OUT itself: every element is read and written by the same lane
+        st4(OUT + at, v);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
+      const int node = sNode[row];
+      if (node >= 0) {
+        const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
+        float *op = OUT + at;
+        if (residual) {  // may be OUT itself: every element is read and written by the same lane
+          const float *rp = residual + at;
+#pragma unroll
+          for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale + rp[32 * t];
+        } else {
+#pragma unroll
+          for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+        }
       }
     }
   }
