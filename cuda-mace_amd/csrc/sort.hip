@@ -4,6 +4,7 @@
 // item index.  The result is the unique stable order, so it is reproducible bit for bit although
 // atomics are used on the way.
 #include <algorithm>
+#include <mutex>
 
 #include "common.hpp"
 
@@ -89,6 +90,35 @@ extern "C" size_t cm_stable_key_sort_workspace(int64_t n, int64_t nkeys) {
   return (bytes + 255) & ~static_cast<size_t>(255);
 }
 
+namespace cm {
+namespace {
+
+// Enqueues the five kernels of the sort; `workspace` holds cm_stable_key_sort_workspace(n, nkeys) bytes.
+int sort_enqueue(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm, int32_t *offsets, void *workspace,
+                 hipStream_t st, const char *what) {
+  int32_t *counts = static_cast<int32_t *>(workspace);
+  int32_t *cursor = counts + nkeys;
+  int32_t *bucketed = cursor + nkeys;
+  const int block = 256;
+  if (nkeys > 0) {
+    const unsigned g = static_cast<unsigned>(std::min<int64_t>(ceil_div(nkeys, block), 4096));
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(block), 0, st, counts, nkeys, 0);
+  }
+  const unsigned gn = static_cast<unsigned>(ceil_div(n > 0 ? n : 1, block));
+  if (n > 0)
+    hipLaunchKernelGGL(histogram_kernel, dim3(gn), dim3(block), 0, st, keys, n, static_cast<int>(nkeys), counts);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kScanThreads), 0, st, counts, static_cast<int>(nkeys), offsets, cursor);
+  if (n > 0) {
+    hipLaunchKernelGGL(bucket_fill_kernel, dim3(gn), dim3(block), 0, st, keys, n, static_cast<int>(nkeys), cursor, bucketed);
+    hipLaunchKernelGGL(bucket_rank_kernel, dim3(gn), dim3(block), 0, st, keys, bucketed, offsets,
+                       static_cast<int>(nkeys), perm);
+  }
+  return check_launch(what);
+}
+
+}  // namespace
+}  // namespace cm
+
 extern "C" int cm_stable_key_sort(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm,
                                   int32_t *offsets, void *workspace, size_t workspace_bytes,
                                   cm_stream_t stream) {
@@ -101,23 +131,64 @@ extern "C" int cm_stable_key_sort(const int32_t *keys, int64_t n, int64_t nkeys,
                   cm_stable_key_sort_workspace(n, nkeys));
     return CM_ENOSPC;
   }
-  hipStream_t st = cm::as_stream(stream);
-  int32_t *counts = static_cast<int32_t *>(workspace);
-  int32_t *cursor = counts + nkeys;
-  int32_t *bucketed = cursor + nkeys;
-  const int block = 256;
-  if (nkeys > 0) {
-    const unsigned g = static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(nkeys, block), 4096));
-    hipLaunchKernelGGL(cm::fill_i32_kernel, dim3(g), dim3(block), 0, st, counts, nkeys, 0);
+  return cm::sort_enqueue(keys, n, nkeys, perm, offsets, workspace, cm::as_stream(stream), "cm_stable_key_sort");
+}
+
+// ---- the same sort without a caller's workspace ---------------------------------------------------------------
+// The counters, cursors and the bucketed item list live in a device array that is part of the library's code object:
+// every GPU the library runs on holds its own copy at its own address for the life of the process.
+#define CM_SORT_STATIC_BYTES (32u << 20)
+static __device__ __align__(256) unsigned char scratch[CM_SORT_STATIC_BYTES];
+
+namespace cm {
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each GPU, looked up once per GPU
+
+// Device address of this GPU's copy of `scratch` (nullptr after storing an error message).  In host code the
+// array's name is only a handle for the runtime; kernels and copies must be given the address returned here.
+void *static_scratch_of_current_device() {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("cm_stable_key_sort_static: no usable current device (%s)", hipGetErrorString(err));
+    return nullptr;
   }
-  const unsigned gn = static_cast<unsigned>(cm::ceil_div(n > 0 ? n : 1, block));
-  if (n > 0)
-    hipLaunchKernelGGL(cm::histogram_kernel, dim3(gn), dim3(block), 0, st, keys, n, static_cast<int>(nkeys), counts);
-  hipLaunchKernelGGL(cm::scan_kernel, dim3(1), dim3(cm::kScanThreads), 0, st, counts, static_cast<int>(nkeys), offsets, cursor);
-  if (n > 0) {
-    hipLaunchKernelGGL(cm::bucket_fill_kernel, dim3(gn), dim3(block), 0, st, keys, n, static_cast<int>(nkeys), cursor, bucketed);
-    hipLaunchKernelGGL(cm::bucket_rank_kernel, dim3(gn), dim3(block), 0, st, keys, bucketed, offsets,
-                       static_cast<int>(nkeys), perm);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *ptr = nullptr;
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr) {
+      set_error("cm_stable_key_sort_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(err));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
   }
-  return cm::check_launch("cm_stable_key_sort");
+  return g_scratch_ptr[dev];
+}
+
+}  // namespace
+}  // namespace cm
+
+extern "C" size_t cm_stable_key_sort_static_capacity(void) { return CM_SORT_STATIC_BYTES; }
+
+extern "C" int cm_stable_key_sort_static(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm,
+                                         int32_t *offsets, cm_stream_t stream) {
+  CM_REQUIRE(n >= 0 && nkeys >= 0, "cm_stable_key_sort_static: negative size");
+  CM_REQUIRE(n < INT32_MAX && nkeys < INT32_MAX, "cm_stable_key_sort_static: sizes exceed int32 indexing");
+  CM_REQUIRE(offsets != nullptr, "cm_stable_key_sort_static: offsets is NULL");
+  CM_REQUIRE(n == 0 || (keys && perm), "cm_stable_key_sort_static: NULL pointer");
+  const size_t need = cm_stable_key_sort_workspace(n, nkeys);
+  if (need > CM_SORT_STATIC_BYTES) {
+    cm::set_error("cm_stable_key_sort_static: n = %lld items with nkeys = %lld need %zu bytes of scratch, the built-in "
+                  "buffer holds %zu (4 * (n + 2 * nkeys) must not exceed it); use cm_stable_key_sort with a workspace",
+                  static_cast<long long>(n), static_cast<long long>(nkeys), need,
+                  static_cast<size_t>(CM_SORT_STATIC_BYTES));
+    return CM_ENOSPC;
+  }
+  void *ws = cm::static_scratch_of_current_device();
+  if (ws == nullptr) return CM_ELAUNCH;
+  return cm::sort_enqueue(keys, n, nkeys, perm, offsets, ws, cm::as_stream(stream), "cm_stable_key_sort_static");
 }

@@ -40,6 +40,8 @@ SIGNATURES = {
     "cm_first_occurences": (_i32, [_p, _i64, _i64, _p, _p]),
     "cm_stable_key_sort_workspace": (_sz, [_i64, _i64]),
     "cm_stable_key_sort": (_i32, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),
+    "cm_stable_key_sort_static_capacity": (_sz, []),
+    "cm_stable_key_sort_static": (_i32, [_p, _i64, _i64, _p, _p, _p]),
     "cm_mp_forward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _p, _p]),
     "cm_mp_backward": (_i32, [_p] * 8 + [_i64, _i64, _i32] + [_p] * 5),
     "cm_mp_spline_forward": (_i32, [_p] * 5 + [_i32, _f32, _f32, _p, _p, _i64, _i64, _i32, _p, _p]),
@@ -145,6 +147,20 @@ def stable_key_sort(keys: torch.Tensor, nkeys: int):
         )
     )
     return perm, offsets
+
+
+def stable_key_sort_static(keys: torch.Tensor, nkeys: int, perm: torch.Tensor, offsets: torch.Tensor) -> None:
+    """cm_stable_key_sort_static: the same sort into caller-provided `perm` [n] and `offsets` [nkeys + 1], with the
+    library's built-in scratch buffer in place of a workspace, so nothing is allocated.  Raises when the sizes exceed
+    that buffer.  Calls on one GPU share the buffer and must not overlap."""
+    n = keys.numel()
+    if perm.numel() != n or offsets.numel() != nkeys + 1:
+        raise CudaMaceError("perm must hold n = %d and offsets nkeys + 1 = %d entries" % (n, nkeys + 1))
+    _check(
+        lib.cm_stable_key_sort_static(
+            _dev(keys, I32, "keys"), n, nkeys, _dev(perm, I32, "perm"), _dev(offsets, I32, "offsets"), _stream()
+        )
+    )
 
 
 # ---- message passing --------------------------------------------------------------------------

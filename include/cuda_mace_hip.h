@@ -73,6 +73,19 @@ int cm_stable_key_sort(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *p
                        cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * cm_stable_key_sort without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same operands and result as cm_stable_key_sort; the counters, cursors and bucketed item list live in a buffer of
+ * cm_stable_key_sort_static_capacity() bytes (32 MiB) that is part of the library image on every GPU, so the call
+ * allocates nothing.  It returns CM_ENOSPC when cm_stable_key_sort_workspace(n, nkeys) = 4 * (n + 2 * nkeys) bytes
+ * (rounded up to 256) exceeds that capacity.  All calls on one GPU share that GPU's buffer: calls that may overlap
+ * on one GPU (different streams, different threads) race and must be serialised by the caller.
+ */
+size_t cm_stable_key_sort_static_capacity(void);
+int cm_stable_key_sort_static(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm,
+                              int32_t *offsets, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Invariant message passing, forward.
  * Replaces jit_forward_message_passing (jit_wrappers/src/invariant_message_passing_wrapper.cpp:72-155)
  * and inv_tp_kernel_ptr (cuda/src/invariant_message_passing_impl.cu:74-165).
