@@ -27,8 +27,17 @@ Pin status of each function (what fixes it besides its own formula):
                           replication of the cell into a non-periodic cluster
                           searched by a non-periodic cKDTree (small cells,
                           several images of a pair), (i,j,S) <-> (j,i,-S)
-  reference model         rotation / translation / permutation invariance,
-                          F = -dE/dx by central differences, sum F = 0;
-                          equality with upstream mace on a real checkpoint is
-                          PARITY UNPINNED for the same reason
+  reference model         message passing, linears and readouts are the op
+                          definitions above; Bessel basis by orthonormality
+                          under r^2 dr (quadrature); envelope by its boundary
+                          conditions f(0)=1, f(1)=f'(1)=f''(1)=0; activation
+                          constant by the seeded Monte-Carlo recipe and
+                          Gauss-Hermite quadrature; 1/sqrt(fan_in) by unit
+                          second moments; nested contraction vs the dense
+                          brute-force-pinned form; one- and two-atom closed
+                          forms; rotation / translation / permutation
+                          invariance, F = -dE/dx by central differences;
+                          equality with upstream mace on a real checkpoint
+                          (U path order/sign, e3nn flat weight order) is
+                          PARITY UNPINNED: upstream is not available offline
 """

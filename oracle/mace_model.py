@@ -14,7 +14,11 @@ pos[receiver] - pos[sender] + shift.  The reference swaps sender and receiver (m
 which flips the sign of odd-l message components and leaves energies and forces unchanged.
 
 Equality with upstream mace on a trained checkpoint is PARITY UNPINNED (upstream unavailable offline).
-What pins this file: invariances and F = -dE/dx finite differences in tests/test_oracle_model.py.
+What pins this file (tests/test_oracle_model.py): message passing, per-l / per-element linears and readouts are the
+op definitions of oracle/ops.py (each pinned there); Bessel orthonormality by quadrature; the envelope's boundary
+conditions; the activation constant by Gauss-Hermite quadrature; the 1/sqrt(fan_in) convention by the unit second
+moment of the radial network's output; the nested contraction against the brute-force-pinned dense form; invariances
+and F = -dE/dx finite differences of the whole.
 """
 from __future__ import annotations
 
@@ -29,13 +33,24 @@ from .u_tensors import u_tensors
 SILU_2MOM = 1.6791767923989418
 
 
-def radial_basis(r: torch.Tensor, r_max: float, num_bessel: int, p: int) -> torch.Tensor:
-    """[E] -> [E, num_bessel]: sqrt(2/r_max) sin(n pi r/r_max)/r times the polynomial cutoff envelope."""
+def bessel_basis(r: torch.Tensor, r_max: float, num_bessel: int) -> torch.Tensor:
+    """[E] -> [E, num_bessel]: b_n(r) = sqrt(2 / r_max) sin(n pi r / r_max) / r, n = 1..num_bessel; orthonormal on
+    [0, r_max] under the measure r^2 dr (pinned by quadrature in tests/test_oracle_model.py)."""
     n = torch.arange(1, num_bessel + 1, dtype=r.dtype)
-    bessel = math.sqrt(2.0 / r_max) * torch.sin(n * math.pi / r_max * r[:, None]) / r[:, None]
-    x = r / r_max
+    return math.sqrt(2.0 / r_max) * torch.sin(n * math.pi / r_max * r[:, None]) / r[:, None]
+
+
+def polynomial_cutoff(x: torch.Tensor, p: int) -> torch.Tensor:
+    """Envelope f(x) = 1 - (p+1)(p+2)/2 x^p + p(p+2) x^(p+1) - p(p+1)/2 x^(p+2) for x < 1, else 0: the polynomial
+    of that shape with f(0) = 1 and f(1) = f'(1) = f''(1) = 0 (those four conditions fix the three coefficients;
+    pinned in tests/test_oracle_model.py)."""
     env = 1.0 - (p + 1) * (p + 2) / 2.0 * x ** p + p * (p + 2.0) * x ** (p + 1) - p * (p + 1) / 2.0 * x ** (p + 2)
-    return bessel * (env * (x < 1.0).to(r.dtype))[:, None]
+    return env * (x < 1.0).to(x.dtype)
+
+
+def radial_basis(r: torch.Tensor, r_max: float, num_bessel: int, p: int) -> torch.Tensor:
+    """[E] -> [E, num_bessel]: Bessel functions times the polynomial cutoff envelope."""
+    return bessel_basis(r, r_max, num_bessel) * polynomial_cutoff(r / r_max, p)[:, None]
 
 
 def radial_mlp(feats: torch.Tensor, weights) -> torch.Tensor:
@@ -81,7 +96,6 @@ def energy_and_forces(params: Dict[str, object], data: Dict[str, torch.Tensor], 
 
     node_e0 = attrs @ params["E0"].to(dtype)
     h = attrs @ params["W_emb"].to(dtype) / math.sqrt(ne)
-    node_es = torch.zeros(N, dtype=dtype)
     feats = []
     for t, lay in enumerate(params["layers"]):
         sc = None
@@ -89,23 +103,24 @@ def energy_and_forces(params: Dict[str, object], data: Dict[str, torch.Tensor], 
             sc = torch.einsum("nu,ne,uew->nw", h, attrs, lay["W_skip"][0].to(dtype)) / math.sqrt(C * ne)
         u = h @ lay["W_up"].to(dtype) / math.sqrt(C)
         R = radial_mlp(basis, lay["mlp"]).view(-1, 4, C)
-        msg = u[snd][:, None, :] * Y[:, :, None] * R[:, O.L_OF_M, :]  # [E, 16, C]
-        A = torch.zeros(N, 16, C, dtype=dtype).index_add(0, rcv, msg)
-        A = torch.einsum("nmk,mkj->nmj", A, lay["W_lin"].to(dtype)[O.L_OF_M]) / math.sqrt(C) / float(lay["avg_num_neighbors"])
+        # per-edge tensor product and scatter-sum over receivers: the op definition pinned in oracle/ops.py
+        A = O.mp_forward(u, Y.t(), R, snd, rcv, N)
+        A = O.linear(A, lay["W_lin"].to(dtype)) / float(lay["avg_num_neighbors"])
         if t == 0:
-            Wsk = lay["W_skip"].to(dtype)[O.L_OF_M]  # [16, C, ne, C]
-            A = torch.einsum("nmu,ne,muew->nmw", A, attrs, Wsk) / math.sqrt(C * ne)
+            # per-element linear: blocks W_skip[l][:, e, :] with 1/sqrt(ne) folded in (models/InvariantMACE.py:61-64),
+            # 1/sqrt(C) applied by the op
+            Wsk = lay["W_skip"].to(dtype).permute(2, 0, 1, 3) / math.sqrt(ne)  # [ne, 4, C, C]
+            A = O.elemental_linear(A, Wsk, attrs)
         B = contraction_nested(A, elem, lay["W3"], lay["W2"], lay["W1"], U3, U2)
         h = B @ lay["W_prod"].to(dtype) / math.sqrt(C)
         if sc is not None:
             h = h + sc
         feats.append(h)
-        if t == 0:
-            node_es = node_es + (h @ params["w_read0"].to(dtype) / math.sqrt(C)).squeeze(1)
-        else:
-            hid = SILU_2MOM * torch.nn.functional.silu(h @ params["W_read1"].to(dtype) / math.sqrt(C))
-            node_es = node_es + (hid @ params["w_read2"].to(dtype) / math.sqrt(hid.shape[1])).squeeze(1)
-    node_inter = float(params["scale"]) * node_es + float(params["shift"])
+    hidden = params["W_read1"].shape[1]
+    node_inter = O.readout_energies(feats[0], feats[1], params["w_read0"].to(dtype)[:, 0] / math.sqrt(C),
+                                    params["W_read1"].to(dtype) / math.sqrt(C),
+                                    params["w_read2"].to(dtype)[:, 0] / math.sqrt(hidden), SILU_2MOM,
+                                    float(params["scale"]), float(params["shift"]))
     inter_e = node_inter.sum().view(1)
     forces = None
     if compute_forces:

@@ -113,3 +113,179 @@ def test_periodic_images_are_equivalent():
     out = M.energy_and_forces(params, d2)
     torch.testing.assert_close(out["energy"], base["energy"], rtol=1e-10, atol=1e-10)
     torch.testing.assert_close(out["forces"], base["forces"], rtol=1e-8, atol=1e-9)
+
+
+# ---- pins of the model-level helpers: each fails when the constant it names is off by 1 % ------------------------
+def test_bessel_basis_is_orthonormal_under_r2_dr():
+    """int_0^rmax b_n(r) b_m(r) r^2 dr = delta_nm fixes the prefactor sqrt(2 / r_max) and the frequencies n pi / r_max."""
+    r_max, nb = 5.0, 8
+    x, w = np.polynomial.legendre.leggauss(400)
+    r = torch.tensor(0.5 * r_max * (x + 1.0))
+    w = torch.tensor(0.5 * r_max * w)
+    b = M.bessel_basis(r, r_max, nb)
+    gram = torch.einsum("e,en,em->nm", w * r * r, b, b)
+    torch.testing.assert_close(gram, torch.eye(nb, dtype=torch.float64), atol=1e-12, rtol=0)
+    # first zero of every b_n at r_max / n (sin(n pi r / r_max) = 0), and b_n -> sqrt(2 / r_max) n pi / r_max at r -> 0
+    n = torch.arange(1, nb + 1, dtype=torch.float64)
+    b0 = M.bessel_basis(torch.tensor([1e-9], dtype=torch.float64), r_max, nb)[0]
+    torch.testing.assert_close(b0, math.sqrt(2.0 / r_max) * n * math.pi / r_max, rtol=1e-9, atol=0)
+
+
+@pytest.mark.parametrize("p", [5, 6])
+def test_polynomial_cutoff_boundary_conditions(p):
+    """f(0) = 1, f(1) = f'(1) = f''(1) = 0 determine the three coefficients of 1 - a x^p + b x^(p+1) - c x^(p+2)."""
+    x = torch.tensor([1.0 - 1e-300], dtype=torch.float64, requires_grad=True)  # just inside the cutoff
+    f = M.polynomial_cutoff(x, p)
+    (d1,) = torch.autograd.grad(f.sum(), x, create_graph=True)
+    (d2,) = torch.autograd.grad(d1.sum(), x)
+    assert abs(float(f)) < 1e-12 and abs(float(d1)) < 1e-11 and abs(float(d2)) < 1e-10
+    z = torch.tensor([0.0, 1.0, 1.5], dtype=torch.float64)
+    torch.testing.assert_close(M.polynomial_cutoff(z, p), torch.tensor([1.0, 0.0, 0.0], dtype=torch.float64))
+    # independent solve of the 3 x 3 system for (a, b, c)
+    A = np.array([[1.0, 1.0, 1.0], [p, p + 1, p + 2], [p * (p - 1), (p + 1) * p, (p + 2) * (p + 1)]])
+    a, b, c = np.linalg.solve(A, np.array([-1.0, 0.0, 0.0]))
+    xs = torch.linspace(0.05, 0.95, 7, dtype=torch.float64)
+    want = 1.0 + a * xs ** p + b * xs ** (p + 1) + c * xs ** (p + 2)
+    torch.testing.assert_close(M.polynomial_cutoff(xs, p), want, rtol=1e-10, atol=1e-12)
+
+
+def _silu_second_moment():
+    x, w = np.polynomial.hermite_e.hermegauss(200)
+    silu = x / (1.0 + np.exp(-x))
+    return float((w * silu ** 2).sum() / math.sqrt(2.0 * math.pi))
+
+
+def test_activation_constant_normalises_the_second_moment():
+    """SILU_2MOM^2 E_{z ~ N(0,1)}[silu(z)^2] = 1 (the normalize2mom convention).  Upstream's constant is a Monte-Carlo
+    estimate over 10^6 seeded fp64 normals, which this recipe reproduces to the last digit; it lies 0.16 % from the
+    exact value 1.67653 that Gauss-Hermite quadrature gives."""
+    z = torch.randn(1_000_000, generator=torch.Generator().manual_seed(0), dtype=torch.float64)
+    mc = 1.0 / math.sqrt(float((torch.nn.functional.silu(z) ** 2).mean()))
+    assert abs(mc - M.SILU_2MOM) < 1e-14
+    assert abs(M.SILU_2MOM ** 2 * _silu_second_moment() - 1.0) < 5e-3
+
+
+def test_radial_mlp_keeps_unit_second_moment():
+    """Unit-variance weights and inputs of unit second moment give outputs of second moment SILU_2MOM^2 E[silu^2]
+    (= 1.003) and zero mean: fixes the 1/sqrt(fan_in) of every layer (1 % off moves the result by 4 %), the activation
+    constant (2 %) and that the last layer is linear (a gated output would have mean 0.35).  Wide layers keep the
+    finite-width bias and the sampling noise at 0.3 % each."""
+    g = torch.Generator().manual_seed(0)
+    widths = [1024, 1024, 4096]
+    x = torch.randn(2000, widths[0], generator=g, dtype=torch.float64)
+    x = x / x.norm(dim=1, keepdim=True) * math.sqrt(widths[0])
+    Ws = [torch.randn(a, b, generator=g, dtype=torch.float64) for a, b in zip(widths[:-1], widths[1:])]
+    out = M.radial_mlp(x, Ws)
+    want = M.SILU_2MOM ** 2 * _silu_second_moment()
+    assert abs(float((out ** 2).mean()) - want) < 0.01, float((out ** 2).mean())
+    assert abs(float(out.mean())) < 0.03
+    # a single layer is a plain scaled product: second moment |x|^2 / fan_in exactly in expectation
+    one = M.radial_mlp(x[:50], [Ws[1]])
+    assert abs(float((one ** 2).mean()) - 1.0) < 0.01
+
+
+def test_nested_contraction_equals_dense_definition():
+    """contraction_nested (the form the model evaluates) against oracle.ops.symmetric_contraction, which
+    tests/test_oracle_pins.py pins by python-loop brute force."""
+    from oracle import ops as O
+    from oracle.u_tensors import u_tensors
+
+    g = torch.Generator().manual_seed(3)
+    N, C, ne = 13, 5, 3
+    U1, U2, U3 = (torch.from_numpy(u) for u in u_tensors())
+    X = torch.randn(N, 16, C, generator=g, dtype=torch.float64)
+    elem = torch.randint(0, ne, (N,), generator=g)
+    W3 = torch.randn(ne, U3.shape[-1], C, generator=g, dtype=torch.float64)
+    W2 = torch.randn(ne, U2.shape[-1], C, generator=g, dtype=torch.float64)
+    W1 = torch.randn(ne, 1, C, generator=g, dtype=torch.float64)
+    got = M.contraction_nested(X, elem, W3, W2, W1, U3, U2)
+    want = O.symmetric_contraction(X, elem, U3, U2, W3, W2, W1)
+    torch.testing.assert_close(got, want, rtol=1e-11, atol=1e-11)
+
+
+def test_message_has_unit_path_weight(setup):
+    """The per-edge product carries no factor besides u[sender] Y R (path weight 1 of the uvu tensor product, as in the
+    reference's own check, tests/invariant_message_passing.py:93-120): for one edge, one channel and R = 1 the
+    aggregated message on the receiver is exactly u * Y(r), with Y_00 = 1 and sum_m Y_1m^2 = 3."""
+    from oracle import ops as O
+
+    vec = torch.tensor([[0.3, -1.1, 0.7]], dtype=torch.float64)
+    Y = O.spherical_harmonics(vec)  # [16, 1]
+    u = torch.tensor([[2.0], [0.0]], dtype=torch.float64)
+    A = O.mp_forward(u, Y, torch.ones(1, 4, 1, dtype=torch.float64), torch.tensor([0]), torch.tensor([1]), 2)
+    torch.testing.assert_close(A[1, :, 0], 2.0 * Y[:, 0])
+    assert float(A[0].abs().max()) == 0.0
+    assert abs(float(Y[0, 0]) - 1.0) < 1e-14 and abs(float((Y[1:4, 0] ** 2).sum()) - 3.0) < 1e-13
+
+
+def test_single_atom_energy_is_closed_form():
+    """An isolated atom receives no messages: A = 0, so B = 0 (every contraction term is at least linear in A), h1 = 0,
+    the layer-2 skip connection (a function of h1) is 0 and h2 = 0; silu(0) = 0, so both readouts vanish and the energy
+    is E0[element] + shift exactly, whatever the weights and the scale."""
+    e0 = torch.tensor([-13.6, -1029.0, -1485.0, -2042.0], dtype=torch.float64)
+    model = SyntheticInvariantMACE(channels=32, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=9.0, seed=0,
+                                   atomic_energies=e0, scale=0.7, shift=0.25)
+    p = model.export_params()
+    for e in (0, 2):
+        attrs = torch.zeros(1, 4, dtype=torch.float64)
+        attrs[0, e] = 1.0
+        data = dict(positions=torch.zeros(1, 3, dtype=torch.float64), node_attrs=attrs,
+                    edge_index=torch.zeros(2, 0, dtype=torch.long), shifts=torch.zeros(0, 3, dtype=torch.float64))
+        out = M.energy_and_forces(p, data, compute_forces=False)
+        assert abs(float(out["energy"]) - (float(e0[e]) + 0.25)) < 1e-12
+        assert abs(float(out["interaction_energy"]) - 0.25) < 1e-15
+
+
+def test_two_atom_energy_is_closed_form():
+    """Two atoms at distance d along z, one channel per l that matters: with Y(z-axis) known in closed form (Y_l0 =
+    sqrt(2l+1), every other component 0) the whole first layer is a hand-computable scalar chain.  Checks the chain
+    radial basis -> MLP -> message -> 1/avg_num_neighbors -> linear -> per-element linear -> contraction -> product
+    linear -> linear readout, with independent arithmetic (numpy, explicit loops over the 16 components)."""
+    model = SyntheticInvariantMACE(channels=32, atomic_numbers=(1, 6), avg_num_neighbors=3.0, seed=5)
+    p = model.export_params()
+    C, ne, d = 32, 2, 1.7
+    attrs = torch.tensor([[1.0, 0.0], [0.0, 1.0]], dtype=torch.float64)
+    pos = torch.tensor([[0.0, 0.0, 0.0], [0.0, 0.0, d]], dtype=torch.float64)
+    data = dict(positions=pos, node_attrs=attrs, edge_index=torch.tensor([[0, 1], [1, 0]]),
+                shifts=torch.zeros(2, 3, dtype=torch.float64))
+    out = M.energy_and_forces(p, data, compute_forces=False)
+    from oracle import ops as O
+    from oracle.u_tensors import u_tensors
+
+    U1, U2, U3 = u_tensors()
+    lay = p["layers"][0]
+    r_max, nb, pw = float(p["r_max"]), int(p["num_bessel"]), int(p["p"])
+    x = d / r_max
+    env = 1 - (pw + 1) * (pw + 2) / 2 * x ** pw + pw * (pw + 2) * x ** (pw + 1) - pw * (pw + 1) / 2 * x ** (pw + 2)
+    basis = np.array([math.sqrt(2 / r_max) * math.sin(n * math.pi * d / r_max) / d * env for n in range(1, nb + 1)])
+    z = basis
+    mlp = [W.double().numpy() for W in lay["mlp"]]
+    for i, W in enumerate(mlp):
+        z = z @ W / math.sqrt(W.shape[0])
+        if i + 1 < len(mlp):
+            z = M.SILU_2MOM * z / (1 + np.exp(-z))
+    R = z.reshape(4, C)
+    h0 = (attrs @ p["W_emb"].double() / math.sqrt(ne)).numpy()
+    u = h0 @ lay["W_up"].double().numpy() / math.sqrt(C)
+    h1 = np.zeros((2, C))
+    W_lin, W_skip = lay["W_lin"].double().numpy(), lay["W_skip"].double().numpy()
+    for rcv, snd, sign in ((1, 0, +1.0), (0, 1, -1.0)):  # edge vector = pos[rcv] - pos[snd] = +-d along the 3rd axis
+        # harmonics of +-z in the oracle's component order, taken from the scipy-pinned routine
+        Y = O.spherical_harmonics(torch.tensor([[0.0, 0.0, sign * d]], dtype=torch.float64))[:, 0].numpy()
+        A = np.zeros((16, C))
+        for m in range(16):
+            l = int(math.isqrt(m))
+            msg = u[snd] * Y[m] * R[l]
+            A[m] = (msg @ W_lin[l]) / math.sqrt(C) / 3.0
+            A[m] = (A[m] @ W_skip[l][:, rcv, :]) / math.sqrt(C * ne)  # element of atom rcv is rcv
+        e = rcv
+        B = np.zeros(C)
+        W3, W2, W1 = (lay[k].double().numpy()[e] for k in ("W3", "W2", "W1"))
+        for c in range(C):
+            a = A[:, c]
+            B[c] = np.einsum("ijkp,p,i,j,k->", U3, W3[:, c], a, a, a) + np.einsum("ijp,p,i,j->", U2, W2[:, c], a, a) + W1[0, c] * a[0]
+        h1[rcv] = B @ lay["W_prod"].double().numpy() / math.sqrt(C)
+    e1 = h1 @ p["w_read0"].double().numpy()[:, 0] / math.sqrt(C)
+    got1 = out["node_feats"][:, :C].numpy()
+    np.testing.assert_allclose(got1, h1, rtol=1e-10, atol=1e-13)
+    assert np.abs(h1).max() > 1e-4 and np.abs(e1).max() > 1e-6
