@@ -175,8 +175,12 @@ class _ScaleShift(torch.nn.Module):
 class _Contraction(torch.nn.Module):
     """Weight holder of one output irrep: weights_max [ne, 23, C] (order 3), weights = [[ne, 4, C], [ne, 1, C]]."""
 
-    def __init__(self, num_elements: int, channels: int, generator: torch.Generator):
+    def __init__(self, num_elements: int, channels: int, generator: torch.Generator, coupling=None):
         super().__init__()
+        if coupling is not None:
+            # upstream's contraction modules keep the coupling tensors their weights refer to as buffers of these names
+            for nu, U in zip((1, 2, 3), coupling):
+                self.register_buffer("U_matrix_%d" % nu, U.clone())
         self.weights_max = torch.nn.Parameter(torch.randn(num_elements, 23, channels, generator=generator, dtype=torch.float64) / 23)
         self.weights = torch.nn.ParameterList([
             torch.nn.Parameter(torch.randn(num_elements, 4, channels, generator=generator, dtype=torch.float64) / 4),
@@ -184,20 +188,37 @@ class _Contraction(torch.nn.Module):
         ])
 
 
+def permuted_coupling_basis(seed: int):
+    """(U1, U2, U3) of ops/u_matrix.py with the paths of U2 and U3 in a seeded random order and with seeded random
+    signs: another valid basis of the same invariants, as a model trained elsewhere may carry."""
+    import numpy as np
+
+    from ..ops.u_matrix import _u_tensors_np
+
+    U1, U2, U3 = _u_tensors_np()
+    rng = np.random.default_rng(seed)
+    out = [torch.from_numpy(U1.copy())]
+    for U in (U2, U3):
+        order = rng.permutation(U.shape[-1])
+        signs = rng.choice(np.array([-1.0, 1.0]), size=U.shape[-1])
+        out.append(torch.from_numpy(U[..., order] * signs))
+    return tuple(out)
+
+
 class _SymmetricContraction(torch.nn.Module):
-    def __init__(self, channels: int, num_elements: int, generator: torch.Generator):
+    def __init__(self, channels: int, num_elements: int, generator: torch.Generator, coupling=None):
         super().__init__()
         self.irreps_in = Irreps("+".join("%dx%d%s" % (channels, l, "eo"[l % 2]) for l in range(4)))
         self.irreps_out = Irreps("%dx0e" % channels)
-        self.contractions = torch.nn.ModuleList([_Contraction(num_elements, channels, generator)])
+        self.contractions = torch.nn.ModuleList([_Contraction(num_elements, channels, generator, coupling)])
 
 
 class _ProductBasis(torch.nn.Module):
     """EquivariantProductBasisBlock: symmetric contraction, linear, optional residual."""
 
-    def __init__(self, channels: int, num_elements: int, use_sc: bool, generator: torch.Generator):
+    def __init__(self, channels: int, num_elements: int, use_sc: bool, generator: torch.Generator, coupling=None):
         super().__init__()
-        self.symmetric_contractions = _SymmetricContraction(channels, num_elements, generator)
+        self.symmetric_contractions = _SymmetricContraction(channels, num_elements, generator, coupling)
         self.linear = _Linear0e(channels, channels, generator)
         self.use_sc = use_sc
 
@@ -225,9 +246,12 @@ class SyntheticInvariantMACE(torch.nn.Module):
     def __init__(self, channels: int = 128, atomic_numbers=(1, 6, 7, 8), r_max: float = 5.0, num_bessel: int = 8,
                  num_polynomial_cutoff: int = 5, radial_mlp=(64, 64, 64), mlp_hidden: int = 16,
                  avg_num_neighbors: float = 1.0, atomic_energies: Optional[torch.Tensor] = None, scale: float = 1.0,
-                 shift: float = 0.0, seed: int = 0):
+                 shift: float = 0.0, seed: int = 0, coupling_basis_seed: Optional[int] = None):
+        """coupling_basis_seed: when given, the contraction modules carry `U_matrix_1/2/3` buffers (as upstream's do)
+        holding a permuted, sign-flipped path basis, and their weights refer to that basis."""
         super().__init__()
         g = torch.Generator().manual_seed(seed)
+        coupling = None if coupling_basis_seed is None else permuted_coupling_basis(coupling_basis_seed)
         ne = len(atomic_numbers)
         self.channels, self.num_elements = channels, ne
         self.register_buffer("atomic_numbers", torch.tensor(list(atomic_numbers), dtype=torch.int64))
@@ -241,7 +265,8 @@ class SyntheticInvariantMACE(torch.nn.Module):
             _Interaction(channels, ne, num_bessel, list(radial_mlp), False, avg_num_neighbors, g),
             _Interaction(channels, ne, num_bessel, list(radial_mlp), True, avg_num_neighbors, g),
         ])
-        self.products = torch.nn.ModuleList([_ProductBasis(channels, ne, False, g), _ProductBasis(channels, ne, True, g)])
+        self.products = torch.nn.ModuleList([_ProductBasis(channels, ne, False, g, coupling),
+                                             _ProductBasis(channels, ne, True, g, coupling)])
         self.readouts = torch.nn.ModuleList([_LinearReadout(channels, g), _NonLinearReadout(channels, mlp_hidden, g)])
         self.scale_shift = _ScaleShift(scale, shift)
 
@@ -262,6 +287,8 @@ class SyntheticInvariantMACE(torch.nn.Module):
                 W_prod=pr.linear.weight.detach().view(C, C).clone(),
                 avg_num_neighbors=it.avg_num_neighbors,
             ))
+            if hasattr(con, "U_matrix_3"):  # the basis the weights refer to, when the module carries one
+                layers[-1].update(U2=con.U_matrix_2.detach().clone(), U3=con.U_matrix_3.detach().clone())
         ro0, ro1 = self.readouts
         return dict(
             channels=C, num_elements=ne, r_max=float(self.r_max), num_bessel=self.radial_embedding.out_dim,

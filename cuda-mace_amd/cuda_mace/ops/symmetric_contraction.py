@@ -5,6 +5,56 @@ from . import classes
 from .u_matrix import U_matrix_real
 
 
+U_ZERO = 1e-10  # coupling coefficients below this are rounding residue of a change of basis, not couplings
+
+
+def coupling_tensors_of(symm_contract, correlation: int = 3):
+    """{nu: fp64 tensor [16]*nu + [paths]} for nu = 1..correlation.
+
+    The weights of a trained model multiply the coupling paths in the order and with the signs of the basis they were
+    trained in.  The reference takes that basis from upstream's `U_matrix_real` (ops/symmetric_contraction.py:29-34);
+    upstream's contraction modules keep the very same tensors as buffers `U_matrix_1`, `U_matrix_2`, `U_matrix_3`
+    next to the weights, so they are read from there when the module has them (a leading axis of length 1, as a
+    single scalar output can carry, is dropped).  Only a module without such buffers gets the tensors of
+    `ops/u_matrix.py`, whose path order and signs are this package's own."""
+    con = symm_contract.contractions[0]
+    found = {nu: getattr(con, "U_matrix_%d" % nu, None) for nu in range(1, correlation + 1)}
+    have = [nu for nu, U in found.items() if U is not None]
+    if have and len(have) != correlation:
+        raise ValueError("the contraction module has coupling buffers for orders %s only; need 1..%d" % (have, correlation))
+    out = {}
+    for nu in range(1, correlation + 1):
+        if have:
+            U = found[nu].detach().to("cpu", torch.float64)
+            while U.dim() > nu + 1 and U.shape[0] == 1:
+                U = U[0]
+            U = torch.where(U.abs() < U_ZERO, torch.zeros_like(U), U)
+        else:
+            U = U_matrix_real(irreps_in=symm_contract.irreps_in, irreps_out="0e", correlation=nu, dtype=torch.float64)[-1]
+        out[nu] = U
+    return out
+
+
+def check_coupling_tensor(U: torch.Tensor, nu: int, num_weight_paths: int) -> None:
+    """What the packed tables and the kernels assume of a coupling tensor, whatever its source: shape [16]*nu +
+    [paths] with as many paths as the weights have, at most one path per index tuple (the packed word has room for
+    one), and unit Frobenius norm per path (the normalisation under which upstream's weights are trained; a tensor
+    that fails it is most likely not a coupling tensor of this model)."""
+    if tuple(U.shape[:-1]) != (16,) * nu:
+        raise ValueError("coupling tensor of order %d has shape %s, expected %s + [paths]" % (nu, tuple(U.shape), [16] * nu))
+    if U.shape[-1] != num_weight_paths:
+        raise ValueError("coupling tensor of order %d has %d paths, the weights have %d" % (nu, U.shape[-1], num_weight_paths))
+    if int((U != 0).sum(-1).max()) > 1:
+        raise ValueError("coupling tensor of order %d couples one index tuple through several paths" % nu)
+    if nu == 1 and not (float(U[0, 0]) == 1.0 and int((U != 0).sum()) == 1):
+        # the kernels apply the order-1 weights to component 0 with coefficient 1, as the reference's do
+        # (cuda/src/symmetric_contraction_impl.cu:113-117)
+        raise ValueError("coupling tensor of order 1 must be the unit vector of component 0")
+    norms = (U.double() ** 2).sum(dim=tuple(range(nu))).sqrt()
+    if not torch.allclose(norms, torch.ones_like(norms), atol=1e-5):
+        raise ValueError("coupling tensor of order %d: paths must have unit Frobenius norm, found %s" % (nu, norms.tolist()))
+
+
 class SymmetricContraction(torch.nn.Module):
     """Correlation-3 symmetric contraction to a scalar per channel:  x [nnodes, 16, C], atom_types int32
     [nnodes] -> [nnodes, 1, C].
@@ -34,10 +84,7 @@ class SymmetricContraction(torch.nn.Module):
         self.nlout = (self.irreps_out.lmax + 1) ** 2
         assert self.nlout == 1, "only a scalar (0e) output is supported"
 
-        self.U_matrices = {
-            nu: {0: U_matrix_real(irreps_in=self.irreps_in, irreps_out="0e", correlation=nu, dtype=torch.float64)[-1]}
-            for nu in range(1, self.correlation + 1)
-        }
+        self.U_matrices = {nu: {0: U} for nu, U in coupling_tensors_of(symm_contract, self.correlation).items()}
         self.W_tensors = {}
         for j in range(len(symm_contract.contractions)):
             con = symm_contract.contractions[j]
@@ -46,6 +93,8 @@ class SymmetricContraction(torch.nn.Module):
                 2: con.weights[0].detach().clone().type(torch.float32),
                 1: con.weights[1].detach().clone().type(torch.float32),
             }
+        for nu in (1, 2, 3):
+            check_coupling_tensor(self.U_matrices[nu][0], nu, int(self.W_tensors["0"][nu].shape[-2]))
         self.setup_sparse_matrices()
         self.setup_weights()
 

@@ -111,7 +111,10 @@ def energy_and_forces(params: Dict[str, object], data: Dict[str, torch.Tensor], 
             # 1/sqrt(C) applied by the op
             Wsk = lay["W_skip"].to(dtype).permute(2, 0, 1, 3) / math.sqrt(ne)  # [ne, 4, C, C]
             A = O.elemental_linear(A, Wsk, attrs)
-        B = contraction_nested(A, elem, lay["W3"], lay["W2"], lay["W1"], U3, U2)
+        # a layer may name the coupling basis its weights refer to; otherwise the oracle's own derivation
+        U3l = lay["U3"].to(dtype) if "U3" in lay else U3
+        U2l = lay["U2"].to(dtype) if "U2" in lay else U2
+        B = contraction_nested(A, elem, lay["W3"], lay["W2"], lay["W1"], U3l, U2l)
         h = B @ lay["W_prod"].to(dtype) / math.sqrt(C)
         if sc is not None:
             h = h + sc

@@ -9,6 +9,7 @@ import torch
 
 from cuda_mace.utils.synthetic import make_system, to_device
 from oracle import mace_model as M
+from tests.util import carve_cluster as _carve
 
 pytestmark = pytest.mark.gpu
 
@@ -240,3 +241,72 @@ def test_config5_full_size_properties(cabi):
     _say("  E %.10g translated %.10g rel %.2e" % (e0, e1, abs(e0 - e1) / abs(e0)))
     assert abs(e0 - e1) <= 2e-6 * abs(e0)
     assert float((c["forces"].detach() - a["forces"].detach()).abs().max()) <= 2e-5 * max(fmax, 1.0)
+
+
+# ---- oracle parity at the full sizes of configurations 4 and 5 ------------------------------------------------------
+def _check_against_carved_clusters(params, data, out, centres, cutoff=5.0):
+    node_e = out["node_energy"].detach().double().cpu()
+    forces = out["forces"].detach().double().cpu()
+    worst_e, worst_f, checked = 0.0, 0.0, 0
+    for centre in centres:
+        cluster, keep, cdist = _carve(data, int(centre), 4 * cutoff, 3 * cutoff, cutoff)
+        ref = M.energy_and_forces(params, cluster)
+        inner = np.flatnonzero(cdist < 2 * cutoff - 1e-9)  # nodes whose energy is exact in the cluster
+        e_ref = ref["node_energy"][inner]
+        e_got = node_e[keep[inner]]
+        scale = float(e_ref.abs().max())
+        err_e = float((e_got - e_ref).abs().max()) / scale
+        me = int(np.flatnonzero(keep == centre)[0])
+        err_f = float((forces[centre] - ref["forces"][me]).abs().max())
+        _say("  atom %6d: cluster of %d atoms, %d edges; %d node energies max err %.2e of max |E_n| = %.3g; |dF| %.2e (|F| %.3g)"
+             % (centre, keep.size, cluster["edge_index"].shape[1], inner.size, err_e, scale, err_f,
+                float(ref["forces"][me].abs().max())))
+        assert err_e <= E_RTOL, (centre, err_e)
+        assert err_f <= F_ATOL, (centre, err_f)
+        worst_e, worst_f, checked = max(worst_e, err_e), max(worst_f, err_f), checked + inner.size
+    return worst_e, worst_f, checked
+
+
+def test_config4_full_size_against_reference_clusters(cabi):
+    """Benchmark configuration 4 at its real size (25 000 atoms, 128 channels, 1.3 M edges): node energies of about 400
+    atoms around each of several centres and the force on every centre against the fp64 reference evaluated on the
+    carved neighbourhoods.  Centres include the first and last atom and atoms at both ends of the box."""
+    _say("model c4 vs reference clusters")
+    data = make_system(25000, 10, seed=0, density=0.1)
+    params, model = _build(128, tuple(range(1, 11)), data, seed=0)
+    out = model(to_device(data, "cuda"))
+    centres = [0, 24999] + np.random.default_rng(1).integers(0, 25000, 3).tolist()
+    worst_e, worst_f, checked = _check_against_carved_clusters(params, data, out, centres)
+    _say("  c4: %d node energies within %.2e, %d forces within %.2e" % (checked, worst_e, len(centres), worst_f))
+
+
+def test_config5_full_size_against_reference_clusters(cabi):
+    """Benchmark configuration 5 at its real size (100 000 atoms, 192 channels, 5.2 M edges), as above."""
+    _say("model c5 vs reference clusters")
+    data = make_system(100000, 10, seed=0, density=0.1)
+    params, model = _build(192, tuple(range(1, 11)), data, seed=0)
+    out = model(to_device(data, "cuda"))
+    centres = [0, 99999] + np.random.default_rng(2).integers(0, 100000, 2).tolist()
+    worst_e, worst_f, checked = _check_against_carved_clusters(params, data, out, centres)
+    _say("  c5: %d node energies within %.2e, %d forces within %.2e" % (checked, worst_e, len(centres), worst_f))
+
+
+def test_model_in_a_foreign_coupling_basis(cabi):
+    """A source model whose contraction modules carry their own coupling tensors (upstream's U_matrix buffers) in a
+    permuted, sign-flipped path basis: the converted model follows that basis, and matches the fp64 reference fed the
+    same tensors, in the fused and in the separate-op contraction."""
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+
+    data = make_system(300, 4, seed=8, density=0.1)
+    avg = data["edge_index"].shape[1] / 300
+    up = SyntheticInvariantMACE(channels=64, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=avg, seed=6, coupling_basis_seed=5)
+    params = up.export_params()
+    assert "U3" in params["layers"][0]
+    for fused_contraction in (True, False):
+        model = OptimizedInvariantMACE(up, device="cuda", fused_contraction=fused_contraction)
+        _compare(params, model, data)
+    # the same weights read in the package's own basis give another model: the buffers matter
+    own = SyntheticInvariantMACE(channels=64, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=avg, seed=6)
+    ref_own = M.energy_and_forces(own.export_params(), data)
+    ref = M.energy_and_forces(params, data)
+    assert abs(float(ref_own["interaction_energy"]) - float(ref["interaction_energy"])) > 1e-3 * abs(float(ref["interaction_energy"]))

@@ -63,6 +63,7 @@ MP_CASES = [
     (60, 10, 224, "poisson", 0.0, 7),
     (80, 25, 256, "poisson", 0.3, 8),
     (3, 1, 128, "fixed", 0.0, 9),
+    (4096, 30, 96, "fixed", 0.0, 0),  # benchmark configuration 2 at its real size: 122 880 edges, uniform random senders
 ]
 
 

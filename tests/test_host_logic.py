@@ -119,3 +119,78 @@ def test_model_constructs_on_cpu_and_refuses_to_run_there():
     data = make_system(10, 4, seed=0, density=None, cluster_box=6.0)
     with pytest.raises(RuntimeError, match="GPU"):
         model(data)
+
+
+def test_contraction_tables_follow_the_coupling_basis_of_the_source_module():
+    """A contraction module that carries its own coupling tensors (upstream's `U_matrix_1/2/3` buffers) is packed in
+    that basis: with a permuted, sign-flipped path basis the packed tables unpack to exactly those tensors and the
+    monomial form reproduces the dense contraction evaluated with them -- and differs from the result in the
+    package's own basis, which the same weights would give if the buffers were ignored."""
+    from cuda_mace.models.upstream_like import _SymmetricContraction, permuted_coupling_basis
+    from cuda_mace.ops._autograd import monomials_from_packed
+    from cuda_mace.ops.symmetric_contraction import SymmetricContraction
+
+    basis = permuted_coupling_basis(7)
+    own = _SymmetricContraction(32, 3, torch.Generator().manual_seed(0))
+    up = _SymmetricContraction(32, 3, torch.Generator().manual_seed(0), coupling=basis)
+    assert hasattr(up.contractions[0], "U_matrix_3") and not hasattr(own.contractions[0], "U_matrix_3")
+    sc, sc_own = SymmetricContraction(up, device="cpu"), SymmetricContraction(own, device="cpu")
+    U3d, U2d = O.unpack_u_tables(sc.U3_num_nonsparse, sc.U3_indices, sc.U3_values, sc.U2_num_nonsparse, sc.U2_indices,
+                                 sc.U2_values, 23, 4)
+    np.testing.assert_allclose(U3d.numpy(), basis[2].numpy().astype(np.float32), atol=0)
+    np.testing.assert_allclose(U2d.numpy(), basis[1].numpy().astype(np.float32), atol=0)
+    assert not torch.equal(sc.U3_indices, sc_own.U3_indices)
+
+    g = torch.Generator().manual_seed(1)
+    X = torch.randn(6, 16, 32, generator=g, dtype=torch.float64)
+    types = torch.tensor([0, 2, 1, 1, 0, 2])
+    W3, W2, W1 = (w[0].double() for w in (sc.weights_3, sc.weights_2, sc.weights_1))
+    ref = O.symmetric_contraction(X, types, basis[2], basis[1], W3, W2, W1)
+    U1, U2, U3 = u_tensors()
+    other = O.symmetric_contraction(X, types, torch.from_numpy(U3), torch.from_numpy(U2), W3, W2, W1)
+    assert float((ref - other).abs().max()) > 1e-2
+
+    def monomial_form(mod):
+        (m3, o3, p3, v3), (m2, o2, p2, v2) = monomials_from_packed(mod.U3_num_nonsparse, mod.U3_indices, mod.U3_values,
+                                                                   mod.U2_num_nonsparse, mod.U2_indices, mod.U2_values)
+        out = W1[types][:, 0] * X[:, 0]
+        for t in range(len(m3)):
+            i, j, k = m3[t] & 255, (m3[t] >> 8) & 255, (m3[t] >> 16) & 255
+            out = out + sum(float(v3[q]) * W3[types][:, int(p3[q])] for q in range(o3[t], o3[t + 1])) * X[:, i] * X[:, j] * X[:, k]
+        for t in range(len(m2)):
+            i, j = m2[t] & 255, (m2[t] >> 8) & 255
+            out = out + sum(float(v2[q]) * W2[types][:, int(p2[q])] for q in range(o2[t], o2[t + 1])) * X[:, i] * X[:, j]
+        return out
+
+    torch.testing.assert_close(monomial_form(sc), ref, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(monomial_form(sc_own), other, rtol=1e-6, atol=1e-6)
+
+
+def test_coupling_tensor_checks():
+    from cuda_mace.models.upstream_like import _SymmetricContraction, permuted_coupling_basis
+    from cuda_mace.ops.symmetric_contraction import SymmetricContraction, check_coupling_tensor, coupling_tensors_of
+
+    U1, U2, U3 = permuted_coupling_basis(0)
+    for nu, U, paths in ((1, U1, 1), (2, U2, 4), (3, U3, 23)):
+        check_coupling_tensor(U, nu, paths)
+    with pytest.raises(ValueError, match="unit Frobenius norm"):
+        check_coupling_tensor(U3 * 1.01, 3, 23)
+    with pytest.raises(ValueError, match="paths, the weights have"):
+        check_coupling_tensor(U3[..., :22], 3, 23)
+    two = U3.clone()
+    two[..., 1] = two[..., 0]
+    with pytest.raises(ValueError, match="several paths"):
+        check_coupling_tensor(two, 3, 23)
+    with pytest.raises(ValueError, match="order 1"):
+        check_coupling_tensor(-U1, 1, 1)
+    with pytest.raises(ValueError, match="shape"):
+        check_coupling_tensor(U3[:9], 3, 23)
+    # a leading axis of length one and rounding residue of a basis change are accepted when read from a module
+    up = _SymmetricContraction(32, 2, torch.Generator().manual_seed(0), coupling=(U1, U2, U3))
+    con = up.contractions[0]
+    con.U_matrix_3 = (U3 + 1e-17)[None]
+    got = coupling_tensors_of(up)
+    assert torch.equal(got[3] != 0, U3 != 0) and torch.allclose(got[3], U3, atol=1e-15, rtol=0) and torch.equal(got[2], U2)
+    del con.U_matrix_2
+    with pytest.raises(ValueError, match="orders"):
+        SymmetricContraction(up, device="cpu")

@@ -289,3 +289,31 @@ def test_two_atom_energy_is_closed_form():
     got1 = out["node_feats"][:, :C].numpy()
     np.testing.assert_allclose(got1, h1, rtol=1e-10, atol=1e-13)
     assert np.abs(h1).max() > 1e-4 and np.abs(e1).max() > 1e-6
+
+
+def test_carving_is_exact_on_the_reference_itself():
+    """The locality argument behind the carved clusters, checked on the CPU in fp64: node energies within two cutoffs
+    of the centre and the force on the centre, computed on the cluster, equal those of the whole periodic box."""
+    from tests.util import carve_cluster
+
+    cutoff = 1.8  # a short cutoff and a dense box keep 4 cutoffs inside half the box of a small system
+    data = make_system(1000, 3, seed=11, density=0.3, cutoff=cutoff)
+    up = SyntheticInvariantMACE(channels=32, atomic_numbers=(1, 6, 8), r_max=cutoff,
+                                avg_num_neighbors=data["edge_index"].shape[1] / 1000, seed=4)
+    params = up.export_params()
+    full = M.energy_and_forces(params, data)
+    teeth = 0.0
+    for centre in (0, 350, 999):
+        cluster, keep, cdist = carve_cluster(data, centre, 4 * cutoff, 3 * cutoff, cutoff)
+        assert keep.size < 600
+        ref = M.energy_and_forces(params, cluster)
+        inner = np.flatnonzero(cdist < 2 * cutoff - 1e-9)
+        assert inner.size >= 5
+        torch.testing.assert_close(ref["node_energy"][inner], full["node_energy"][keep[inner]], rtol=1e-10, atol=1e-12)
+        me = int(np.flatnonzero(keep == centre)[0])
+        torch.testing.assert_close(ref["forces"][me], full["forces"][centre], rtol=1e-9, atol=1e-11)
+        # a cluster that is too small fails the same comparison: the check has teeth
+        small, keep_s, _ = carve_cluster(data, centre, 2 * cutoff, 1.5 * cutoff, cutoff)
+        bad = M.energy_and_forces(params, small)
+        teeth += float((bad["forces"][int(np.flatnonzero(keep_s == centre)[0])] - full["forces"][centre]).abs().max())
+    assert teeth > 1e-5

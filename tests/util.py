@@ -32,3 +32,38 @@ def close(actual, expected, rtol, atol_scale):
     actual = actual.double().cpu()
     scale = float(expected.abs().max()) if expected.numel() else 1.0
     torch.testing.assert_close(actual, expected, rtol=rtol, atol=atol_scale * max(scale, 1e-30))
+
+
+def carve_cluster(data, centre, r_atoms, r_receivers, cutoff=5.0):
+    """The neighbourhood of atom `centre` of a periodic cubic box as a non-periodic cluster for the fp64 reference.
+
+    A two-layer model with cutoff rc is local: the energy of node n depends on atoms within 2 rc of n, so the force on
+    atom i depends on atoms within 4 rc of i.  The cluster holds every periodic image within r_atoms of the centre,
+    unwrapped, and every pair within the cutoff whose receiving end lies within r_receivers of the centre.  With
+    r_atoms = 4 rc and r_receivers = 3 rc the features of layer 1 are exact within 3 rc, node energies within 2 rc, and
+    the derivative of the cluster's energy with respect to the centre's position is the force of the full system
+    (nodes beyond 2 rc have wrong energies that do not depend on the centre).  Returns (cluster data, original index
+    of every cluster atom, distance of every cluster atom from the centre)."""
+    from scipy.spatial import cKDTree
+
+    pos = data["positions"].numpy()
+    box = float(data["cell"][0, 0])
+    assert box > 2 * r_atoms, "images must be unique inside the cluster"
+    d = pos - pos[centre]
+    d -= box * np.round(d / box)
+    dist = np.linalg.norm(d, axis=1)
+    keep = np.flatnonzero(dist < r_atoms)
+    cpos, cdist = d[keep], dist[keep]
+    pairs = cKDTree(cpos).query_pairs(cutoff, output_type="ndarray")
+    snd = np.concatenate([pairs[:, 0], pairs[:, 1]])
+    rcv = np.concatenate([pairs[:, 1], pairs[:, 0]])
+    live = cdist[rcv] < r_receivers
+    snd, rcv = snd[live], rcv[live]
+    order = np.lexsort((rcv, snd))
+    cluster = {
+        "positions": torch.from_numpy(cpos.copy()),
+        "node_attrs": data["node_attrs"][keep],
+        "edge_index": torch.from_numpy(np.stack([snd[order], rcv[order]]).astype(np.int64)),
+        "shifts": torch.zeros(int(live.sum()), 3, dtype=torch.float64),
+    }
+    return cluster, keep, cdist
