@@ -24,18 +24,35 @@ sys.path.insert(0, os.path.join(ROOT, "cuda-mace_amd"))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
-# HBM bytes per launch at the default workload (25 000 atoms, 128 channels) from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE, each scaled by what the same counter reads for a 1 GiB copy (factors 2.000 and 1.000); the counter
-# summary with the commands is kept with the other profile summaries.  Null for any other workload.
-MEASURED_TRAFFIC = {
-    "mp_forward_kernel<128>": 3563800000,
-    "mp_backward_edge_kernel<128,true,true,false>": 6331300000,
-    # the two fused kernels as they run inside the model step (atoms relabelled by spatial bin); with the box's random atom
-    # order, as the isolated-ops program launches them, they move 776.8 MB and 818.3 MB
-    "mp_spline_forward_kernel<128,true>": 377000000,
-    "mp_spline_backward_edge_kernel<128,true,true,true,false>": 384500000,
-    "linear_ring_kernel<4,false>": 411200000,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_25k_atoms_128ch.json")
+KERNEL_SOURCES = os.path.join(ROOT, "cuda-mace_amd", "csrc")
+
+
+def kernel_sources_digest():
+    """sha256 over the kernel sources (names and contents, sorted): ties a counter measurement to the code it was made on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(KERNEL_SOURCES)):
+        if name.endswith((".hip", ".hpp")):
+            h.update(name.encode())
+            with open(os.path.join(KERNEL_SOURCES, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic():
+    """HBM bytes per launch at the default workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (calibrated against a
+    copy of known size), as recorded with the profile summaries together with the digest of the kernel sources they were
+    measured on.  Returns {} when the sources have changed since: a stale figure is not reported."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return {}
+    if rec.get("kernel_sources_sha256") != kernel_sources_digest():
+        return {}
+    return {k: int(v) for k, v in rec.get("bytes_per_launch", {}).items()}
 
 
 def linear_kernel_name(C):
@@ -58,17 +75,25 @@ def mp_algorithmic_bytes(N, E, C):
     return fwd, bwd_edge, fwd_fused, bwd_fused
 
 
-def isolated_ops(args, torch, cabi, make_system, reps=3):
-    """A reference copy (reads and writes `copy_bytes` each) followed by the message-passing kernels (tabulated radial
-    weights, and fully fused from the edge vectors) and the channel-mixing linear on random operands at the benchmark
-    shape; prints one line per kernel with its average duration."""
+def _time_ms(torch, fn, reps):
+    """Average duration of `fn` over `reps` back-to-back calls, by events on the stream the kernels are launched on
+    (torch's current stream, which is what the ctypes binding hands to the library)."""
+    fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(reps):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / reps
+
+
+def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=True):
+    """(label, kernels, algorithmic bytes, callable) for every stand-alone op of the path on random operands of the given
+    shape.  Bytes count each operand once.  `rcv` (sorted) and `snd` are int32 device tensors."""
     import numpy as np
 
-    N, C = args.atoms, args.channels
-    data = make_system(N, args.elements, seed=0, density=0.1)
-    rcv = data["edge_index"][0].int().cuda().contiguous()
-    snd = data["edge_index"][1].int().cuda().contiguous()
-    E = rcv.numel()
     g = torch.Generator(device="cuda").manual_seed(0)
     X = torch.randn(N, C, device="cuda", generator=g)
     Y = torch.randn(16, E, device="cuda", generator=g)
@@ -76,39 +101,169 @@ def isolated_ops(args, torch, cabi, make_system, reps=3):
     G = torch.randn(N, 16, C, device="cuda", generator=g)
     vec = torch.randn(E, 3, device="cuda", generator=g)
     vec = vec / vec.norm(dim=1, keepdim=True) * (torch.rand(E, 1, device="cuda", generator=g) * 4.0 + 0.9)
+    r = vec.norm(dim=1).contiguous()
     kn, h = np.linspace(1e-12, 6.0, 256, retstep=True)
     knots = torch.tensor(kn, dtype=torch.float32, device="cuda")
     coeffs = torch.randn(255, 4, 4 * C, device="cuda", generator=g)
     fo = cabi.first_occurences(rcv, N)
-    WT = torch.randn(4, C, C, device="cuda", generator=g)
-    copy_bytes = 1 << 30
-    src = torch.empty(copy_bytes // 4, dtype=torch.float32, device="cuda").normal_(generator=g)
-    dst = torch.empty_like(src)
+    perm, off = cabi.stable_key_sort(snd, N)
     fwd_b, bwd_b, fwd_fb, bwd_fb = mp_algorithmic_bytes(N, E, C)
+    bwd_full_b = 4 * (8 * E * C + 32 * E + 18 * N * C) + 8 * E
     cases = [
-        ("copy (reads %d B, writes %d B)" % (copy_bytes, copy_bytes), 2 * copy_bytes, lambda: dst.copy_(src)),
-        ("mp_forward_kernel<%d>" % C, fwd_b, lambda: cabi.mp_forward(X, Y, R, snd, fo, N)),
-        ("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b,
+        ("mp_forward (tabulated R)", "mp_forward_kernel<%d>" % C, fwd_b, lambda: cabi.mp_forward(X, Y, R, snd, fo, N)),
+        ("mp_backward gY,gR (tabulated R)", "mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b,
          lambda: cabi.mp_backward(X, Y, R, G, snd, fo, None, None, N, need_gX=False)),
-        ("mp_spline_forward_kernel<%d,true>" % C, fwd_fb,
-         lambda: cabi.mp_edge_forward(X, vec, knots, coeffs, float(h), 5.0, snd, fo, N)),
-        ("mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb,
-         lambda: cabi.mp_edge_backward(X, vec, knots, coeffs, float(h), 5.0, G, snd, fo, None, None, N, need_gX=False)),
-        # channel-mixing linear [N,16,C] x [C,C] per l: reads X and the four weight blocks, writes OUT
-        (linear_kernel_name(C), 4 * (32 * N * C + 4 * C * C), lambda: cabi.linear(G, WT)),
+        ("mp_backward gX,gY,gR (tabulated R): edge pass + sender pass",
+         "mp_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,false>" % (C, C), bwd_full_b,
+         lambda: cabi.mp_backward(X, Y, R, G, snd, fo, perm, off, N)),
     ]
+    if with_fused:
+        cases += [
+            ("mp_edge_forward (fused harmonics + spline)", "mp_spline_forward_kernel<%d,true>" % C, fwd_fb,
+             lambda: cabi.mp_edge_forward(X, vec, knots, coeffs, float(h), 5.0, snd, fo, N)),
+            ("mp_edge_backward grad_vectors (fused)", "mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb,
+             lambda: cabi.mp_edge_backward(X, vec, knots, coeffs, float(h), 5.0, G, snd, fo, None, None, N, need_gX=False)),
+        ]
+    if with_node_ops:
+        from cuda_mace.models.upstream_like import _SymmetricContraction
+        from cuda_mace.ops._autograd import monomials_from_packed
+        from cuda_mace.ops.symmetric_contraction import SymmetricContraction
+
+        WT = torch.randn(4, C, C, device="cuda", generator=g)
+        gY = torch.randn(16, E, device="cuda", generator=g)
+        gN = torch.randn(N, C, device="cuda", generator=g)
+        mod = SymmetricContraction(_SymmetricContraction(C, ne, torch.Generator().manual_seed(0)), device="cuda")
+        (m3, o3, p3, v3), (m2, o2, p2, v2) = monomials_from_packed(mod.U3_num_nonsparse, mod.U3_indices, mod.U3_values,
+                                                                   mod.U2_num_nonsparse, mod.U2_indices, mod.U2_values)
+        t = lambda a: torch.from_numpy(a).cuda()
+        T3, T2, T1 = cabi.symcon_tables(t(o3), t(p3), t(v3), t(o2), t(p2), t(v2), mod.weights_3[0], mod.weights_2[0],
+                                        mod.weights_1[0])
+        types = torch.randint(0, ne, (N,), device="cuda", generator=g).int()
+        eperm, eoff = cabi.stable_key_sort(types, ne)
+        m3d, m2d = t(m3), t(m2)
+        cases += [
+            ("spherical harmonics forward", "sh_forward_kernel", 76 * E, lambda: cabi.sh_forward(vec)),
+            ("spherical harmonics backward", "sh_backward_kernel", 88 * E, lambda: cabi.sh_backward(vec, gY)),
+            ("spline forward (R only)", "spline_forward_kernel", 4 * (E + 4 * E * C),
+             lambda: cabi.spline_forward(r, knots, coeffs, float(h), 5.0)),
+            ("spline backward", "spline_backward_kernel", 4 * (4 * E * C + 2 * E),
+             lambda: cabi.spline_backward(r, knots, coeffs, R.view(E, 4 * C), float(h), 5.0)),
+            ("symmetric contraction forward + gradient", "symcon_lmax3_kernel", 4 * (33 * N * C + N),
+             lambda: cabi.symcon_forward(G, eperm, eoff, m3d, m2d, T3, T2, T1, builtin=True)),
+            ("symmetric contraction backward", "symcon_backward_kernel", 4 * 33 * N * C, lambda: cabi.symcon_backward(G, gN)),
+            # channel-mixing linear [N,16,C] x [C,C] per l: reads X and the four weight blocks, writes OUT
+            ("linear [N,16,C] x [C,C]", linear_kernel_name(C), 4 * (32 * N * C + 4 * C * C), lambda: cabi.linear(G, WT)),
+        ]
+    return cases
+
+
+def box_edges(torch, make_system, N, ne):
+    data = make_system(N, ne, seed=0, density=0.1)
+    return data["edge_index"][0].int().cuda().contiguous(), data["edge_index"][1].int().cuda().contiguous()
+
+
+def config2_edges(torch, N=4096, degree=30):
+    """Benchmark configuration 2: every node receives `degree` edges, senders uniform random (torch.manual_seed(0))."""
+    g = torch.Generator().manual_seed(0)
+    rcv = torch.arange(N, dtype=torch.int32).repeat_interleave(degree)
+    snd = torch.randint(0, N, (N * degree,), generator=g, dtype=torch.int32)
+    return rcv.cuda(), snd.cuda()
+
+
+def isolated_ops(args, torch, cabi, make_system, reps=3):
+    """A reference copy (reads and writes `copy_bytes` each) followed by every stand-alone op of the path on random
+    operands at the benchmark shape, and the message-passing op at the shape of configuration 2; prints one line per op
+    with its average duration (for rocprofv3 --kernel-trace / --pmc runs)."""
+    N, C = args.atoms, args.channels
+    rcv, snd = box_edges(torch, make_system, N, args.elements)
+    E = rcv.numel()
+    copy_bytes = 1 << 30
+    src = torch.empty(copy_bytes // 4, dtype=torch.float32, device="cuda").normal_()
+    dst = torch.empty_like(src)
+    cases = [("copy (reads %d B, writes %d B)" % (copy_bytes, copy_bytes), "copy", 2 * copy_bytes, lambda: dst.copy_(src))]
+    cases += op_cases(torch, cabi, N, E, C, args.elements, rcv, snd)
     print("# isolated ops at N=%d E=%d C=%d" % (N, E, C), flush=True)
-    for name, nbytes, fn in cases:
-        fn()
-        torch.cuda.synchronize()
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        for _ in range(reps):
-            fn()
-        e.record()
-        torch.cuda.synchronize()
-        ms = s.elapsed_time(e) / reps
-        print("%-60s %9.1f us  algorithmic %12d B  %8.1f GB/s" % (name, ms * 1e3, nbytes, nbytes / ms / 1e6), flush=True)
+    for label, kernel, nbytes, fn in cases:
+        ms = _time_ms(torch, fn, reps)
+        print("%-62s %-70s %9.1f us  algorithmic %12d B  %8.1f GB/s" % (label, kernel, ms * 1e3, nbytes, nbytes / ms / 1e6), flush=True)
+    rcv2, snd2 = config2_edges(torch)
+    print("# configuration 2: N=4096 E=%d C=96" % rcv2.numel(), flush=True)
+    for label, kernel, nbytes, fn in op_cases(torch, cabi, 4096, rcv2.numel(), 96, args.elements, rcv2, snd2, with_fused=False,
+                                              with_node_ops=False):
+        ms = _time_ms(torch, fn, 10 * reps)
+        print("%-62s %-70s %9.1f us  algorithmic %12d B  %8.1f GB/s" % (label, kernel, ms * 1e3, nbytes, nbytes / ms / 1e6), flush=True)
+
+
+def standalone_rooflines(torch, cabi, N, E, C, ne, rcv, snd, reps=10):
+    """Roofline entries (HBM) of every stand-alone op at the benchmark shape and of the message-passing op at the shape of
+    configuration 2, each timed on its own outside the timed steps."""
+    def rows(cases, reps, **extra):
+        out = []
+        for label, kernel, nbytes, fn in cases:
+            ms = _time_ms(torch, fn, reps)
+            gbps = nbytes / (ms * 1e-3) / 1e9
+            out.append(dict(op=label, kernel=kernel, bound="hbm", achieved=round(gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
+                            frac=round(gbps / HBM_PEAK_GBPS, 4), algorithmic_bytes_per_launch=nbytes,
+                            avg_launch_ms=round(ms, 4), **extra))
+        return out
+
+    at_c4 = rows(op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=False), reps, shape="N=%d E=%d C=%d" % (N, E, C))
+    rcv2, snd2 = config2_edges(torch)
+    at_c2 = rows(op_cases(torch, cabi, 4096, rcv2.numel(), 96, ne, rcv2, snd2, with_fused=False, with_node_ops=False), 5 * reps,
+                 shape="configuration 2: N=4096 E=%d C=96, uniform random senders" % rcv2.numel())
+    fwd, full = at_c2[0], at_c2[2]
+    c2 = {"workload": "isolated invariant message passing forward + full backward (gX, gY, gR), 4096 nodes x 30 edges, 96 "
+                      "channels, R[E,4,C] as the reference's op takes it",
+          "fwd_ms": fwd["avg_launch_ms"], "bwd_ms": full["avg_launch_ms"],
+          "fwd_plus_bwd_ms": round(fwd["avg_launch_ms"] + full["avg_launch_ms"], 4),
+          "algorithmic_bytes": fwd["algorithmic_bytes_per_launch"] + full["algorithmic_bytes_per_launch"],
+          "GB/s": round((fwd["algorithmic_bytes_per_launch"] + full["algorithmic_bytes_per_launch"])
+                        / ((fwd["avg_launch_ms"] + full["avg_launch_ms"]) * 1e-3) / 1e9, 1)}
+    c2["frac_of_hbm_peak"] = round(c2["GB/s"] / HBM_PEAK_GBPS, 4)
+    return at_c4 + at_c2, c2
+
+
+def other_configs(torch, make_system, to_device, OptimizedInvariantMACE, SyntheticInvariantMACE):
+    """Energy+forces steps of the other benchmark configurations (1: 21-atom cluster, eager and as one HIP graph;
+    3: 5 000 atoms, 96 channels; 5: 100 000 atoms, 192 channels), each timed like the headline."""
+    from cuda_mace.utils.graph import GraphedStep
+
+    def run(label, data_cpu, C, numbers, warmup, steps, graph=False):
+        N, E = int(data_cpu["positions"].shape[0]), int(data_cpu["edge_index"].shape[1])
+        up = SyntheticInvariantMACE(channels=C, atomic_numbers=numbers, avg_num_neighbors=E / N, seed=0)
+        model = OptimizedInvariantMACE(up, device="cuda")
+        data = to_device(data_cpu, "cuda")
+
+        def timed(fn):
+            for _ in range(warmup):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+            return 1e3 * (time.perf_counter() - t0) / steps
+
+        ms = timed(lambda: model(dict(data)))
+        out = {"workload": label, "atoms": N, "edges": E, "channels": C, "ms_per_step": round(ms, 4),
+               "atoms_steps_per_s": round(N / ms * 1e3, 1), "steps": steps}
+        if graph:
+            step = GraphedStep(model, data)
+            ms_g = timed(lambda: step(data["positions"]))
+            out.update(ms_per_step_hip_graph=round(ms_g, 4), atoms_steps_per_s_hip_graph=round(N / ms_g * 1e3, 1))
+        del model, data
+        torch.cuda.empty_cache()
+        return out
+
+    res = {}
+    res["c1"] = run("21-atom cluster in an 8 A cube, {H,C,N,O}, 64x0e (fp32 kernels; the fp64 CPU reference is the parity "
+                    "oracle of this configuration)", make_system(21, 4, seed=0, density=None, cluster_box=8.0), 64,
+                    (1, 6, 7, 8), 20, 200, graph=True)
+    res["c3"] = run("5 000-atom periodic box, 96x0e, 10 elements", make_system(5000, 10, seed=0, density=0.1), 96,
+                    tuple(range(1, 11)), 10, 50)
+    res["c5"] = run("100 000-atom periodic box, 192x0e, 10 elements", make_system(100000, 10, seed=0, density=0.1), 192,
+                    tuple(range(1, 11)), 3, 10)
+    return res
 
 
 def main():
@@ -126,6 +281,9 @@ def main():
     ap.add_argument("--tabulated-radial", action="store_true",
                     help="keep the reference's separate spline step (R[E,4,C] in HBM) instead of the fused kernels")
     ap.add_argument("--cpu-atoms", type=int, default=1500, help="size of the box the CPU baseline is timed on")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip what is measured besides the timed steps: stand-alone op rooflines, the other configurations, "
+                         "neighbour list, MD loop (keeps a profiler's trace of this run to the timed steps)")
     ap.add_argument("--isolated-ops", action="store_true",
                     help="instead of the model step, launch a plain copy of known size and each message-passing kernel a few "
                          "times at the benchmark shape (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
@@ -222,12 +380,13 @@ def main():
         return sum(ts) / len(ts) if ts else None
 
     default_workload = (N, C, ne) == (25000, 128, 10)
+    traffic = measured_traffic()
 
     def entry(kernel, nbytes, ms, **extra):
         gbps = nbytes / (ms * 1e-3) / 1e9
         d = {"kernel": kernel, "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
              "frac": round(gbps / HBM_PEAK_GBPS, 4),
-             "traffic": MEASURED_TRAFFIC.get(kernel) if default_workload else None,
+             "traffic": traffic.get(kernel) if default_workload else None,
              "algorithmic_bytes_per_launch": nbytes, "avg_launch_ms": round(ms, 4)}
         d.update(extra)
         return d
@@ -265,7 +424,7 @@ def main():
             tf = flops / (t_lin * 1e-3) / 1e12
             others.append({"kernel": linear_kernel_name(C), "bound": "mfma", "achieved": round(tf, 1),
                            "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
-                           "traffic": MEASURED_TRAFFIC.get(linear_kernel_name(C)) if default_workload else None,
+                           "traffic": traffic.get(linear_kernel_name(C)) if default_workload else None,
                            "algorithmic_flops_per_launch": flops, "avg_launch_ms": round(t_lin, 4),
                            "launches_timed": len(events["linear"]),
                            "note": "fp32-equivalent flops of the [N,16,C] x [C,C] channel mixing against the fp32 matrix "

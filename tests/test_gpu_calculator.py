@@ -1,6 +1,10 @@
-"""DeviceCalculator: Verlet list on the GPU + graph replays reproduce the model on an exact, freshly built list."""
+"""DeviceCalculator / MACECalculator: Verlet list on the GPU + graph replays against the fp64 reference model evaluated
+on a host-built exact list (energy within 1e-5 relative, forces within 1e-4 eV/A, stress against a strain finite
+difference of the reference energy), and against the model itself on a freshly built device list."""
 import pytest
 import torch
+
+from tests.util import reference_on_fresh_list
 
 pytestmark = pytest.mark.gpu
 
@@ -15,8 +19,10 @@ def test_md_like_walk(cabi, use_graph):
     n = 400
     data = to_device(make_system(n, 10, seed=11, density=0.1), "cuda")
     avg = data["edge_index"].shape[1] / n
-    model = OptimizedInvariantMACE(SyntheticInvariantMACE(channels=64, atomic_numbers=tuple(range(1, 11)),
-                                                          avg_num_neighbors=avg, seed=12), device="cuda",
+    upstream = SyntheticInvariantMACE(channels=64, atomic_numbers=tuple(range(1, 11)), avg_num_neighbors=avg, seed=12)
+    params = upstream.export_params()
+    box = float(data["cell"][0, 0])
+    model = OptimizedInvariantMACE(upstream, device="cuda",
                                    spatial_order_min_atoms=0 if use_graph else None)  # one of the two with relabelling
     calc = DeviceCalculator(model, data["node_attrs"], cutoff=5.0, skin=0.4, pbc=(True, True, True), cell=data["cell"],
                             use_graph=use_graph)
@@ -29,6 +35,11 @@ def test_md_like_walk(cabi, use_graph):
         scale = float(exact["forces"].abs().max())
         torch.testing.assert_close(got["energy"], exact["energy"].detach(), rtol=1e-7, atol=1e-7)
         torch.testing.assert_close(got["forces"], exact["forces"].detach(), rtol=0, atol=2e-6 * scale)
+        if it % 6 == 0 or it == 24:  # the fp64 reference on a host-built exact list for the same positions
+            ref = reference_on_fresh_list(params, pos.cpu().numpy(), data["node_attrs"], box)
+            e, e_ref = float(got["energy"].double().sum()), float(ref["energy"])
+            assert abs(e - e_ref) <= 1e-5 * abs(e_ref), (it, e, e_ref)
+            assert float((got["forces"].double().cpu() - ref["forces"]).abs().max()) <= 1e-4
     assert 1 < calc.builds < 25 and calc.steps == 25
 
 
@@ -53,7 +64,8 @@ class _Atoms:
 
 
 def test_ase_protocol_calculator(cabi):
-    """Energy, forces and Voigt stress through the ASE calculator protocol equal the model on a freshly built list."""
+    """Energy and forces through the ASE calculator protocol against the fp64 reference model, the Voigt stress against
+    a central strain difference of the reference energy; all three also against the model on a freshly built list."""
     import numpy as np
 
     from cuda_mace.calculators import MACECalculator
@@ -65,8 +77,10 @@ def test_ase_protocol_calculator(cabi):
     zs = (1, 6, 7, 8)
     data = to_device(make_system(n, len(zs), seed=21, density=0.1), "cuda")
     avg = data["edge_index"].shape[1] / n
-    model = OptimizedInvariantMACE(SyntheticInvariantMACE(channels=32, atomic_numbers=zs, avg_num_neighbors=avg, seed=22),
-                                   device="cuda")
+    upstream = SyntheticInvariantMACE(channels=32, atomic_numbers=zs, avg_num_neighbors=avg, seed=22)
+    params = upstream.export_params()
+    box = float(data["cell"][0, 0])
+    model = OptimizedInvariantMACE(upstream, device="cuda")
     numbers = np.asarray(zs)[data["node_attrs"].argmax(1).cpu().numpy()]
     atoms = _Atoms(data["positions"].cpu().numpy(), numbers, data["cell"].reshape(3, 3).cpu().numpy(), (True, True, True))
     calc = MACECalculator(model)
@@ -88,11 +102,32 @@ def test_ase_protocol_calculator(cabi):
     voigt = np.array([full[0, 0], full[1, 1], full[2, 2], full[1, 2], full[0, 2], full[0, 1]])
     np.testing.assert_allclose(s, voigt, rtol=0, atol=2e-6 * float(np.abs(voigt).max()))
 
+    # the fp64 reference: energy, forces, and stress = (1/V) dE/d(strain) by central differences
+    oracle = reference_on_fresh_list(params, atoms.positions, data["node_attrs"], box)
+    assert abs(e - float(oracle["energy"])) <= 1e-5 * abs(float(oracle["energy"]))
+    assert float(np.abs(f - oracle["forces"].numpy()).max()) <= 1e-4
+    h, vol = 1e-5, box ** 3
+    for comp, (a, b) in enumerate([(0, 0), (1, 1), (2, 2), (1, 2), (0, 2), (0, 1)]):
+        if comp in (1, 2, 4):
+            continue  # three of the six components pin the convention (diagonal, two off-diagonal orders)
+        es = []
+        for sign in (+1, -1):
+            eps = np.zeros((3, 3))
+            eps[a, b] += sign * h / 2
+            eps[b, a] += sign * h / 2
+            es.append(float(reference_on_fresh_list(params, atoms.positions, data["node_attrs"], box, strain=eps,
+                                                    compute_forces=False)["interaction_energy"]))
+        fd = (es[0] - es[1]) / (2 * h) / vol
+        assert abs(fd - s[comp]) <= 2e-3 * float(np.abs(s).max()), (comp, fd, s[comp])
+
     # moved atoms: results are recomputed; an unknown species is refused
     atoms.positions = atoms.positions + 0.02 * np.random.default_rng(0).normal(size=atoms.positions.shape)
     assert calc.calculation_required(atoms, ["forces"])
     ref2 = exact(atoms.positions)
     np.testing.assert_allclose(calc.get_forces(atoms), ref2["forces"].detach().cpu().numpy(), rtol=0, atol=2e-6 * scale)
+    oracle2 = reference_on_fresh_list(params, atoms.positions, data["node_attrs"], box)
+    assert float(np.abs(calc.get_forces(atoms) - oracle2["forces"].numpy()).max()) <= 1e-4
+    assert abs(calc.get_potential_energy(atoms) - float(oracle2["energy"])) <= 1e-5 * abs(float(oracle2["energy"]))
     assert abs(calc.get_potential_energy(atoms) - float(ref2["energy"].sum())) <= 1e-7 * max(1.0, abs(e))
     atoms.numbers = atoms.numbers.copy()
     atoms.numbers[0] = 79

@@ -161,3 +161,28 @@ def test_model_surgery_tool(cabi, tmp_path, capsys):
     out = back(batch)
     assert bool(torch.isfinite(out["energy"]).all()) and out["forces"].shape == (64, 3)
     assert float(out["forces"].sum(0).abs().max()) < 1e-4 * max(1.0, float(out["forces"].abs().max()))
+
+
+def test_model_surgery_tool_against_a_callable_source_model(cabi, tmp_path, capsys):
+    """The tool's own accuracy check (the reference's tools/model_surgery.py:66-143 compares the optimised model with
+    the original one in fp64) on a saved source model that can be evaluated: here its forward is the fp64 reference
+    model.  The errors the tool prints must meet the parity bar; the diamond cell of size 2 is narrower than two
+    cutoffs, so pairs interact through several periodic images."""
+    import re
+
+    from tests.util import oracle_backed_model
+
+    from cuda_mace.tools import model_surgery
+
+    src = tmp_path / "source.model"
+    torch.save(oracle_backed_model(channels=32, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=60.0, seed=3), src)
+    out_path = tmp_path / "optimized.model"
+    model_surgery.main(["--model", str(src), "--size", "2", "--accuracy", "--output", str(out_path)])
+    printed = capsys.readouterr().out
+    errs = {m.group(1): (float(m.group(2)), float(m.group(3)))
+            for m in re.finditer(r"absolute (\w+) error \(mean, max\)---\n(\S+) (\S+)", printed)}
+    energy = float(re.search(r"energy org tensor\(\[([-0-9.e]+)", printed).group(1))
+    assert set(errs) == {"energy", "forces"}, printed
+    assert errs["energy"][1] <= 1e-5 * abs(energy), printed
+    assert errs["forces"][1] <= 1e-4, printed
+    assert torch.load(out_path, weights_only=False).orig_model is not None

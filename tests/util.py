@@ -67,3 +67,46 @@ def carve_cluster(data, centre, r_atoms, r_receivers, cutoff=5.0):
         "shifts": torch.zeros(int(live.sum()), 3, dtype=torch.float64),
     }
     return cluster, keep, cdist
+
+
+def reference_on_fresh_list(params, positions, node_attrs, box, cutoff=5.0, strain=None, compute_forces=True):
+    """The fp64 reference model on a neighbour list built on the host (scipy) for these positions in a cubic periodic
+    box; `strain` (3x3, symmetric) deforms positions and cell together, for finite-difference virials."""
+    from cuda_mace.utils.synthetic import neighbour_list
+    from oracle import mace_model as M
+
+    pos = np.asarray(positions, dtype=np.float64)
+    ei, S = neighbour_list(pos, cutoff, box)
+    cell = np.eye(3) * box
+    if strain is not None:
+        pos = pos + pos @ strain
+        cell = cell + cell @ strain
+    data = {"positions": torch.from_numpy(pos), "node_attrs": node_attrs.detach().cpu().double(),
+            "edge_index": torch.from_numpy(ei), "shifts": torch.from_numpy(S @ cell)}
+    return M.energy_and_forces(params, data, compute_forces=compute_forces)
+
+
+def oracle_backed_model(**kwargs):
+    """A source model for the conversion tool that can also be called, like an upstream model: the random-init weight
+    container of the package with a forward that evaluates the fp64 reference (oracle) on the host."""
+    from cuda_mace.models import SyntheticInvariantMACE
+
+    return OracleBackedMACE(**kwargs)
+
+
+def _oracle_forward(self, data, training=False, compute_force=True, **unused):
+    from oracle import mace_model as M
+
+    cpu = {k: v.detach().cpu() for k, v in data.items()}
+    out = M.energy_and_forces(self.export_params(), cpu, compute_forces=compute_force)
+    dev = data["positions"].device
+    return {k: (v.to(dev) if v is not None else None) for k, v in out.items()}
+
+
+try:
+    from cuda_mace.models import SyntheticInvariantMACE as _Synthetic
+
+    class OracleBackedMACE(_Synthetic):
+        forward = _oracle_forward
+except ImportError:  # the package needs its built library; tests that use this class fail loudly on their own
+    OracleBackedMACE = None
