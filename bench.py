@@ -437,37 +437,16 @@ def main():
                          launches_timed=len(events[bwd_name]))
         others = [entry("mp_forward_kernel<%d>" % C, fwd_b, t_fwd)]
 
-    # the message-passing op with the reference's signature (tabulated R[E,4,C]) at the same shape, timed on its own
-    def isolated_mp():
-        g = torch.Generator(device="cuda").manual_seed(0)
-        X = torch.randn(N, C, device="cuda", generator=g)
-        Yt = torch.randn(16, E, device="cuda", generator=g)
-        R = torch.randn(E, 4, C, device="cuda", generator=g)
-        G = torch.randn(N, 16, C, device="cuda", generator=g)
-        rcv = data["edge_index"][0].int().contiguous()
-        snd = data["edge_index"][1].int().contiguous()
-        fo = cabi.first_occurences(rcv, N)
-
-        def time_it(fn, reps=10):
-            fn()
-            torch.cuda.synchronize()
-            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s.record()
-            for _ in range(reps):
-                fn()
-            e.record()
-            torch.cuda.synchronize()
-            return s.elapsed_time(e) / reps
-
-        tf = time_it(lambda: cabi.mp_forward(X, Yt, R, snd, fo, N))
-        tb = time_it(lambda: cabi.mp_backward(X, Yt, R, G, snd, fo, None, None, N, need_gX=False))
-        return tf, tb
-
-    if fused:
-        tf, tb = isolated_mp()
-        others.append(entry("mp_forward_kernel<%d>" % C, fwd_b, tf, context="isolated op with tabulated R[E,4,C]"))
-        others.append(entry("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b, tb,
-                            context="isolated op with tabulated R[E,4,C]"))
+    # every stand-alone op of the path (the reference's op list: message passing with tabulated R[E,4,C] incl. the full
+    # backward, harmonics, spline, contraction, linear) at the same shape, and configuration 2, each timed on its own
+    standalone, config2 = None, None
+    if not args.no_extras:
+        rcv32 = data["edge_index"][0].int().contiguous()
+        snd32 = data["edge_index"][1].int().contiguous()
+        standalone, config2 = standalone_rooflines(torch, cabi, N, E, C, ne, rcv32, snd32)
+        for row in standalone:
+            row["traffic"] = traffic.get(row["kernel"]) if default_workload and row["shape"].startswith("N=") else None
+        others += standalone
 
     # the step before the path: neighbour list rebuilt on the device (excluded from the timed steps, as the reference's
     # own timing excludes it); checked against the host-built list of the generator
@@ -476,14 +455,16 @@ def main():
     def build_list():
         return get_neighborhood(data["positions"].detach(), 5.0, (True, True, True), data["cell"])
 
-    ei_dev = build_list()[0]
-    torch.cuda.synchronize()
-    t_nl = time.perf_counter()
-    for _ in range(5):
-        build_list()
-    torch.cuda.synchronize()
-    neighbour_list = {"ms_per_build": round(1e3 * (time.perf_counter() - t_nl) / 5, 3), "pairs": int(ei_dev.shape[1]),
-                      "identical_to_host_list": bool(torch.equal(ei_dev, data["edge_index"]))}
+    neighbour_list = None
+    if not args.no_extras:
+        ei_dev = build_list()[0]
+        torch.cuda.synchronize()
+        t_nl = time.perf_counter()
+        for _ in range(5):
+            build_list()
+        torch.cuda.synchronize()
+        neighbour_list = {"ms_per_build": round(1e3 * (time.perf_counter() - t_nl) / 5, 3), "pairs": int(ei_dev.shape[1]),
+                          "identical_to_host_list": bool(torch.equal(ei_dev, data["edge_index"]))}
 
     # an MD-like loop through the device-side calculator: every atom moves 0.02 A per step in a random direction, the
     # Verlet list (cutoff + 0.5 A skin) is rebuilt on the device whenever an atom has moved more than half the skin
@@ -492,7 +473,7 @@ def main():
     calc = DeviceCalculator(model, data["node_attrs"], cutoff=5.0, skin=0.5, pbc=(True, True, True), cell=data["cell"])
     gen = torch.Generator(device="cuda").manual_seed(0)
     pos = data["positions"].detach().clone()
-    md_steps = 0 if args.no_md_loop else 60
+    md_steps = 0 if (args.no_md_loop or args.no_extras) else 60
 
     def md_step(p):
         d = torch.randn(p.shape, device="cuda", dtype=p.dtype, generator=gen)
@@ -514,6 +495,12 @@ def main():
                "hip_graph": calc.use_graph,
                "note": "energy+forces through DeviceCalculator incl. neighbour-list rebuilds on the device; the list holds "
                        "(1 + skin/cutoff)^3 = 1.33x the pairs of the exact list"}
+
+    configs = None
+    if not args.no_extras:
+        del calc
+        configs = other_configs(torch, make_system, to_device, OptimizedInvariantMACE, SyntheticInvariantMACE)
+        configs["c2"] = config2
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
@@ -545,7 +532,7 @@ def main():
                                "l_max 3, correlation 3, %d elements, random-init weights (seed 0)" % (N, E, C, ne),
                    "atoms": N, "edges": E, "channels": C, "radial": "fused spline" if fused else "tabulated"},
         "roofline": roofline, "roofline_other_kernels": others, "cpu_baseline": cpu_baseline,
-        "neighbour_list": neighbour_list, "md_loop": md_loop,
+        "neighbour_list": neighbour_list, "md_loop": md_loop, "other_configs": configs,
     }
     if cpu_baseline:
         line["speedup_vs_cpu_baseline"] = round(value / cpu_baseline["value"], 1)

@@ -42,6 +42,15 @@ inline int check_launch(const char *what) {
 // l(m) = floor(sqrt(m)) for m in 0..15 without a sqrt.
 __device__ __forceinline__ constexpr int l_of_m(int m) { return m == 0 ? 0 : (m < 4 ? 1 : (m < 9 ? 2 : 3)); }
 
+// Edge range [e0, e1) of a node as read from caller-provided CSR offsets, forced into [0, nedges] with e0 <= e1: offsets
+// derived from an unsorted or out-of-range receiver list then name a wrong but addressable range instead of memory
+// outside the edge arrays.
+__host__ __device__ __forceinline__ void clamp_edge_range(int &e0, int &e1, int64_t nedges) {
+  const int ne = static_cast<int>(nedges);
+  e0 = e0 < 0 ? 0 : (e0 > ne ? ne : e0);
+  e1 = e1 < e0 ? e0 : (e1 > ne ? ne : e1);
+}
+
 // Orders LDS traffic of one wavefront: stores issued before are visible to loads issued after.
 __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -96,7 +96,9 @@ __global__ __launch_bounds__(256) void edge_geometry_backward_kernel(
     acc[2] += g[2];
   }
   // edges that start at this atom (row a, contiguous): - gradient
-  for (int e = a_first_occ[node] + lane; e < a_first_occ[nnodes + node]; e += kWave) {
+  int ea0 = a_first_occ[node], ea1 = a_first_occ[nnodes + node];
+  clamp_edge_range(ea0, ea1, nedges);
+  for (int e = ea0 + lane; e < ea1; e += kWave) {
     edge_grad<HAS_GLEN>(pos, shifts, a, b, rows, gvec, glen, e, nnodes, g);
     acc[0] -= g[0];
     acc[1] -= g[1];

@@ -256,7 +256,7 @@ constexpr int kStages = 3;
 constexpr int kStageBytes = kTileNodes * kKC * 4;
 
 __device__ __forceinline__ void dma16(const float *src, unsigned lds_byte_address) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(src), "s"(lds_byte_address) : "memory");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(src), "s"(lds_byte_address) : "memory", "m0");
 }
 __device__ __forceinline__ void ldg16(f4 &dst, const float *src) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src) : "memory");
@@ -514,15 +514,24 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
   // The ring variant wherever it runs two workgroups per compute unit or the plain one does not either (Nout up to 128,
   // and 224 / 256), and K has more than one chunk to overlap; measured at 25 000 nodes: 108 vs 119-127 us at 128
   // columns, 76 vs 80-83 at 96, equal at 64, 224 and 256, slower at 32 (one chunk), 160 and 192 (one workgroup per CU).
+  // The row_scale variant at 256 columns does not fit the register file and would spill, which the hand-issued loads
+  // of the ring kernel do not tolerate (the build checks that no instantiated ring kernel uses scratch memory): it
+  // runs on the plain kernel.
   constexpr bool kRing = NT == 2 || NT == 3 || NT == 4 || NT >= 7;
-  if (kRing && K > kKC) {
-    if (row_scale)
-      hipLaunchKernelGGL((linear_ring_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
-                         zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
-    else
+  constexpr bool kRingScaled = kRing && NT < 8;
+  if constexpr (kRing) {
+    if (K > kKC && (!row_scale || kRingScaled)) {
+      if constexpr (kRingScaled) {
+        if (row_scale) {
+          hipLaunchKernelGGL((linear_ring_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes),
+                             ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
+          return check_launch("cm_linear");
+        }
+      }
       hipLaunchKernelGGL((linear_ring_kernel<NT, false>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
                          zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
-    return check_launch("cm_linear");
+      return check_launch("cm_linear");
+    }
   }
   if (row_scale)
     hipLaunchKernelGGL((linear_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,

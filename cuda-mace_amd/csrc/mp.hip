@@ -51,6 +51,23 @@ __global__ void first_occurences_kernel(const int32_t *__restrict__ receiver, in
   }
 }
 
+__global__ void fill_zero_i32_kernel(int32_t *p, int64_t n) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    p[i] = 0;
+}
+
+// status[0] = 1 if receiver[e - 1] > receiver[e] anywhere, status[1] = 1 if a value lies outside [0, nnodes); both
+// are cleared by the fill launched before this kernel.  Offending threads store the same value: no atomics needed.
+__global__ void receiver_list_status_kernel(const int32_t *__restrict__ receiver, int64_t nedges, int nnodes,
+                                            int32_t *__restrict__ status) {
+  const int64_t e = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (e >= nedges) return;
+  const int cur = receiver[e];
+  if (e > 0 && receiver[e - 1] > cur) status[0] = 1;
+  if (cur < 0 || cur >= nnodes) status[1] = 1;
+}
+
 // -----------------------------------------------------------------------------------------------
 // forward
 // -----------------------------------------------------------------------------------------------
@@ -69,8 +86,9 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
   const int cl = lane % K::SW;
   const bool active = cl < K::LPE;
   const int node = blockIdx.x;
-  const int e0 = first_occ[node];
-  const int e1 = first_occ[nnodes + node];
+  int e0 = first_occ[node];
+  int e1 = first_occ[nnodes + node];
+  clamp_edge_range(e0, e1, nedges);
 
   vec acc[16];
 #pragma unroll
@@ -150,8 +168,9 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
   const int slot = lane / K::SW;
   const int cl = lane % K::SW;
   const bool active = cl < K::LPE;
-  const int e0 = first_occ[node];
-  const int e1 = first_occ[nnodes + node];
+  int e0 = first_occ[node];
+  int e1 = first_occ[nnodes + node];
+  clamp_edge_range(e0, e1, nedges);
   if (e0 >= e1) return;
 
   vec g[16];
@@ -488,9 +507,25 @@ extern "C" int cm_first_occurences(const int32_t *receiver, int64_t nedges, int6
   const int block = 256;
   const int64_t work = nedges > 0 ? nedges : nnodes;
   const unsigned grid = static_cast<unsigned>(nedges > 0 ? cm::ceil_div(work, block) : std::min<int64_t>(cm::ceil_div(work, block), 1024));
+  // a list that is not sorted leaves entries unwritten: they then read 0, an empty range, instead of what the buffer held
+  hipLaunchKernelGGL(cm::fill_zero_i32_kernel, dim3(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(2 * nnodes, block), 1024))),
+                     dim3(block), 0, cm::as_stream(stream), first_occ, 2 * nnodes);
   hipLaunchKernelGGL(cm::first_occurences_kernel, dim3(grid), dim3(block), 0, cm::as_stream(stream), receiver,
                      static_cast<int>(nedges), static_cast<int>(nnodes), first_occ);
   return cm::check_launch("cm_first_occurences");
+}
+
+extern "C" int cm_receiver_list_status(const int32_t *receiver, int64_t nedges, int64_t nnodes, int32_t *status,
+                                       cm_stream_t stream) {
+  CM_REQUIRE(nedges >= 0 && nnodes >= 0, "cm_receiver_list_status: negative size");
+  CM_REQUIRE(nedges < INT32_MAX && nnodes < INT32_MAX / 2, "cm_receiver_list_status: sizes exceed int32 indexing");
+  CM_REQUIRE(status != nullptr, "cm_receiver_list_status: status is NULL");
+  CM_REQUIRE(nedges == 0 || receiver != nullptr, "cm_receiver_list_status: receiver is NULL");
+  hipLaunchKernelGGL(cm::fill_zero_i32_kernel, dim3(1), dim3(64), 0, cm::as_stream(stream), status, 2);
+  if (nedges > 0)
+    hipLaunchKernelGGL(cm::receiver_list_status_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nedges, 256))), dim3(256), 0,
+                       cm::as_stream(stream), receiver, nedges, static_cast<int>(nnodes), status);
+  return cm::check_launch("cm_receiver_list_status");
 }
 
 extern "C" int cm_mp_forward(const float *X, const float *Y, const float *R, const int32_t *sender,

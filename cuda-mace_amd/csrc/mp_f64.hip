@@ -41,8 +41,9 @@ __global__ __launch_bounds__(kWave) void mp_forward_f64_kernel(const double *__r
                                                               int64_t nedges, int C, double *__restrict__ out) {
   const int lane = threadIdx.x;
   const int node = blockIdx.x;
-  const int e0 = first_occ[node];
-  const int e1 = first_occ[nnodes + node];
+  int e0 = first_occ[node];
+  int e1 = first_occ[nnodes + node];
+  clamp_edge_range(e0, e1, nedges);
   double acc[16][KS];
 #pragma unroll
   for (int m = 0; m < 16; ++m)
@@ -84,8 +85,9 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_f64_kernel(
     double *__restrict__ gY, double *__restrict__ gR, double *__restrict__ gXe) {
   const int lane = threadIdx.x;
   const int node = blockIdx.x;
-  const int e0 = first_occ[node];
-  const int e1 = first_occ[nnodes + node];
+  int e0 = first_occ[node];
+  int e1 = first_occ[nnodes + node];
+  clamp_edge_range(e0, e1, nedges);
   if (e0 >= e1) return;
 
   double g[16][KS];

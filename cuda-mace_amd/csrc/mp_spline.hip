@@ -141,8 +141,9 @@ __global__ __launch_bounds__(kWave, (Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVE
   const int slot = lane / K::SW;
   const int cl = lane % K::SW;
   const bool active = cl < K::LPE;
-  const int e0 = first_occ[node];
-  const int e1 = first_occ[nnodes + node];
+  int e0 = first_occ[node];
+  int e1 = first_occ[nnodes + node];
+  clamp_edge_range(e0, e1, nedges);
 
   vec acc[16];
 #pragma unroll
@@ -225,8 +226,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   const int cl = lane % K::SW;
   const bool active = cl < K::LPE;
   const unsigned cla = active ? cl : 0;  // lanes beyond the channel count read lane 0's addresses; their g is zero
-  const int e0 = first_occ[node];
-  const int e1 = first_occ[nnodes + node];
+  int e0 = first_occ[node];
+  int e1 = first_occ[nnodes + node];
+  clamp_edge_range(e0, e1, nedges);
   if (e0 >= e1) return;
 
   vec g[16];

@@ -1,8 +1,10 @@
 // Stable counting sort of item indices by integer key (sender-sorted edge view, nodes grouped by
-// element).  Buckets are filled with integer atomics in arbitrary order and then every item is
-// moved to its rank within the bucket, the rank being the number of bucket members with a smaller
-// item index.  The result is the unique stable order, so it is reproducible bit for bit although
-// atomics are used on the way.
+// element).  Two routes to the same unique stable order, reproducible bit for bit:
+//  - many keys, small buckets (edges by sender): buckets are filled with integer atomics in arbitrary order and then
+//    every item is moved to its rank within the bucket, the rank being the number of bucket members with a smaller
+//    item index (a scan of the bucket: quadratic in the bucket size, which is tens of items here);
+//  - few keys, large buckets (atoms by element): per-workgroup histograms, one scan over (key, workgroup), and a rank
+//    inside the workgroup's 256 items, so the cost per item does not grow with the bucket.
 #include <algorithm>
 #include <mutex>
 
@@ -28,7 +30,7 @@ __global__ void histogram_kernel(const int32_t *__restrict__ keys, int64_t n, in
 }
 
 // One workgroup: offsets = exclusive scan of counts (nkeys + 1 entries), cursor = copy of the first
-// nkeys.  Every thread owns a contiguous run of keys.
+// nkeys (skipped when NULL).  Every thread owns a contiguous run of keys.
 __global__ __launch_bounds__(kScanThreads) void scan_kernel(const int32_t *__restrict__ counts, int nkeys,
                                                             int32_t *__restrict__ offsets,
                                                             int32_t *__restrict__ cursor) {
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(const int32_t *__res
   int run = part[t] - sum;  // exclusive prefix of this thread's run
   for (int k = lo; k < hi; ++k) {
     offsets[k] = run;
-    cursor[k] = run;
+    if (cursor) cursor[k] = run;
     run += counts[k];
   }
   if (t == kScanThreads - 1) offsets[nkeys] = part[t];
@@ -80,13 +82,65 @@ __global__ void bucket_rank_kernel(const int32_t *__restrict__ keys, const int32
   perm[lo + rank] = item;
 }
 
+// ---- few keys, large buckets ----------------------------------------------------------------------------------
+constexpr int kFewKeys = 64;       // route bound: keys per LDS histogram
+constexpr int kFewBlock = 256;     // items per workgroup
+constexpr int64_t kFewMinItems = 4096;
+
+inline bool few_keys_route(int64_t n, int64_t nkeys) { return nkeys >= 1 && nkeys <= kFewKeys && n >= kFewMinItems; }
+
+// block_counts[k * nblocks + b] = items of workgroup b with key k
+__global__ __launch_bounds__(kFewBlock) void block_histogram_kernel(const int32_t *__restrict__ keys, int64_t n, int nkeys,
+                                                                     int nblocks, int32_t *__restrict__ block_counts) {
+  __shared__ int hist[kFewKeys];
+  const int t = threadIdx.x;
+  if (t < kFewKeys) hist[t] = 0;
+  __syncthreads();
+  const int64_t i = blockIdx.x * static_cast<int64_t>(kFewBlock) + t;
+  if (i < n) {
+    const int k = keys[i];
+    if (static_cast<unsigned>(k) < static_cast<unsigned>(nkeys)) atomicAdd(&hist[k], 1);
+  }
+  __syncthreads();
+  if (t < nkeys) block_counts[static_cast<int64_t>(t) * nblocks + blockIdx.x] = hist[t];
+}
+
+// base = exclusive scan of block_counts in (key, workgroup) order: item i of workgroup b with key k goes to
+// base[k * nblocks + b] + (number of earlier items of b with key k).
+__global__ __launch_bounds__(kFewBlock) void block_place_kernel(const int32_t *__restrict__ keys, int64_t n, int nkeys,
+                                                                 int nblocks, const int32_t *__restrict__ base,
+                                                                 int32_t *__restrict__ perm, int32_t *__restrict__ offsets) {
+  __shared__ int skey[kFewBlock];
+  const int t = threadIdx.x;
+  const int64_t i = blockIdx.x * static_cast<int64_t>(kFewBlock) + t;
+  int k = -1;
+  if (i < n) {
+    k = keys[i];
+    if (static_cast<unsigned>(k) >= static_cast<unsigned>(nkeys)) k = -1;
+  }
+  skey[t] = k;
+  __syncthreads();
+  if (k >= 0) {
+    int rank = 0;
+    for (int j = 0; j < t; ++j) rank += skey[j] == k ? 1 : 0;
+    perm[base[static_cast<int64_t>(k) * nblocks + blockIdx.x] + rank] = static_cast<int32_t>(i);
+  }
+  if (blockIdx.x == 0 && t <= nkeys) offsets[t] = base[static_cast<int64_t>(t) * nblocks];
+}
+
 }  // namespace
 }  // namespace cm
 
 extern "C" size_t cm_stable_key_sort_workspace(int64_t n, int64_t nkeys) {
   if (n < 0 || nkeys < 0) return 0;
-  // counts[nkeys] + cursor[nkeys] + bucketed[n], each int32, rounded up to 256 bytes
-  const size_t bytes = static_cast<size_t>(2 * nkeys + n) * sizeof(int32_t);
+  // counts[nkeys] + cursor[nkeys] + bucketed[n], each int32; the few-keys route instead keeps two tables over
+  // (key, workgroup) plus the closing total; rounded up to 256 bytes
+  size_t ints = static_cast<size_t>(2 * nkeys + n);
+  if (cm::few_keys_route(n, nkeys)) {
+    const size_t table = static_cast<size_t>(nkeys) * static_cast<size_t>(cm::ceil_div(n, cm::kFewBlock));
+    ints = std::max(ints, 2 * table + 2);
+  }
+  const size_t bytes = ints * sizeof(int32_t);
   return (bytes + 255) & ~static_cast<size_t>(255);
 }
 
@@ -96,6 +150,19 @@ namespace {
 // Enqueues the five kernels of the sort; `workspace` holds cm_stable_key_sort_workspace(n, nkeys) bytes.
 int sort_enqueue(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm, int32_t *offsets, void *workspace,
                  hipStream_t st, const char *what) {
+  if (few_keys_route(n, nkeys)) {
+    const int nblocks = static_cast<int>(ceil_div(n, kFewBlock));
+    const int entries = static_cast<int>(nkeys) * nblocks;
+    int32_t *block_counts = static_cast<int32_t *>(workspace);
+    int32_t *base = block_counts + entries;  // entries + 1 values
+    hipLaunchKernelGGL(block_histogram_kernel, dim3(nblocks), dim3(kFewBlock), 0, st, keys, n, static_cast<int>(nkeys), nblocks,
+                       block_counts);
+    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kScanThreads), 0, st, block_counts, entries, base,
+                       static_cast<int32_t *>(nullptr));
+    hipLaunchKernelGGL(block_place_kernel, dim3(nblocks), dim3(kFewBlock), 0, st, keys, n, static_cast<int>(nkeys), nblocks, base,
+                       perm, offsets);
+    return check_launch(what);
+  }
   int32_t *counts = static_cast<int32_t *>(workspace);
   int32_t *cursor = counts + nkeys;
   int32_t *bucketed = cursor + nkeys;

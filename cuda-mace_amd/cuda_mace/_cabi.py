@@ -38,6 +38,7 @@ SIGNATURES = {
     "cm_trace_push": (None, [ctypes.c_char_p]),
     "cm_trace_pop": (None, []),
     "cm_first_occurences": (_i32, [_p, _i64, _i64, _p, _p]),
+    "cm_receiver_list_status": (_i32, [_p, _i64, _i64, _p, _p]),
     "cm_stable_key_sort_workspace": (_sz, [_i64, _i64]),
     "cm_stable_key_sort": (_i32, [_p, _i64, _i64, _p, _p, _p, _sz, _p]),
     "cm_stable_key_sort_static_capacity": (_sz, []),
@@ -128,7 +129,25 @@ def _typed(name: str, like: torch.Tensor):
 
 
 # ---- index kernels ---------------------------------------------------------------------------
+DEBUG = os.environ.get("CUDA_MACE_DEBUG", "0") not in ("", "0")
+
+
+def receiver_list_status(receiver: torch.Tensor, nnodes: int):
+    """(decreases somewhere, holds a value outside [0, nnodes)) for a receiver list; synchronises."""
+    status = torch.empty(2, dtype=I32, device=receiver.device)
+    _check(lib.cm_receiver_list_status(_dev(receiver, I32, "receiver_list"), receiver.numel(), nnodes, _dev(status, I32, "status"), _stream()))
+    unsorted, out_of_range = status.tolist()
+    return bool(unsorted), bool(out_of_range)
+
+
 def first_occurences(receiver: torch.Tensor, nnodes: int) -> torch.Tensor:
+    """CSR offsets of a non-decreasing receiver list.  With CUDA_MACE_DEBUG set the list is checked first (one host
+    synchronisation) and a list that is unsorted or out of range raises instead of giving wrong sums."""
+    if DEBUG:
+        unsorted, out_of_range = receiver_list_status(receiver, nnodes)
+        if unsorted or out_of_range:
+            raise CudaMaceError("receiver_list must be non-decreasing with values in [0, %d): %s" % (
+                nnodes, " and ".join(w for w, on in (("it decreases somewhere", unsorted), ("it holds values out of range", out_of_range)) if on)))
     out = torch.empty(2 * nnodes, dtype=I32, device=receiver.device)
     _check(lib.cm_first_occurences(_dev(receiver, I32, "receiver_list"), receiver.numel(), nnodes, _dev(out, I32, "out"), _stream()))
     return out

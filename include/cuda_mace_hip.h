@@ -55,6 +55,14 @@ void cm_trace_pop(void);
  */
 int cm_first_occurences(const int32_t *receiver, int64_t nedges, int64_t nnodes,
                         int32_t *first_occ, cm_stream_t stream);
+/* Checks what cm_first_occurences assumes of its input (the reference does not check it either: an unsorted list
+ * silently gives wrong sums there, jit_wrappers/src/invariant_message_passing_wrapper.cpp:19-70).
+ *   status int32 [2] (device): [0] = 1 if the list decreases somewhere, [1] = 1 if a value lies outside [0, nnodes).
+ * cm_first_occurences itself clamps out-of-range values and gives empty ranges to nodes an unsorted list skips, and
+ * every kernel that reads first_occ forces the ranges into [0, nedges], so a bad list gives wrong sums, never an
+ * access outside the edge arrays.  The Python binding runs this check when CUDA_MACE_DEBUG is set. */
+int cm_receiver_list_status(const int32_t *receiver, int64_t nedges, int64_t nnodes, int32_t *status,
+                            cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Stable counting sort of item indices by key: perm lists items by non-decreasing key, ties in

@@ -76,3 +76,48 @@ def test_profiler_ranges_are_off_unless_asked_for():
     have_markers = any(os.path.exists(os.path.join(d, n)) for d in ("/opt/rocm/lib", "/opt/rocm/lib64")
                        for n in ("librocprofiler-sdk-roctx.so", "libroctx64.so"))
     assert seen["1"] == (1 if have_markers else 0)
+
+
+def test_edge_range_clamp_arithmetic(tmp_path):
+    """cm::clamp_edge_range, which every kernel applies to the CSR offsets it reads, compiled for the host and run on
+    valid, reversed, out-of-range and random offsets (tests/host/clamp_edge_range_check.cpp)."""
+    import shutil
+    import subprocess
+
+    import pytest
+
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    exe = tmp_path / "clamp_check"
+    src = os.path.join(ROOT, "tests", "host", "clamp_edge_range_check.cpp")
+    res = subprocess.run([hipcc, "--cuda-host-only", "-x", "hip", "-O1", "-I" + os.path.join(ROOT, "include"),
+                          "-I" + os.path.join(ROOT, "cuda-mace_amd", "csrc"), src, "-o", str(exe)],
+                         capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0 and run.stdout.strip() == "ok", run.stdout + run.stderr
+
+
+def test_build_refuses_scratch_in_hand_scheduled_kernels():
+    """The build parses the compiler's resource-usage remarks and fails when a kernel whose loads are issued from inline
+    assembly spills registers (its correctness depends on loaded registers staying where the load put them)."""
+    import importlib.util
+
+    import pytest
+
+    spec = importlib.util.spec_from_file_location("_cm_build", os.path.join(ROOT, "cuda-mace_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    line = "csrc/linear.hip:1:1: remark: %s [-Rpass-analysis=kernel-resource-usage]"
+    ok = "\n".join(line % t for t in ("Function Name: _ZN2cm18linear_ring_kernelILi4ELb0EEE", "    VGPRs: 216",
+                                      "    ScratchSize [bytes/lane]: 0", "    SGPRs Spill: 0", "    VGPRs Spill: 0",
+                                      "Function Name: _ZN2cm13linear_kernelILi8ELb1EEE", "    ScratchSize [bytes/lane]: 100"))
+    build._check_no_scratch("linear.hip", ok)  # the plain kernel may spill, the ring kernel does not
+    bad = ok.replace("ScratchSize [bytes/lane]: 0", "ScratchSize [bytes/lane]: 100", 1)
+    with pytest.raises(RuntimeError, match="ScratchSize"):
+        build._check_no_scratch("linear.hip", bad)
+    with pytest.raises(RuntimeError, match="VGPRs Spill"):
+        build._check_no_scratch("linear.hip", ok.replace("VGPRs Spill: 0", "VGPRs Spill: 24"))
+    with pytest.raises(RuntimeError, match="no resource-usage remark"):
+        build._check_no_scratch("mp.hip", ok)

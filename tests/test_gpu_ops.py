@@ -38,7 +38,10 @@ def test_first_occurences_exact(cabi, nnodes, avg, iso, seed):
     assert torch.equal(got, ref)
 
 
-@pytest.mark.parametrize("n,nkeys,seed", [(0, 5, 0), (1, 1, 1), (1000, 10, 2), (122880, 4096, 3), (5000, 1, 4), (3000, 10000, 5)])
+@pytest.mark.parametrize("n,nkeys,seed", [(0, 5, 0), (1, 1, 1), (1000, 10, 2), (122880, 4096, 3), (5000, 1, 4), (3000, 10000, 5),
+                                          # few keys, large buckets (atoms grouped by element): the workgroup-histogram route
+                                          (100000, 1, 6), (100000, 11, 7), (200003, 64, 8), (4096, 3, 9), (4095, 3, 10),
+                                          (70000, 65, 11)])
 def test_stable_key_sort_exact(cabi, n, nkeys, seed):
     _say("stable_key_sort", n, nkeys, seed)
     keys = torch.from_numpy(np.random.default_rng(seed).integers(0, nkeys, n).astype(np.int32))
@@ -46,6 +49,45 @@ def test_stable_key_sort_exact(cabi, n, nkeys, seed):
     perm, off = cabi.stable_key_sort(keys.to(DEV), nkeys)
     assert torch.equal(off.cpu(), off_ref)
     assert torch.equal(perm.cpu(), perm_ref)
+
+
+def test_stable_key_sort_skips_keys_out_of_range(cabi):
+    """Items whose key lies outside [0, nkeys) are left out on both routes (that is where atoms whose one-hot row names
+    no element go): offsets[nkeys] counts the items placed."""
+    for n, nkeys in ((1000, 10), (50000, 10)):
+        rng = np.random.default_rng(n)
+        keys = rng.integers(-2, nkeys + 2, n).astype(np.int32)
+        perm, off = cabi.stable_key_sort(torch.from_numpy(keys).to(DEV), nkeys)
+        valid = np.flatnonzero((keys >= 0) & (keys < nkeys))
+        order = valid[np.argsort(keys[valid], kind="stable")]
+        total = int(off[-1])
+        assert total == valid.size
+        assert np.array_equal(perm.cpu().numpy()[:total], order.astype(np.int32))
+        assert np.array_equal(off.cpu().numpy(), np.searchsorted(keys[order], np.arange(nkeys + 1)).astype(np.int32))
+
+
+def test_receiver_list_status(cabi):
+    """The check of what the CSR kernel assumes of its input: sorted, values in range."""
+    good = torch.tensor([0, 0, 1, 3, 3, 7], dtype=torch.int32, device=DEV)
+    assert cabi.receiver_list_status(good, 8) == (False, False)
+    assert cabi.receiver_list_status(good, 7) == (False, True)
+    bad = torch.tensor([0, 2, 1, 3], dtype=torch.int32, device=DEV)
+    assert cabi.receiver_list_status(bad, 4) == (True, False)
+    assert cabi.receiver_list_status(torch.tensor([5, -1], dtype=torch.int32, device=DEV), 4) == (True, True)
+    assert cabi.receiver_list_status(torch.zeros(0, dtype=torch.int32, device=DEV), 4) == (False, False)
+    big = torch.arange(300000, dtype=torch.int32, device=DEV) // 7
+    assert cabi.receiver_list_status(big, 300000 // 7 + 1) == (False, False)
+    big[123456] = 0
+    assert cabi.receiver_list_status(big, 300000 // 7 + 1) == (True, False)
+    # with the debug switch on, the binding refuses such a list instead of computing offsets from it
+    old = cabi.DEBUG
+    cabi.DEBUG = True
+    try:
+        with pytest.raises(cabi.CudaMaceError, match="non-decreasing"):
+            cabi.first_occurences(bad, 4)
+        assert torch.equal(cabi.first_occurences(good, 8).cpu(), O.first_occurences(good.cpu(), 8))
+    finally:
+        cabi.DEBUG = old
 
 
 # ------------------------------------------------------------------------------------------------

@@ -18,7 +18,7 @@ def test_static_sort_matches_workspace_sort_on_two_calls_in_a_row():
 
     dev = torch.device("cuda:0")
     # outputs pre-allocated up front: the calls under test allocate nothing
-    cases = [(1_301_200, 25_000, 0), (4_097, 300, 1), (100_000, 11, 2), (0, 5, 3), (33, 1, 4)]
+    cases = [(1_301_200, 25_000, 0), (4_097, 300, 1), (100_000, 11, 2), (0, 5, 3), (33, 1, 4), (5_000, 64, 5)]
     keys = [_pair(n, k, s, dev) for n, k, s in cases]
     perms = [torch.full((n,), -7, dtype=torch.int32, device=dev) for n, _, _ in cases]
     offs = [torch.full((k + 1,), -7, dtype=torch.int32, device=dev) for _, k, _ in cases]
