@@ -326,41 +326,38 @@ def main():
         step()
     torch.cuda.synchronize()
 
-    # live timing of the message-passing kernels: events on the launch stream around every forward launch and around
-    # every backward edge pass that runs without the sender pass (first layer: one kernel per call)
+    # Live timing of the dominant kernels inside the timed steps, by events on the launch stream.  The default model hands
+    # the step to the library in one call, which brackets the chosen stages itself (message passing forward of both
+    # layers, the backward edge pass of the first layer, which runs without the sender pass, and the two [N,16,C]
+    # channel-mixing launches); with --tabulated-radial the step goes through the Python wrappers, which are bracketed here.
+    import ctypes
+
     fwd_name, bwd_name = ("mp_edge_forward", "mp_edge_backward") if fused else ("mp_forward", "mp_backward")
-    events = {fwd_name: [], bwd_name: []}
-    originals = {fwd_name: getattr(cabi, fwd_name), bwd_name: getattr(cabi, bwd_name)}
+    events = {fwd_name: [], bwd_name: [], "linear": []}
+    originals = {}
+    native = fused and model._native_step_of() is not None
+    STAGES = {fwd_name: (1, 7), bwd_name: (21,), "linear": (2, 8)}
+    if native:
+        cabi._check(cabi.lib.cm_mace_step_timing(sum(1 << s for ids in STAGES.values() for s in ids)))
+    else:
+        originals = {fwd_name: getattr(cabi, fwd_name), bwd_name: getattr(cabi, bwd_name), "linear": cabi.linear}
 
-    def timed(name, fn, pred):
-        def wrapper(*a, **k):
-            if not pred(k):
-                return fn(*a, **k)
-            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s.record()
-            r = fn(*a, **k)
-            e.record()
-            events[name].append((s, e))
-            return r
-        return wrapper
+        def timed(name, fn, pred):
+            def wrapper(*a, **k):
+                if not pred(a, k):
+                    return fn(*a, **k)
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                r = fn(*a, **k)
+                e.record()
+                events[name].append((s, e))
+                return r
+            return wrapper
 
-    setattr(cabi, bwd_name, timed(bwd_name, originals[bwd_name], lambda k: not k.get("need_gX", True)))
-    setattr(cabi, fwd_name, timed(fwd_name, originals[fwd_name], lambda k: True))
-    # the 16-component channel-mixing launches (forward ones: no row_scale), when the model routes them through the C ABI
-    events["linear"] = []
-    originals["linear"] = cabi.linear
-
-    def timed_linear(X, *a, **k):
-        if X.dim() != 3 or k.get("row_scale") is not None:
-            return originals["linear"](X, *a, **k)
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
-        r = originals["linear"](X, *a, **k)
-        e.record()
-        events["linear"].append((s, e))
-        return r
-
-    cabi.linear = timed_linear
+        setattr(cabi, bwd_name, timed(bwd_name, originals[bwd_name], lambda a, k: not k.get("need_gX", True)))
+        setattr(cabi, fwd_name, timed(fwd_name, originals[fwd_name], lambda a, k: True))
+        # the 16-component channel-mixing launches (forward ones: no row_scale)
+        cabi.linear = timed("linear", originals["linear"], lambda a, k: a[0].dim() == 3 and k.get("row_scale") is None)
 
     torch.cuda.synchronize()
     t_start = time.perf_counter()
@@ -370,12 +367,22 @@ def main():
     elapsed = time.perf_counter() - t_start
     for name, fn in originals.items():
         setattr(cabi, name, fn)
+    stage_ms, stage_n = (ctypes.c_double * 32)(), (ctypes.c_int64 * 32)()
+    if native:
+        cabi._check(min(cabi.lib.cm_mace_step_timing_read(ctypes.addressof(stage_ms), ctypes.addressof(stage_n), 32), 0))
+        cabi._check(cabi.lib.cm_mace_step_timing(0))
 
     ms_per_step = 1e3 * elapsed / args.steps
     value = N * args.steps / elapsed
     assert bool(torch.isfinite(energy).all()) and bool(torch.isfinite(forces).all())
 
+    def launches(name):
+        return int(sum(stage_n[i] for i in STAGES[name])) if native else len(events[name])
+
     def avg_ms(name):
+        if native:
+            n = launches(name)
+            return sum(stage_ms[i] for i in STAGES[name]) / n if n else None
         ts = [s.elapsed_time(e) for s, e in events[name]]
         return sum(ts) / len(ts) if ts else None
 
@@ -396,7 +403,7 @@ def main():
     if fused:
         sh_b, spline_b = 88 * E, 4 * (8 * E * C + E)  # harmonics backward, spline backward (each operand once)
         sh_f, spline_f = 76 * E, 4 * (E + 8 * E * C)  # harmonics forward, spline forward (each operand once)
-        roofline = entry("mp_spline_forward_kernel<%d,true>" % C, fwd_fb, t_fwd, launches_timed=len(events[fwd_name]),
+        roofline = entry("mp_spline_forward_kernel<%d,true>" % C, fwd_fb, t_fwd, launches_timed=launches(fwd_name),
                          note="dominant kernel of the step by total time (two launches per step). Harmonics and radial "
                               "weights are evaluated in-kernel, so its own HBM operands are small: the radial coefficients "
                               "come from the 2 MB spline table in L2 (16 loads of 16 B per lane and edge, texture-address "
@@ -416,7 +423,7 @@ def main():
                                         "passing with tabulated R, spline evaluation, harmonics) divided by this launch's "
                                         "duration"})
         others = [entry("mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb, t_bwd,
-                        launches_timed=len(events[bwd_name]),
+                        launches_timed=launches(bwd_name),
                         note="bounded by VALU issue (~80% of all issue slots), see the counter summary")]
         t_lin = avg_ms("linear")
         if t_lin:
@@ -426,7 +433,7 @@ def main():
                            "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
                            "traffic": traffic.get(linear_kernel_name(C)) if default_workload else None,
                            "algorithmic_flops_per_launch": flops, "avg_launch_ms": round(t_lin, 4),
-                           "launches_timed": len(events["linear"]),
+                           "launches_timed": launches("linear"),
                            "note": "fp32-equivalent flops of the [N,16,C] x [C,C] channel mixing against the fp32 matrix "
                                    "peak; the kernel computes them as six bf16 piece products per fp32 product on "
                                    "v_mfma_f32_32x32x16_bf16 (6x the instruction flops: %.0f TFLOP/s of the 2500 TFLOP/s "
@@ -434,7 +441,7 @@ def main():
                                    % (6 * tf, 4 * (32 * N * C + 4 * C * C) // 10**6)})
     else:
         roofline = entry("mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b, t_bwd,
-                         launches_timed=len(events[bwd_name]))
+                         launches_timed=launches(bwd_name))
         others = [entry("mp_forward_kernel<%d>" % C, fwd_b, t_fwd)]
 
     # every stand-alone op of the path (the reference's op list: message passing with tabulated R[E,4,C] incl. the full

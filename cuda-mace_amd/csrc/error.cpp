@@ -17,5 +17,5 @@ void set_error(const char *fmt, ...) {
 }
 }  // namespace cm
 
-extern "C" int cm_abi_version(void) { return 7; }
+extern "C" int cm_abi_version(void) { return 8; }
 extern "C" const char *cm_last_error(void) { return cm::g_error; }

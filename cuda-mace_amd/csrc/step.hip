@@ -1,0 +1,271 @@
+// One energy + forces evaluation of the two-layer invariant model: the library enqueues every kernel of the step
+// itself, forward and then the hand-written backward chain, through the same entry points a caller could use one by
+// one.  Nothing here computes; this file is the order of the launches and the layout of the workspace.
+//
+// Forward                                         Backward (seed -1 on every node energy: the chain delivers forces)
+//   vec        = pos[snd] - pos[rcv] + shift        g1, g2    = readout backward
+//   M1         = MP(X1, vec, spline 0)              gB2       = g2 . Wprod2^T
+//   A          = mix0(M1)        (per element)      gA        = (gB2 * grad2) . Wmix1^T      (contraction backward folded)
+//   B1, grad1  = contraction 0 (A)                  gX2, gv2  = MP backward(X2, vec, spline 1, gA)
+//   h1         = B1 . Wprod1                        gh1       = gX2 . Wup^T + g1 ;  gh1 += skip^T(g2)
+//   sc         = skip(h1)        (per element)      gB1       = gh1 . Wprod1^T
+//   X2         = h1 . Wup                           gA        = (gB1 * grad1) . Wmix0^T      (per element)
+//   M2         = MP(X2, vec, spline 1)              gv1       = MP backward(X1, vec, spline 0, gA)   (no gX: X1 is constant)
+//   A          = mix1(M2)                           forces    = geometry backward(gv1 + gv2)
+//   B2, grad2  = contraction 1 (A)
+//   h2         = B2 . Wprod2 + sc
+//   E_n, dE/dh2, feats = readouts(h1, h2);  E_graph = sum over the graph's nodes
+#include <mutex>
+#include <vector>
+
+#include "common.hpp"
+
+namespace cm {
+namespace {
+
+// ---- optional per-stage timing: events on the launch stream around chosen stages of the step --------------------
+constexpr int kStages = 24;
+struct Pending {
+  int stage;
+  hipEvent_t start, stop;
+};
+std::mutex g_timing_mutex;
+unsigned g_timing_mask = 0;  // bit s set: stage s is bracketed by events
+std::vector<Pending> g_pending;
+std::vector<hipEvent_t> g_event_pool;
+double g_stage_ms[kStages] = {};
+int64_t g_stage_launches[kStages] = {};
+
+hipEvent_t take_event() {
+  if (!g_event_pool.empty()) {
+    hipEvent_t e = g_event_pool.back();
+    g_event_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+
+// Brackets one stage with events when its bit is set; used only through CM_STAGE below.
+struct StageTimer {
+  hipStream_t st;
+  int stage;
+  hipEvent_t start = nullptr;
+  StageTimer(hipStream_t s, int stage_, unsigned mask) : st(s), stage(stage_) {
+    if (mask >> stage & 1u) {
+      std::lock_guard<std::mutex> lock(g_timing_mutex);
+      start = take_event();
+      if (start) (void)hipEventRecord(start, st);
+    }
+  }
+  ~StageTimer() {
+    if (!start) return;
+    std::lock_guard<std::mutex> lock(g_timing_mutex);
+    hipEvent_t stop = take_event();
+    if (stop) {
+      (void)hipEventRecord(stop, st);
+      g_pending.push_back({stage, start, stop});
+    } else {
+      g_event_pool.push_back(start);
+    }
+  }
+};
+
+__global__ void fill_f64_kernel(double *p, int64_t n, double value) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    p[i] = value;
+}
+
+// a += b, 16 bytes per lane where the length allows
+__global__ void add_f32_kernel(float *__restrict__ a, const float *__restrict__ b, int64_t n) {
+  const int64_t n4 = n / 4;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n4;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    st4(a + 4 * i, ld4(a + 4 * i) + ld4(b + 4 * i));
+  if (blockIdx.x == 0 && threadIdx.x < n - 4 * n4) a[4 * n4 + threadIdx.x] += b[4 * n4 + threadIdx.x];
+}
+
+// out[g] = sum of x over the nodes ptr[g] .. ptr[g + 1]: one workgroup per graph, every thread a strided partial sum, a
+// tree over the partials: the same order on every run.
+constexpr int kSumThreads = 1024;
+__global__ __launch_bounds__(kSumThreads) void segment_sum_f64_kernel(const double *__restrict__ x, const int32_t *__restrict__ ptr,
+                                                                     double *__restrict__ out) {
+  __shared__ double part[kSumThreads];
+  const int lo = ptr[blockIdx.x], hi = ptr[blockIdx.x + 1];
+  double s = 0.0;
+  for (int i = lo + threadIdx.x; i < hi; i += kSumThreads) s += x[i];
+  part[threadIdx.x] = s;
+  __syncthreads();
+  for (int d = kSumThreads / 2; d > 0; d >>= 1) {
+    if (threadIdx.x < d) part[threadIdx.x] += part[threadIdx.x + d];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = part[0];
+}
+
+inline size_t align256(size_t n) { return (n + 255) & ~static_cast<size_t>(255); }
+
+// Carves the workspace; the same walk sizes it (base == nullptr) and lays it out.
+struct Layout {
+  float *vec, *len, *gv1, *gv2, *bufM1, *bufM2, *bufA, *edge_scratch;
+  float *B1, *h1, *sc, *X2, *B2, *h2, *d_h2, *g1, *g2, *gB, *gX2, *gh1a, *gh1;
+  double *seed;
+  size_t bytes;
+
+  Layout(void *base, int64_t N, int64_t E, int C) {
+    size_t at = 0;
+    auto take = [&](size_t n) {
+      char *p = base ? static_cast<char *>(base) + at : nullptr;
+      at += align256(n);
+      return p;
+    };
+    auto f = [&](int64_t n) { return reinterpret_cast<float *>(take(static_cast<size_t>(n) * sizeof(float))); };
+    const int64_t NC = N * C;
+    vec = f(3 * E), len = f(E), gv1 = f(3 * E), gv2 = f(3 * E);
+    bufM1 = f(16 * NC), bufM2 = f(16 * NC), bufA = f(16 * NC);
+    edge_scratch = f(E * C);
+    B1 = f(NC), h1 = f(NC), sc = f(NC), X2 = f(NC), B2 = f(NC), h2 = f(NC), d_h2 = f(NC);
+    g1 = f(NC), g2 = f(NC), gB = f(NC), gX2 = f(NC), gh1a = f(NC), gh1 = f(NC);
+    seed = reinterpret_cast<double *>(take(static_cast<size_t>(N) * sizeof(double)));
+    bytes = at;
+  }
+};
+
+}  // namespace
+}  // namespace cm
+
+extern "C" size_t cm_mace_step_workspace(int64_t nnodes, int64_t nedges, int channels) {
+  if (nnodes < 0 || nedges < 0 || channels <= 0) return 0;
+  return cm::Layout(nullptr, nnodes, nedges, channels).bytes;
+}
+
+// Runs one stage; with the stage's timing bit set, between two events recorded on the stream.
+#define CM_STAGE(id, call)                          \
+  do {                                              \
+    cm::StageTimer timer_(st, (id), timing_mask);   \
+    const int rc_ = (call);                         \
+    if (rc_ != CM_OK) return rc_;                   \
+  } while (0)
+
+extern "C" int cm_mace_step_timing(unsigned stage_mask) {
+  std::lock_guard<std::mutex> lock(cm::g_timing_mutex);
+  cm::g_timing_mask = stage_mask & ((1u << cm::kStages) - 1u);
+  for (cm::Pending &p : cm::g_pending) {
+    cm::g_event_pool.push_back(p.start);
+    cm::g_event_pool.push_back(p.stop);
+  }
+  cm::g_pending.clear();
+  for (int s = 0; s < cm::kStages; ++s) cm::g_stage_ms[s] = 0.0, cm::g_stage_launches[s] = 0;
+  return CM_OK;
+}
+
+extern "C" int cm_mace_step_timing_read(double *total_ms, int64_t *launches, int capacity) {
+  CM_REQUIRE(total_ms && launches && capacity >= cm::kStages, "cm_mace_step_timing_read: need room for %d stages", cm::kStages);
+  std::lock_guard<std::mutex> lock(cm::g_timing_mutex);
+  for (cm::Pending &p : cm::g_pending) {
+    float ms = 0.f;
+    if (hipEventSynchronize(p.stop) == hipSuccess && hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess) {
+      cm::g_stage_ms[p.stage] += ms;
+      cm::g_stage_launches[p.stage] += 1;
+    }
+    cm::g_event_pool.push_back(p.start);
+    cm::g_event_pool.push_back(p.stop);
+  }
+  cm::g_pending.clear();
+  for (int s = 0; s < cm::kStages; ++s) total_ms[s] = cm::g_stage_ms[s], launches[s] = cm::g_stage_launches[s];
+  return cm::kStages;
+}
+
+extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, const double *positions, const double *shifts,
+                            void *workspace, size_t workspace_bytes, double *interaction_energy, double *node_energy,
+                            double *forces, double *node_feats, cm_stream_t stream) {
+  CM_REQUIRE(w && g, "cm_mace_step: NULL weights or graph");
+  const int64_t N = g->nnodes, E = g->nedges;
+  const int C = w->channels, ne = w->nelements;
+  CM_REQUIRE(N >= 0 && E >= 0 && g->ngraphs >= 1, "cm_mace_step: negative size or no graph");
+  CM_REQUIRE(cm_channels_supported(C), "cm_mace_step: channels=%d must be a multiple of 32 in [32, 256]", C);
+  CM_REQUIRE(ne >= 1, "cm_mace_step: nelements must be at least 1");
+  CM_REQUIRE(interaction_energy && g->graph_ptr, "cm_mace_step: NULL energy output or graph_ptr");
+  hipStream_t st = cm::as_stream(stream);
+  unsigned timing_mask;
+  {
+    std::lock_guard<std::mutex> lock(cm::g_timing_mutex);
+    timing_mask = cm::g_timing_mask;
+  }
+  if (N == 0) {
+    hipLaunchKernelGGL(cm::fill_f64_kernel, dim3(1), dim3(64), 0, st, interaction_energy, static_cast<int64_t>(g->ngraphs), 0.0);
+    return cm::check_launch("cm_mace_step");
+  }
+  CM_REQUIRE(positions && node_energy && forces, "cm_mace_step: NULL positions or output");
+  CM_REQUIRE(E == 0 || shifts, "cm_mace_step: NULL shifts");
+  CM_REQUIRE(g->first_occ && g->sender_offsets && g->elem_perm && g->elem_offsets && g->onehot_perm && g->onehot_offsets && g->X1,
+             "cm_mace_step: NULL graph structure");
+  CM_REQUIRE(E == 0 || (g->receiver && g->sender && g->sender_perm), "cm_mace_step: NULL edge list");
+  for (int t = 0; t < 2; ++t)
+    CM_REQUIRE(w->spline[t] && w->mix_WT[t] && w->mix_W[t] && w->T3[t] && w->T2[t] && w->T1[t] && w->prod_WT[t] && w->prod_W[t] &&
+                   (w->mono3[t] == nullptr) == (w->mono2[t] == nullptr),
+               "cm_mace_step: NULL weight of layer %d", t);
+  CM_REQUIRE(w->r_knots && w->up_WT && w->up_W && w->skip_WT && w->skip_W && w->w1 && w->W2a && w->w2b, "cm_mace_step: NULL weight");
+  const cm::Layout L(workspace, N, E, C);
+  if (workspace == nullptr || workspace_bytes < L.bytes) {
+    cm::set_error("cm_mace_step: workspace of %zu bytes, need %zu", workspace_bytes, L.bytes);
+    return CM_ENOSPC;
+  }
+  CM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255) == 0, "cm_mace_step: workspace must be 256-byte aligned");
+  const int32_t *oh_perm = g->onehot_perm, *oh_off = g->onehot_offsets;
+  const int32_t *el_perm = g->elem_perm, *el_off = g->elem_offsets;
+  const float *none = nullptr;
+
+  // ---- forward ----
+  CM_STAGE(0, cm_edge_geometry_forward(positions, g->receiver, g->sender, shifts, g->node_rows, N, E, L.vec, L.len, stream));
+  const float *X[2] = {g->X1, L.X2};
+  float *bufM[2] = {L.bufM1, L.bufM2};
+  float *B[2] = {L.B1, L.B2};
+  float *h[2] = {L.h1, L.h2};
+  for (int t = 0; t < 2; ++t) {
+    if (t == 1) {
+      // residual skip connection per element and linear_up, both of the first layer's output
+      CM_STAGE(5, cm_linear(L.h1, w->skip_WT, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, w->skip_scale, none, none, L.sc, stream));
+      CM_STAGE(6, cm_linear(L.h1, w->up_WT, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.X2, stream));
+    }
+    CM_STAGE(t == 0 ? 1 : 7, cm_mp_edge_forward(X[t], L.vec, w->r_knots, w->spline[t], w->nknots, w->r_width, w->r_max, g->sender, g->first_occ, N,
+                               E, C, bufM[t], stream));
+    if (t == 0)
+      CM_STAGE(2, cm_linear(bufM[t], w->mix_WT[t], oh_perm, oh_off, N, ne + 1, 1, 16, C, C, w->mix_scale[t], none, none, L.bufA, stream));
+    else
+      CM_STAGE(8, cm_linear(bufM[t], w->mix_WT[t], nullptr, nullptr, N, 1, 0, 16, C, C, w->mix_scale[t], none, none, L.bufA, stream));
+    // the contraction's gradient table takes the place of the message, which is no longer needed
+    CM_STAGE(t == 0 ? 3 : 9, cm_symcon_forward(L.bufA, el_perm, el_off, w->mono3[t], w->n3[t], w->mono2[t], w->n2[t], w->T3[t], w->T2[t], w->T1[t], N,
+                              ne, C, B[t], bufM[t], stream));
+    CM_STAGE(t == 0 ? 4 : 10, cm_linear(B[t], w->prod_WT[t], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, t == 1 ? L.sc : none, h[t], stream));
+  }
+  CM_STAGE(11, cm_readout_forward(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden, node_energy,
+                             L.d_h2, node_feats, g->node_rows, stream));
+  hipLaunchKernelGGL(cm::segment_sum_f64_kernel, dim3(g->ngraphs), dim3(cm::kSumThreads), 0, st, node_energy, g->graph_ptr,
+                     interaction_energy);
+
+  // ---- backward: d(-sum of node energies) / d positions ----
+  hipLaunchKernelGGL(cm::fill_f64_kernel, dim3(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(N, 256), 1024))), dim3(256), 0,
+                     st, L.seed, N, -1.0);
+  CM_STAGE(13, cm_readout_backward(L.seed, w->w1, L.d_h2, w->scale, N, C, L.g1, L.g2, stream));
+  // layer 1 (second interaction)
+  CM_STAGE(14, cm_linear(L.g2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.gB, stream));
+  CM_STAGE(15, cm_linear(L.bufM2, w->mix_W[1], nullptr, nullptr, N, 1, 0, 16, C, C, w->mix_scale[1], L.gB, none, L.bufA, stream));
+  CM_STAGE(16, cm_mp_edge_backward(L.X2, L.vec, w->r_knots, w->spline[1], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
+                              g->first_occ, g->sender_perm, g->sender_offsets, N, E, C, L.gX2, L.gv2, L.edge_scratch, stream));
+  CM_STAGE(17, cm_linear(L.gX2, w->up_W, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, L.g1, L.gh1a, stream));
+  CM_STAGE(18, cm_linear(L.g2, w->skip_W, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, w->skip_scale, none, L.gh1a, L.gh1, stream));
+  // layer 0 (first interaction): its input features depend on the species alone, so no gradient with respect to them
+  CM_STAGE(19, cm_linear(L.gh1, w->prod_W[0], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.gB, stream));
+  CM_STAGE(20, cm_linear(L.bufM1, w->mix_W[0], oh_perm, oh_off, N, ne + 1, 1, 16, C, C, w->mix_scale[0], L.gB, none, L.bufA, stream));
+  CM_STAGE(21, cm_mp_edge_backward(g->X1, L.vec, w->r_knots, w->spline[0], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
+                              g->first_occ, nullptr, nullptr, N, E, C, nullptr, L.gv1, nullptr, stream));
+  if (E > 0)
+    hipLaunchKernelGGL(cm::add_f32_kernel, dim3(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(3 * E, 4 * 256), 2048))),
+                       dim3(256), 0, st, L.gv1, L.gv2, 3 * E);
+  CM_STAGE(23, cm_edge_geometry_backward(positions, g->receiver, g->sender, shifts, g->node_rows, g->first_occ, g->sender_perm,
+                                    g->sender_offsets, L.gv1, nullptr, N, E, forces, nullptr, stream));
+  return cm::check_launch("cm_mace_step");
+}

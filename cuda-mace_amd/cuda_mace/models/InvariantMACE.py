@@ -304,7 +304,8 @@ class _WeightsToken:
 
 class OptimizedInvariantMACE(torch.nn.Module):
     def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True,
-                 fused_readout: bool = True, fused_contraction: bool = True, spatial_order_min_atoms: Optional[int] = 8192):
+                 fused_readout: bool = True, fused_contraction: bool = True, spatial_order_min_atoms: Optional[int] = 8192,
+                 native_step: bool = True):
         """fused_radial=True evaluates the spherical harmonics and the radial spline inside the message-passing kernels
         (same numbers; no [16, nedges] or [nedges, 4C] tensors in memory); False keeps the reference's separate
         SphericalHarmonics -> CubicSpline -> message passing steps.  fused_readout=True evaluates both readouts, scale
@@ -312,6 +313,10 @@ class OptimizedInvariantMACE(torch.nn.Module):
         form, or several heads) runs the modules themselves in fp64 as the reference does.  fused_contraction=True runs the
         channel-mixing linear before each symmetric contraction and the contraction as one autograd node whose backward is
         a single kernel; False keeps the reference's separate Linear / ElementalLinear and SymmetricContraction ops.
+        native_step=True (with all three fusions on) hands an inference step without strain -- energy and forces of one
+        head -- to the library as ONE call that enqueues every kernel of the forward and of the backward chain itself
+        (no interpreter or autograd engine between the launches; same kernels, order and numbers as the autograd path,
+        which still serves training, virials / stress and compute_force=False).
         spatial_order_min_atoms: from this many atoms on, the model works on a relabelled copy of the graph in which
         atoms that are close in space have close indices (derived once per edge_index tensor), so that the gathers of
         sender rows hit in cache; outputs come back in the caller's order.  None switches the relabelling off."""
@@ -375,6 +380,22 @@ class OptimizedInvariantMACE(torch.nn.Module):
         # kept for reference like upstream does, but not as a registered sub-module: moving or casting the
         # optimised model must not touch the caller's original model
         object.__setattr__(self, "orig_model", mace_model)
+        self.native_step = bool(native_step)
+        object.__setattr__(self, "_native", None)  # NativeStep, built on first use (holds device addresses: not pickled)
+
+    def __getstate__(self):
+        state = dict(self.__dict__)
+        state["_native"] = None
+        return state
+
+    def _native_step_of(self):
+        if self._native is None:
+            from cuda_mace.ops.native_step import NativeStep
+
+            if self._contraction_builtin is None:
+                self._fold_contraction_tables()
+            object.__setattr__(self, "_native", NativeStep(self) if NativeStep.supported(self) else False)
+        return self._native or None
 
     def _fold_contraction_tables(self):
         """Per layer: the packed coupling tables regrouped into monomials (host, once) and folded with the per-element
@@ -497,6 +518,23 @@ class OptimizedInvariantMACE(torch.nn.Module):
                                    lambda: (edge_index[0].int().contiguous(), edge_index[1].int().contiguous()))
         node_attrs32, atom_types = _cached(node_attrs, "_cm_species", None,
                                            lambda: (node_attrs.detach().float(), node_attrs.detach().argmax(dim=-1).int()))
+
+        strained = compute_virials or compute_stress or compute_displacement
+        if (self.native_step and not training and compute_force and not strained and node_heads is None
+                and positions.is_cuda and (node_rows is None or positions_in_caller_order)):
+            native = self._native_step_of()
+            if native is not None:
+                rows32 = None if node_rows is None else node_rows[0]
+                handle = _cached_for(edge_index, "_cm_native_graph_%d" % id(self._weights_token), node_attrs,
+                                     lambda: native.graph(edge_index, receiver, sender, node_attrs32, atom_types, data["ptr"],
+                                                          node_feats_up, rows32))
+                res = native(handle, positions, shifts)
+                inter_e = res["interaction_energy"]
+                return {
+                    "energy": e0 + inter_e, "node_energy": node_e0 + res["node_energy"], "interaction_energy": inter_e,
+                    "forces": res["forces"].to(data["positions"].dtype), "virials": None, "stress": None, "hessian": None,
+                    "displacement": displacement, "node_feats": res["node_feats"], "edge_forces": None,
+                }
 
         # vectors = positions[edge_index[1]] - positions[edge_index[0]] + shifts in fp64, rounded once to fp32
         vectors32, lengths32 = EdgeGeometryAutograd.apply(positions, shifts, receiver, sender,

@@ -381,6 +381,83 @@ int cm_readout_forward(const float *h1, const float *h2, const double *w1, const
 int cm_readout_backward(const double *grad_node_energies, const double *w1, const float *d_h2, double scale,
                         int64_t nnodes, int channels, float *grad_h1, float *grad_h2, cm_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * One energy + forces evaluation of the two-layer invariant model as a single call: every kernel of the step, forward
+ * and backward, enqueued back to back by the library itself.  It replaces, for inference, what the reference runs as a
+ * Python forward over its TorchScript classes followed by an autograd backward (models/InvariantMACE.py:246-379:
+ * interactions :76-160, products :330, readouts :336, scale/shift :344, forces through get_outputs :354): same kernels,
+ * same order, same numbers as that sequence, without a Python interpreter or an autograd engine between the launches
+ * (about thirty launches; host cost of a step drops from ~0.4 ms to well under 0.1 ms).
+ *
+ * cm_mace_weights: the model's frozen weights in the layouts the op modules hold them (device pointers).
+ *   spline[t]      [nknots - 1, 4, 4C]   radial spline table of layer t (cm_spline_forward's coeffs)
+ *   mix_WT/mix_W   channel mixing between message passing and contraction, transposed / plain blocks with mix_scale:
+ *                  layer 0 per element [ne, 4, C, C] (the per-l linear composed with the per-element linear,
+ *                  models/InvariantMACE.py:56-74, 113-116), layer 1 [4, C, C]; 1 / avg_num_neighbors folded in
+ *   T3/T2/T1       contraction coefficient tables of layer t (cm_symcon_tables); mono3/mono2 NULL selects the
+ *                  built-in l_max = 3 structure, otherwise the monomial lists with n3/n2 entries
+ *   prod_WT/prod_W [C, C] linear after the contraction (1/sqrt(C) folded in), both orientations
+ *   up_WT/up_W     [C, C] linear_up of layer 1 (the second layer; layer 0's acts on species-only features, see X1)
+ *   skip_WT/skip_W [ne, C, C] residual skip connection of the second layer per element, with skip_scale
+ *   w1, W2a [C, hidden], w2b [hidden], act_cst, scale, shift: cm_readout_forward's operands
+ * cm_mace_graph: what depends on the neighbour list and the species only (device pointers; rebuilt when they change).
+ *   receiver (non-decreasing) / sender int32 [nedges]; first_occ = cm_first_occurences(receiver);
+ *   sender_perm / sender_offsets = cm_stable_key_sort(sender, nedges, nnodes);
+ *   elem_perm / elem_offsets = cm_stable_key_sort(element index, nnodes, ne)           [nnodes], [ne + 1]
+ *   onehot_perm / onehot_offsets: the same grouping with one more, empty-weight group for atoms whose one-hot row
+ *     names no element [nnodes], [ne + 2] (pass the element grouping with a closing repeated offset if there are none)
+ *   node_rows int32 [nnodes] or NULL: atom n of the lists is row node_rows[n] of positions / forces / node_feats
+ *   graph_ptr int32 [ngraphs + 1]: node range of every graph of the batch, in the order of the lists
+ *   X1 fp32 [nnodes, C]: linear_up(node_embedding(species)) of the first layer
+ * Per call: positions fp64 [nnodes, 3], shifts fp64 [nedges, 3]; outputs interaction_energy fp64 [ngraphs] (sum of the
+ * node energies of each graph, in a fixed order), node_energy fp64 [nnodes] (interaction part, in list order), forces
+ * fp64 [nnodes, 3] = -d(sum of energies)/d positions (rows of the caller when node_rows is given), node_feats fp64
+ * [nnodes, 2C] or NULL.  workspace: cm_mace_step_workspace(nnodes, nedges, channels) bytes, 256-byte aligned; its
+ * contents are scratch.  Nothing is allocated, so the call can be captured into a HIP graph.
+ */
+typedef struct cm_mace_weights {
+  int channels, nelements, nknots, hidden;
+  float r_width, r_max;
+  const float *r_knots;
+  const float *spline[2];
+  const float *mix_WT[2], *mix_W[2];
+  float mix_scale[2];
+  const float *T3[2], *T2[2], *T1[2];
+  const int32_t *mono3[2], *mono2[2];
+  int n3[2], n2[2];
+  const float *prod_WT[2], *prod_W[2];
+  const float *up_WT, *up_W;
+  const float *skip_WT, *skip_W;
+  float skip_scale;
+  const double *w1, *W2a, *w2b;
+  double act_cst, scale, shift;
+} cm_mace_weights;
+
+typedef struct cm_mace_graph {
+  int64_t nnodes, nedges;
+  int ngraphs;
+  const int32_t *receiver, *sender, *first_occ, *sender_perm, *sender_offsets;
+  const int32_t *elem_perm, *elem_offsets, *onehot_perm, *onehot_offsets;
+  const int32_t *node_rows, *graph_ptr;
+  const float *X1;
+} cm_mace_graph;
+
+/* Per-stage timing of cm_mace_step (off by default): with bit s of stage_mask set, stage s of every later step is
+ * bracketed by two events recorded on the launch stream; cm_mace_step_timing_read waits for the outstanding events and
+ * returns, per stage, the accumulated milliseconds and the number of timed launches since the mask was set (arrays of
+ * at least 24 entries; the return value is the number of stages).  Setting a mask resets the accumulators.  Leave it
+ * off while a step is being captured into a graph.  Stages: 0 edge geometry; 1 / 7 message passing forward of layer
+ * 0 / 1; 2 / 8 channel mixing; 3 / 9 contraction; 4 / 10 linear after it; 5 skip connection; 6 linear_up; 11 readouts;
+ * 13 readout backward; 14 / 19 linear after the contraction, backward; 15 / 20 channel mixing backward (contraction
+ * backward folded in); 16 message passing backward of layer 1 (edge pass + sender pass); 21 of layer 0 (edge pass
+ * only); 17 linear_up backward; 18 skip backward; 23 edge geometry backward (forces). */
+int cm_mace_step_timing(unsigned stage_mask);
+int cm_mace_step_timing_read(double *total_ms, int64_t *launches, int capacity);
+size_t cm_mace_step_workspace(int64_t nnodes, int64_t nedges, int channels);
+int cm_mace_step(const cm_mace_weights *weights, const cm_mace_graph *graph, const double *positions, const double *shifts,
+                 void *workspace, size_t workspace_bytes, double *interaction_energy, double *node_energy, double *forces,
+                 double *node_feats, cm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

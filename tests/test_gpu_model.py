@@ -310,3 +310,55 @@ def test_model_in_a_foreign_coupling_basis(cabi):
     ref_own = M.energy_and_forces(own.export_params(), data)
     ref = M.energy_and_forces(params, data)
     assert abs(float(ref_own["interaction_energy"]) - float(ref["interaction_energy"])) > 1e-3 * abs(float(ref["interaction_energy"]))
+
+
+@pytest.mark.parametrize("case", ["cluster", "periodic96", "periodic192", "batch_relabelled", "isolated_atoms"])
+def test_native_step_equals_autograd_path(cabi, case):
+    """The step enqueued by the library in one call (cm_mace_step) against the same kernels driven from Python through
+    autograd: identical node energies and features (same kernels in the same order), energies equal up to the order of
+    the final sum, forces equal up to single-precision rounding of the gradient sums (the library adds the three
+    contributions to the gradient of the first layer's features in the linear kernels' epilogues, autograd in separate
+    additions)."""
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.utils.synthetic import collate
+
+    kwargs = {}
+    if case == "cluster":
+        data, C, numbers = make_system(21, 4, seed=0, density=None, cluster_box=8.0), 64, (1, 6, 7, 8)
+    elif case == "periodic96":
+        data, C, numbers = make_system(300, 10, seed=1, density=0.1), 96, tuple(range(1, 11))
+    elif case == "periodic192":
+        data, C, numbers = make_system(250, 10, seed=3, density=0.1), 192, tuple(range(1, 11))
+    elif case == "batch_relabelled":
+        data = collate([make_system(n, 4, seed=30 + k, density=0.1) for k, n in enumerate((150, 230, 120))])
+        C, numbers, kwargs = 64, (1, 6, 7, 8), dict(spatial_order_min_atoms=0)
+    else:  # a sparse cluster: most atoms have no neighbour at all
+        data, C, numbers = make_system(12, 4, seed=2, density=None, cluster_box=40.0, min_dist=3.0), 32, (1, 6, 7, 8)
+    N = data["positions"].shape[0]
+    up = SyntheticInvariantMACE(channels=C, atomic_numbers=numbers, avg_num_neighbors=max(data["edge_index"].shape[1] / N, 1.0),
+                                seed=4, atomic_energies=torch.linspace(-3.0, -1.0, len(numbers), dtype=torch.float64), shift=0.1)
+    native = OptimizedInvariantMACE(up, device="cuda", native_step=True, **kwargs)
+    eager = OptimizedInvariantMACE(up, device="cuda", native_step=False, **kwargs)
+    dev = to_device(data, "cuda")
+    a, b = native(dict(dev)), eager(dict(dev))
+    assert native._native not in (None, False) and eager._native is None  # the fast path ran / stayed off
+    assert a["forces"].grad_fn is None and a["energy"].grad_fn is None
+    _say("  %s: E native %.12g autograd %.12g" % (case, float(a["energy"].sum()), float(b["energy"].sum())))
+    torch.testing.assert_close(a["energy"], b["energy"].detach(), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(a["interaction_energy"], b["interaction_energy"].detach(), rtol=1e-12, atol=1e-12)
+    assert torch.equal(a["node_energy"], b["node_energy"].detach())
+    fscale = float(b["forces"].abs().max())
+    torch.testing.assert_close(a["forces"], b["forces"].detach(), rtol=0, atol=5e-7 * fscale)
+    assert torch.equal(a["node_feats"], b["node_feats"].detach())
+    assert a["virials"] is None and a["stress"] is None and a["displacement"].shape == b["displacement"].shape
+    again = native(dict(dev))
+    assert torch.equal(again["forces"], a["forces"]) and torch.equal(again["energy"], a["energy"])
+    # what the fast path does not cover still works on the same model: strain derivatives go through autograd
+    if case == "periodic96":
+        c = native(dict(dev), compute_virials=True)
+        d = eager(dict(dev), compute_virials=True)
+        assert torch.equal(c["virials"], d["virials"]) and torch.equal(c["forces"], d["forces"])
+        torch.testing.assert_close(c["forces"], a["forces"], rtol=0, atol=5e-7 * fscale)
+    ref = M.energy_and_forces(up.export_params(), data)
+    assert abs(float(a["energy"].sum()) - float(ref["energy"])) <= E_RTOL * abs(float(ref["energy"]))
+    assert float((a["forces"].cpu() - ref["forces"]).abs().max()) <= F_ATOL
