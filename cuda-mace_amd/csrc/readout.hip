@@ -64,7 +64,20 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
   if (live) {
     const float *row1 = h1 + static_cast<int64_t>(node0 + r) * C;
     for (int c = j; c < C; c += kHidden) e1 += static_cast<double>(row1[c]) * w1[c];
-    for (int c = 0; c < C; ++c) z += static_cast<double>(s2[r * kLdS + c]) * sW[c * kLdW + j];
+    // four independent partial sums: the fp64 multiply-add chain is otherwise as long as the channel count
+    double z0 = 0.0, z1 = 0.0, z2 = 0.0, z3 = 0.0;
+    const float *srow = s2 + r * kLdS;
+    const double *wcol = sW + j;
+    int c = 0;
+#pragma unroll 2
+    for (; c + 3 < C; c += 4) {
+      z0 += static_cast<double>(srow[c]) * wcol[c * kLdW];
+      z1 += static_cast<double>(srow[c + 1]) * wcol[(c + 1) * kLdW];
+      z2 += static_cast<double>(srow[c + 2]) * wcol[(c + 2) * kLdW];
+      z3 += static_cast<double>(srow[c + 3]) * wcol[(c + 3) * kLdW];
+    }
+    for (; c < C; ++c) z0 += static_cast<double>(srow[c]) * wcol[c * kLdW];
+    z = (z0 + z1) + (z2 + z3);
   }
   double e2 = 0.0, dj = 0.0;
   if (live && j < H) {
