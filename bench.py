@@ -89,7 +89,7 @@ def _time_ms(torch, fn, reps):
     return s.elapsed_time(e) / reps
 
 
-def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=True):
+def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=True, with_per_component=False):
     """(label, kernels, algorithmic bytes, callable) for every stand-alone op of the path on random operands of the given
     shape.  Bytes count each operand once.  `rcv` (sorted) and `snd` are int32 device tensors."""
     import numpy as np
@@ -117,6 +117,16 @@ def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=
          "mp_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,false>" % (C, C), bwd_full_b,
          lambda: cabi.mp_backward(X, Y, R, G, snd, fo, perm, off, N)),
     ]
+    if with_per_component:
+        # the same op with a radial weight per component, R [E,16,C]: four times the radial bytes
+        R16 = torch.randn(E, 16, C, device="cuda", generator=g)
+        cases += [
+            ("mp_forward (R per component [E,16,C])", "mp_per_m_forward_kernel<%d>" % C,
+             4 * (16 * E * C + 16 * E + 17 * N * C) + 8 * E, lambda: cabi.mp_forward(X, Y, R16, snd, fo, N)),
+            ("mp_backward gX,gY,gR (R per component): edge pass + sender pass",
+             "mp_per_m_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,false>" % (C, C),
+             4 * (32 * E * C + 32 * E + 18 * N * C) + 8 * E, lambda: cabi.mp_backward(X, Y, R16, G, snd, fo, perm, off, N)),
+        ]
     if with_fused:
         cases += [
             ("mp_edge_forward (fused harmonics + spline)", "mp_spline_forward_kernel<%d,true>" % C, fwd_fb,
@@ -189,7 +199,7 @@ def isolated_ops(args, torch, cabi, make_system, reps=3):
     rcv2, snd2 = config2_edges(torch)
     print("# configuration 2: N=4096 E=%d C=96" % rcv2.numel(), flush=True)
     for label, kernel, nbytes, fn in op_cases(torch, cabi, 4096, rcv2.numel(), 96, args.elements, rcv2, snd2, with_fused=False,
-                                              with_node_ops=False):
+                                              with_node_ops=False, with_per_component=True):
         ms = _time_ms(torch, fn, 10 * reps)
         print("%-62s %-70s %9.1f us  algorithmic %12d B  %8.1f GB/s" % (label, kernel, ms * 1e3, nbytes, nbytes / ms / 1e6), flush=True)
 
@@ -209,9 +219,10 @@ def standalone_rooflines(torch, cabi, N, E, C, ne, rcv, snd, reps=10):
 
     at_c4 = rows(op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=False), reps, shape="N=%d E=%d C=%d" % (N, E, C))
     rcv2, snd2 = config2_edges(torch)
-    at_c2 = rows(op_cases(torch, cabi, 4096, rcv2.numel(), 96, ne, rcv2, snd2, with_fused=False, with_node_ops=False), 5 * reps,
+    at_c2 = rows(op_cases(torch, cabi, 4096, rcv2.numel(), 96, ne, rcv2, snd2, with_fused=False, with_node_ops=False,
+                          with_per_component=True), 5 * reps,
                  shape="configuration 2: N=4096 E=%d C=96, uniform random senders" % rcv2.numel())
-    fwd, full = at_c2[0], at_c2[2]
+    fwd, full, fwd16, full16 = at_c2[0], at_c2[2], at_c2[3], at_c2[4]
     c2 = {"workload": "isolated invariant message passing forward + full backward (gX, gY, gR), 4096 nodes x 30 edges, 96 "
                       "channels, R[E,4,C] as the reference's op takes it",
           "fwd_ms": fwd["avg_launch_ms"], "bwd_ms": full["avg_launch_ms"],
@@ -220,6 +231,12 @@ def standalone_rooflines(torch, cabi, N, E, C, ne, rcv, snd, reps=10):
           "GB/s": round((fwd["algorithmic_bytes_per_launch"] + full["algorithmic_bytes_per_launch"])
                         / ((fwd["avg_launch_ms"] + full["avg_launch_ms"]) * 1e-3) / 1e9, 1)}
     c2["frac_of_hbm_peak"] = round(c2["GB/s"] / HBM_PEAK_GBPS, 4)
+    b16 = fwd16["algorithmic_bytes_per_launch"] + full16["algorithmic_bytes_per_launch"]
+    t16 = fwd16["avg_launch_ms"] + full16["avg_launch_ms"]
+    c2["per_component_weights"] = {
+        "workload": "the same with radial weights per component, R[E,16,C] (the shape the configuration is worded with)",
+        "fwd_ms": fwd16["avg_launch_ms"], "bwd_ms": full16["avg_launch_ms"], "algorithmic_bytes": b16,
+        "GB/s": round(b16 / (t16 * 1e-3) / 1e9, 1), "frac_of_hbm_peak": round(b16 / (t16 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
     return at_c4 + at_c2, c2
 
 

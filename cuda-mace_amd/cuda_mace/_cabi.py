@@ -45,6 +45,8 @@ SIGNATURES = {
     "cm_stable_key_sort_static": (_i32, [_p, _i64, _i64, _p, _p, _p]),
     "cm_mp_forward": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _p, _p]),
     "cm_mp_backward": (_i32, [_p] * 8 + [_i64, _i64, _i32] + [_p] * 5),
+    "cm_mp_forward_per_m": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _p, _p]),
+    "cm_mp_backward_per_m": (_i32, [_p] * 8 + [_i64, _i64, _i32] + [_p] * 5),
     "cm_mp_spline_forward": (_i32, [_p] * 5 + [_i32, _f32, _f32, _p, _p, _i64, _i64, _i32, _p, _p]),
     "cm_mp_spline_backward": (_i32, [_p] * 5 + [_i32, _f32, _f32] + [_p] * 5 + [_i64, _i64, _i32] + [_p] * 5),
     "cm_mp_edge_forward": (_i32, [_p] * 4 + [_i32, _f32, _f32, _p, _p, _i64, _i64, _i32, _p, _p]),
@@ -188,14 +190,24 @@ def stable_key_sort_static(keys: torch.Tensor, nkeys: int, perm: torch.Tensor, o
 
 
 # ---- message passing --------------------------------------------------------------------------
+def _radial_blocks(R, E: int, C: int, D) -> int:
+    """4 for radial weights per degree (the reference's [nedges, 4, C]), 16 for weights per component ([nedges, 16, C],
+    fp32 only)."""
+    if R.numel() == E * 4 * C and not (R.dim() == 3 and R.shape[1] == 16):
+        return 4
+    if R.numel() == E * 16 * C and D == F32:
+        return 16
+    raise CudaMaceError("radial must hold nedges*4*channels = %d values (or nedges*16*channels in fp32), got %d" % (E * 4 * C, R.numel()))
+
+
 def mp_forward(X, Y, R, sender, first_occ, nnodes: int) -> torch.Tensor:
     fn, D = _typed("cm_mp_forward", X)
     C = X.shape[-1]
     E = sender.numel()
     if Y.shape != (16, E):
         raise CudaMaceError("Y must be [16, nedges] = [16, %d], got %s" % (E, tuple(Y.shape)))
-    if R.numel() != E * 4 * C:
-        raise CudaMaceError("radial must hold nedges*4*channels = %d values, got %d" % (E * 4 * C, R.numel()))
+    if _radial_blocks(R, E, C, D) == 16:
+        fn = lib.cm_mp_forward_per_m
     if X.shape[0] != nnodes:
         raise CudaMaceError("X must be [nnodes, channels]")
     out = torch.empty(nnodes, 16, C, dtype=D, device=X.device)
@@ -214,9 +226,12 @@ def mp_backward(X, Y, R, grad_out, sender, first_occ, sender_perm, sender_offset
     C = X.shape[-1]
     E = sender.numel()
     dev = X.device
+    blocks = _radial_blocks(R, E, C, D)
+    if blocks == 16:
+        fn = lib.cm_mp_backward_per_m
     gX = torch.empty(nnodes, C, dtype=D, device=dev) if need_gX else None
     gY = torch.empty(16, E, dtype=D, device=dev) if need_gY else None
-    gR = torch.empty(E, 4, C, dtype=D, device=dev) if need_gR else None
+    gR = torch.empty(E, blocks, C, dtype=D, device=dev) if need_gR else None
     scratch = torch.empty(E, C, dtype=D, device=dev) if need_gX else None
     _check(
         fn(

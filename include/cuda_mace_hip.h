@@ -126,6 +126,22 @@ int cm_mp_backward(const float *X, const float *Y, const float *R, const float *
                    float *gX, float *gY, float *gR, float *edge_scratch, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Invariant message passing with one radial weight per component instead of one per degree:
+ *   out[n, m, c] = sum_{e -> n} X[sender[e], c] * Y[m, e] * R[e, m, c],     R [nedges, 16, channels]
+ * The reference's kernels index the weight of component m as radial[edge * 4 * C + floor(sqrt(m)) * C + c]
+ * (cuda/src/invariant_message_passing_impl.cu:138, :246-262, :365-371); these two entry points are cm_mp_forward /
+ * cm_mp_backward for callers that hold a weight per component (gR is then [nedges, 16, channels]); every other
+ * operand, the NULL conventions and the sender-sorted view are the same.
+ */
+int cm_mp_forward_per_m(const float *X, const float *Y, const float *R, const int32_t *sender,
+                        const int32_t *first_occ, int64_t nnodes, int64_t nedges, int channels, float *out,
+                        cm_stream_t stream);
+int cm_mp_backward_per_m(const float *X, const float *Y, const float *R, const float *grad_out, const int32_t *sender,
+                         const int32_t *first_occ, const int32_t *sender_perm, const int32_t *sender_offsets,
+                         int64_t nnodes, int64_t nedges, int channels, float *gX, float *gY, float *gR,
+                         float *edge_scratch, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Message passing with the radial weights evaluated in-kernel from the cubic-spline table:
  *   out[n, m, c] = sum_{e -> n} X[sender[e], c] * Y[m, e] * R(r[e])[l(m) * channels + c]
  * with R(r) exactly what cm_spline_forward computes (coeffs [nknots - 1, 4, 4 * channels], zero beyond

@@ -57,7 +57,8 @@ def stable_key_sort(keys: torch.Tensor, nkeys: int):
 def mp_forward(X, Y, R, sender, receiver, nnodes: int):
     """out[n, m, c] = sum_{e: receiver[e] = n} X[sender[e], c] * Y[m, e] * R[e, l(m), c].
 
-    X [N, C], Y [16, E], R [E, 4, C] -> [N, 16, C].  Definition of the op computed by
+    X [N, C], Y [16, E], R [E, 4, C] -> [N, 16, C] (R [E, 16, C]: one weight per component m instead of per degree
+    l(m), a variant the reference does not have).  Definition of the op computed by
     cuda/src/invariant_message_passing_impl.cu:74-165 (no normalisation factor, Y laid out
     [16, E], one radial weight per l shared by its 2l+1 components), as the reference's own
     test builds it from a per-edge tensor product followed by a scatter-sum
@@ -65,7 +66,8 @@ def mp_forward(X, Y, R, sender, receiver, nnodes: int):
     """
     s = sender.long()
     r = receiver.long()
-    msg = X[s][:, None, :] * Y.t()[:, :, None] * R[:, L_OF_M, :]  # [E, 16, C]
+    Rm = R if R.shape[1] == 16 else R[:, L_OF_M, :]  # a weight per component, or the reference's weight per degree
+    msg = X[s][:, None, :] * Y.t()[:, :, None] * Rm  # [E, 16, C]
     out = torch.zeros(nnodes, 16, X.shape[1], dtype=X.dtype)
     out.index_add_(0, r, msg)
     return out
@@ -87,6 +89,11 @@ def mp_backward(X, Y, R, grad_out, sender, receiver):
     g = grad_out[r]  # [E, 16, C]
     Yt = Y.t()  # [E, 16]
     Xs = X[s]  # [E, C]
+    if R.shape[1] == 16:  # a weight per component: no sum over the components of a degree
+        yg = g * Yt[:, :, None]
+        gX = torch.zeros_like(X)
+        gX.index_add_(0, s, (R * yg).sum(1))
+        return gX, (g * R * Xs[:, None, :]).sum(-1).t().contiguous(), Xs[:, None, :] * yg
     q = torch.zeros(R.shape, dtype=X.dtype)  # [E, 4, C]: sum_{m in l} Y g
     q.index_add_(1, L_OF_M, g * Yt[:, :, None])
     gR = Xs[:, None, :] * q

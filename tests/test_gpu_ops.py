@@ -143,6 +143,39 @@ def test_mp_backward(cabi, case):
     close(gX, gX_ref, RTOL, ATOL)
 
 
+PER_M_CASES = [(64, 8, 32, "poisson", 0.2, 0), (300, 52, 128, "poisson", 0.05, 3), (40, 150, 128, "poisson", 0.0, 4),
+               (100, 20, 160, "poisson", 0.1, 5), (150, 40, 192, "poisson", 0.0, 6), (60, 10, 224, "poisson", 0.0, 7),
+               (80, 25, 256, "poisson", 0.3, 8), (4096, 30, 96, "fixed", 0.0, 0)]
+
+
+@pytest.mark.parametrize("case", PER_M_CASES, ids=lambda c: "N%d_d%d_C%d_%s_s%d" % (c[0], c[1], c[2], c[3], c[5]))
+def test_mp_per_component_weights(cabi, case):
+    """Message passing with radial weights per component, R [E, 16, C] (the literal shape of benchmark configuration 2:
+    4096 nodes x 30 edges, 96 channels, weights edges x 16 x 96): forward and the three gradients against the oracle,
+    and equality with the per-degree op when the weights of a degree's components coincide."""
+    _say("mp per component", case)
+    nnodes, C = case[0], case[2]
+    snd, rcv, X, Y, R4, G = _mp_case(*case)
+    E = snd.numel()
+    R = torch.randn(E, 16, C, generator=torch.Generator().manual_seed(case[5] + 100), dtype=torch.float64)
+    d = lambda t: t.float().to(DEV)
+    fo = cabi.first_occurences(rcv.to(DEV), nnodes)
+    perm, off = cabi.stable_key_sort(snd.to(DEV), nnodes)
+    out = cabi.mp_forward(d(X), d(Y), d(R), snd.to(DEV), fo, nnodes)
+    close(out, O.mp_forward(X, Y, R, snd, rcv, nnodes), RTOL, ATOL)
+    gX, gY, gR = cabi.mp_backward(d(X), d(Y), d(R), d(G), snd.to(DEV), fo, perm, off, nnodes)
+    gX_ref, gY_ref, gR_ref = O.mp_backward(X, Y, R, G, snd, rcv)
+    assert gR.shape == (E, 16, C)
+    close(gR, gR_ref, RTOL, ATOL)
+    close(gY, gY_ref, RTOL, ATOL)
+    close(gX, gX_ref, RTOL, ATOL)
+    only_y = cabi.mp_backward(d(X), d(Y), d(R), d(G), snd.to(DEV), fo, None, None, nnodes, need_gX=False, need_gR=False)
+    assert only_y[0] is None and only_y[2] is None and torch.equal(only_y[1], gY)
+    expanded = d(R4)[:, O.L_OF_M.to(DEV), :].contiguous()
+    same = cabi.mp_forward(d(X), d(Y), expanded, snd.to(DEV), fo, nnodes)
+    close(same, cabi.mp_forward(d(X), d(Y), d(R4), snd.to(DEV), fo, nnodes).double().cpu(), 1e-6, 1e-6)
+
+
 def test_mp_backward_subsets(cabi):
     """Only the requested gradients are produced; each equals the full computation."""
     case = (120, 20, 128, "poisson", 0.1, 21)

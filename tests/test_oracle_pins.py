@@ -78,6 +78,34 @@ def test_mp_backward_is_autograd_of_forward():
     torch.testing.assert_close(gR, Ra.grad)
 
 
+def test_mp_per_component_weights_brute_force_and_autograd():
+    """The variant with one radial weight per component, R [E, 16, C]: python loops for the forward, autograd of the
+    forward for the three gradients; with R[e, m] = R4[e, l(m)] it reduces to the reference's op."""
+    N, C = 5, 3
+    sender = torch.tensor([1, 1, 4, 0, 2, 2], dtype=torch.int32)
+    receiver = torch.tensor([0, 0, 0, 2, 3, 3], dtype=torch.int32)
+    g = torch.Generator().manual_seed(5)
+    X = torch.randn(N, C, generator=g, dtype=torch.float64)
+    Y = torch.randn(16, 6, generator=g, dtype=torch.float64)
+    R = torch.randn(6, 16, C, generator=g, dtype=torch.float64)
+    G = torch.randn(N, 16, C, generator=g, dtype=torch.float64)
+    out = O.mp_forward(X, Y, R, sender, receiver, N)
+    ref = torch.zeros(N, 16, C, dtype=torch.float64)
+    for e in range(6):
+        for m in range(16):
+            for c in range(C):
+                ref[receiver[e], m, c] += X[sender[e], c] * Y[m, e] * R[e, m, c]
+    torch.testing.assert_close(out, ref)
+    Xa, Ya, Ra = (t.clone().requires_grad_(True) for t in (X, Y, R))
+    (O.mp_forward(Xa, Ya, Ra, sender, receiver, N) * G).sum().backward()
+    gX, gY, gR = O.mp_backward(X, Y, R, G, sender, receiver)
+    torch.testing.assert_close(gX, Xa.grad)
+    torch.testing.assert_close(gY, Ya.grad)
+    torch.testing.assert_close(gR, Ra.grad)
+    R4 = torch.randn(6, 4, C, generator=g, dtype=torch.float64)
+    torch.testing.assert_close(O.mp_forward(X, Y, R4[:, O.L_OF_M, :], sender, receiver, N), O.mp_forward(X, Y, R4, sender, receiver, N))
+
+
 # ---- spherical harmonics -------------------------------------------------------------------------------
 def test_sh_against_scipy_closed_form():
     """sqrt(4 pi) x real harmonics built from scipy's complex ones, without Condon-Shortley sign:
