@@ -44,15 +44,24 @@ def kernel_sources_digest():
 def measured_traffic():
     """HBM bytes per launch at the default workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs (calibrated against a
     copy of known size), as recorded with the profile summaries together with the digest of the kernel sources they were
-    measured on.  Returns {} when the sources have changed since: a stale figure is not reported."""
+    measured on: {"in_step": {kernel: bytes}, "standalone": {kernel: bytes}} (inside the model step, where atoms are
+    relabelled by spatial bin, and for the stand-alone ops on the box's random atom order).  Both are empty when the
+    sources have changed since: a stale figure is not reported."""
+    empty = {"in_step": {}, "standalone": {}}
     try:
         with open(TRAFFIC_FILE) as f:
             rec = json.load(f)
     except (OSError, ValueError):
-        return {}
+        return empty
     if rec.get("kernel_sources_sha256") != kernel_sources_digest():
-        return {}
-    return {k: int(v) for k, v in rec.get("bytes_per_launch", {}).items()}
+        return empty
+    return {k: {n: int(v) for n, v in rec.get(k, {}).items()} for k in empty}
+
+
+def traffic_of(table, kernels):
+    """Sum over the kernels of an op ("a + b" names two); None when one of them was not measured."""
+    parts = [table.get(k.strip()) for k in kernels.split("+")]
+    return None if any(p is None for p in parts) else sum(parts)
 
 
 def linear_kernel_name(C):
@@ -114,7 +123,7 @@ def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=
         ("mp_backward gY,gR (tabulated R)", "mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b,
          lambda: cabi.mp_backward(X, Y, R, G, snd, fo, None, None, N, need_gX=False)),
         ("mp_backward gX,gY,gR (tabulated R): edge pass + sender pass",
-         "mp_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,false>" % (C, C), bwd_full_b,
+         "mp_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,0>" % (C, C), bwd_full_b,
          lambda: cabi.mp_backward(X, Y, R, G, snd, fo, perm, off, N)),
     ]
     if with_per_component:
@@ -124,7 +133,7 @@ def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=
             ("mp_forward (R per component [E,16,C])", "mp_per_m_forward_kernel<%d>" % C,
              4 * (16 * E * C + 16 * E + 17 * N * C) + 8 * E, lambda: cabi.mp_forward(X, Y, R16, snd, fo, N)),
             ("mp_backward gX,gY,gR (R per component): edge pass + sender pass",
-             "mp_per_m_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,false>" % (C, C),
+             "mp_per_m_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,0>" % (C, C),
              4 * (32 * E * C + 32 * E + 18 * N * C) + 8 * E, lambda: cabi.mp_backward(X, Y, R16, G, snd, fo, perm, off, N)),
         ]
     if with_fused:
@@ -152,13 +161,13 @@ def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=
         eperm, eoff = cabi.stable_key_sort(types, ne)
         m3d, m2d = t(m3), t(m2)
         cases += [
-            ("spherical harmonics forward", "sh_forward_kernel", 76 * E, lambda: cabi.sh_forward(vec)),
-            ("spherical harmonics backward", "sh_backward_kernel", 88 * E, lambda: cabi.sh_backward(vec, gY)),
-            ("spline forward (R only)", "spline_forward_kernel", 4 * (E + 4 * E * C),
+            ("spherical harmonics forward", "sh_forward_kernel<float>", 76 * E, lambda: cabi.sh_forward(vec)),
+            ("spherical harmonics backward", "sh_backward_kernel<float>", 88 * E, lambda: cabi.sh_backward(vec, gY)),
+            ("spline forward (R only)", "spline_forward_kernel<false>", 4 * (E + 4 * E * C),
              lambda: cabi.spline_forward(r, knots, coeffs, float(h), 5.0)),
             ("spline backward", "spline_backward_kernel", 4 * (4 * E * C + 2 * E),
              lambda: cabi.spline_backward(r, knots, coeffs, R.view(E, 4 * C), float(h), 5.0)),
-            ("symmetric contraction forward + gradient", "symcon_lmax3_kernel", 4 * (33 * N * C + N),
+            ("symmetric contraction forward + gradient", "symcon_lmax3_kernel<float,true>", 4 * (33 * N * C + N),
              lambda: cabi.symcon_forward(G, eperm, eoff, m3d, m2d, T3, T2, T1, builtin=True)),
             ("symmetric contraction backward", "symcon_backward_kernel", 4 * 33 * N * C, lambda: cabi.symcon_backward(G, gN)),
             # channel-mixing linear [N,16,C] x [C,C] per l: reads X and the four weight blocks, writes OUT
@@ -410,7 +419,7 @@ def main():
         gbps = nbytes / (ms * 1e-3) / 1e9
         d = {"kernel": kernel, "bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
              "frac": round(gbps / HBM_PEAK_GBPS, 4),
-             "traffic": traffic.get(kernel) if default_workload else None,
+             "traffic": traffic_of(traffic["in_step"], kernel) if default_workload else None,
              "algorithmic_bytes_per_launch": nbytes, "avg_launch_ms": round(ms, 4)}
         d.update(extra)
         return d
@@ -448,7 +457,7 @@ def main():
             tf = flops / (t_lin * 1e-3) / 1e12
             others.append({"kernel": linear_kernel_name(C), "bound": "mfma", "achieved": round(tf, 1),
                            "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
-                           "traffic": traffic.get(linear_kernel_name(C)) if default_workload else None,
+                           "traffic": traffic_of(traffic["standalone"], linear_kernel_name(C)) if default_workload else None,
                            "algorithmic_flops_per_launch": flops, "avg_launch_ms": round(t_lin, 4),
                            "launches_timed": launches("linear"),
                            "note": "fp32-equivalent flops of the [N,16,C] x [C,C] channel mixing against the fp32 matrix "
@@ -469,7 +478,7 @@ def main():
         snd32 = data["edge_index"][1].int().contiguous()
         standalone, config2 = standalone_rooflines(torch, cabi, N, E, C, ne, rcv32, snd32)
         for row in standalone:
-            row["traffic"] = traffic.get(row["kernel"]) if default_workload and row["shape"].startswith("N=") else None
+            row["traffic"] = traffic_of(traffic["standalone"], row["kernel"]) if default_workload else None
         others += standalone
 
     # the step before the path: neighbour list rebuilt on the device (excluded from the timed steps, as the reference's

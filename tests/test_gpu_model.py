@@ -312,7 +312,7 @@ def test_model_in_a_foreign_coupling_basis(cabi):
     assert abs(float(ref_own["interaction_energy"]) - float(ref["interaction_energy"])) > 1e-3 * abs(float(ref["interaction_energy"]))
 
 
-@pytest.mark.parametrize("case", ["cluster", "periodic96", "periodic192", "batch_relabelled", "isolated_atoms"])
+@pytest.mark.parametrize("case", ["cluster", "periodic96", "periodic192", "batch_relabelled", "isolated_atoms", "single_atom"])
 def test_native_step_equals_autograd_path(cabi, case):
     """The step enqueued by the library in one call (cm_mace_step) against the same kernels driven from Python through
     autograd: identical node energies and features (same kernels in the same order), energies equal up to the order of
@@ -332,6 +332,9 @@ def test_native_step_equals_autograd_path(cabi, case):
     elif case == "batch_relabelled":
         data = collate([make_system(n, 4, seed=30 + k, density=0.1) for k, n in enumerate((150, 230, 120))])
         C, numbers, kwargs = 64, (1, 6, 7, 8), dict(spatial_order_min_atoms=0)
+    elif case == "single_atom":  # no edge at all: the energy is E0 + shift, the force zero
+        data, C, numbers = make_system(1, 4, seed=2, density=None, cluster_box=4.0), 32, (1, 6, 7, 8)
+        assert data["edge_index"].shape[1] == 0
     else:  # a sparse cluster: most atoms have no neighbour at all
         data, C, numbers = make_system(12, 4, seed=2, density=None, cluster_box=40.0, min_dist=3.0), 32, (1, 6, 7, 8)
     N = data["positions"].shape[0]
