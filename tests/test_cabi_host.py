@@ -121,3 +121,23 @@ def test_build_refuses_scratch_in_hand_scheduled_kernels():
         build._check_no_scratch("linear.hip", ok.replace("VGPRs Spill: 0", "VGPRs Spill: 24"))
     with pytest.raises(RuntimeError, match="no resource-usage remark"):
         build._check_no_scratch("mp.hip", ok)
+
+
+def test_header_is_valid_c_and_cpp(tmp_path):
+    """The boundary is a C ABI: the header must compile as plain C (what cgo, a Fortran binding generator or LAMMPS'
+    C glue would include) and as C++, on its own."""
+    import shutil
+    import subprocess
+
+    import pytest
+
+    for compiler, lang, std in (("gcc", "c", "-std=c99"), ("g++", "c++", "-std=c++11")):
+        exe = shutil.which(compiler)
+        if exe is None:
+            pytest.skip("no " + compiler)
+        src = tmp_path / ("use_header." + ("c" if lang == "c" else "cpp"))
+        src.write_text('#include "cuda_mace_hip.h"\nint main(void) { cm_mace_weights w; cm_mace_graph g; (void)w; (void)g; '
+                       'return (int)sizeof(cm_stream_t) == 0; }\n')
+        res = subprocess.run([exe, std, "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I" + os.path.join(ROOT, "include"),
+                              str(src)], capture_output=True, text=True, timeout=120)
+        assert res.returncode == 0, res.stderr
