@@ -295,7 +295,7 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
     const float *__restrict__ gXe, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ offsets, int nnodes, int64_t nedges, const float *__restrict__ live_by, float r_max,
     float *__restrict__ gX) {
-  using K = Cfg<C>;
+  using K = Cfg<C, false, true>;  // a pure row stream: 16 bytes per lane at every channel count
   using vec = typename K::vec;
   constexpr int B = 4;            // edges per slot and iteration
   constexpr int STEP = B * K::EPW;

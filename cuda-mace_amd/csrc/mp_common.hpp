@@ -14,12 +14,14 @@ constexpr int pow2ceil(int v) {
   return p;
 }
 
-template <int C, bool STRIDED = false>
+template <int C, bool STRIDED = false, bool WIDE = false>
 struct Cfg {
   // channels per lane: four (one 16-byte access per row), except where three fill the lanes exactly (96 -> 32 lanes,
   // 192 -> 64 lanes) and four would leave a quarter of them idle; kernels that own strided channels (see below) also
   // run 160 and 224 channels on 32 full lanes, five and seven channels each
-  static constexpr int V = (C == 96 || C == 192) ? 3 : (STRIDED && C == 160) ? 5 : (STRIDED && C == 224) ? 7 : 4;
+  // WIDE: always four (one 16-byte access per lane and row, some lanes idle at 96 and 192 channels): for kernels that
+  // only stream rows, where three dword accesses per row cost the vector-memory path three times the line look-ups
+  static constexpr int V = WIDE ? 4 : (C == 96 || C == 192) ? 3 : (STRIDED && C == 160) ? 5 : (STRIDED && C == 224) ? 7 : 4;
   static constexpr int LPE = C / V;          // lanes that carry one edge
   static constexpr int SW = pow2ceil(LPE);   // slot width in lanes (power of two)
   static constexpr int EPW = kWave / SW;     // edges in flight per wave
