@@ -510,6 +510,346 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
   }
 }
 
+// -----------------------------------------------------------------------------------------------
+// Variant with the weights resident in LDS (16 components per node, K = Nout up to 128).
+//
+// The kernels above stage the K x Nout weight block again for every tile of 128 rows (as many bytes from L2 as the tile
+// has from HBM) and walk K in barrier-separated phases.  Here a launch has one workgroup per compute unit, and a
+// workgroup takes a contiguous piece of the list of all 32-row tiles, ordered by (weight group, l, node tile, m within
+// l), so that it needs one or two weight blocks in its whole life: it splits a block once into three bf16 planes that
+// cover all of K (102 KB at 128 x 128) and then its four waves run independently of each other, one 32-row tile at a
+// time, with no barrier until the weight block changes.
+//
+// What a wave has in flight lives in registers, not in LDS: the loads of tile i + 1 (16 x 16 bytes per lane at 128
+// columns, whole 128-byte lines of 8 rows per instruction) are issued before tile i is multiplied and land in
+// accumulator-file registers; 64 KB per compute unit are on their way at any time.  When its turn comes a tile changes
+// from that row-major layout to the operand layout of the matrix instruction (a lane holds 8 values of one row per
+// 16-wide k step) through the wave's own corner of LDS, 64 columns at a time.  The order of k inside a step is free as
+// long as both operands agree; it is chosen such that a lane reads two aligned 16-byte pieces.  The operands are swapped
+// with respect to the kernels above (weights as the row operand, X rows as the column operand): a lane's accumulators
+// are then 4 consecutive output columns of one row; a block of 32 columns goes back through the same corner of LDS and
+// leaves as whole lines.  The piece products and their order are those of the kernels above.
+//
+// Contract of the hand-issued memory operations of the tile loop (the loads and the stores): a load names its landing
+// registers at issue time although the data arrives by the explicit wait that precedes their first use, which is
+// sound only while the compiler neither copies nor spills them in between; they are accumulator-file registers,
+// which nothing else in the kernel wants, and the build refuses scratch memory in this kernel.  A store is followed
+// by the two idle issue slots that the hardware needs before the stored registers may be overwritten (the compiler
+// inserts them for the stores it knows; without them the last lanes of the following block were stored instead).
+// -----------------------------------------------------------------------------------------------
+constexpr int kResWaves = 4;
+constexpr int kResMaxGroups = 128;
+constexpr int kResMinNodes = 2048;
+constexpr int kOutLd = 36;            // floats per row of a wave's output staging block (32 columns + 16 bytes)
+constexpr int kResSegNodeTiles = 64;  // node tiles whose row numbers a segment keeps in LDS
+
+template <int K, int NT, bool SCALED>
+__global__ __launch_bounds__(kResWaves *kWave, 1) void linear_resident_kernel(
+    const float *__restrict__ X, const float *__restrict__ WT, const int32_t *__restrict__ node_perm,
+    const int32_t *__restrict__ group_offsets, int nnodes, int ngroups, int zero_last_group, int ldo, float scale,
+    const float *__restrict__ row_scale, float *__restrict__ OUT) {
+  constexpr int NOUT = 32 * NT;  // columns of this workgroup: blockIdx.y * NOUT onwards of the ldo columns of OUT
+  constexpr int LD = K + 8;      // row stride of a plane in elements: an odd number of 16-byte units
+  constexpr int KS = K / 16;
+  __shared__ __attribute__((aligned(16))) __bf16 sW[3 * NOUT * LD];
+  __shared__ int sId[kResSegNodeTiles * 32];
+  constexpr int kChunk = K <= 96 ? K : 64;  // columns of X per trip through LDS
+  constexpr int kTLd = kChunk + 4;          // floats per row of the transposition block: an odd number of 16-byte units
+  constexpr int kStageFloats = 32 * (kTLd > kOutLd ? kTLd : kOutLd);  // a wave's own corner of LDS
+  __shared__ __attribute__((aligned(16))) float sStage[kResWaves * kStageFloats];
+  __shared__ int sOff[kResMaxGroups + 1];
+  __shared__ int sCum[kResMaxGroups + 1];
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int mrow = lane % 32;
+  const int half = lane / 32;
+  const int c0 = blockIdx.y * NOUT;
+
+  // groups that have weights, their row ranges in the grouped node order and their first tile in the tile list
+  const int ngw = zero_last_group ? ngroups - 1 : ngroups;
+  if (tid == 0) {
+    int cum = 0;
+    for (int g = 0; g < ngw; ++g) {
+      const int lo = group_offsets ? group_offsets[g] : 0, hi = group_offsets ? group_offsets[g + 1] : nnodes;
+      sOff[g] = lo;
+      sCum[g] = cum;
+      cum += 16 * ((max(hi - lo, 0) + 31) / 32);
+    }
+    sOff[ngw] = group_offsets ? group_offsets[ngw] : nnodes;
+    sCum[ngw] = cum;
+  }
+  if (zero_last_group && blockIdx.y == 0) {
+    // rows that belong to no weight group: defined as zero
+    const int z0 = group_offsets[ngroups - 1], nz = group_offsets[ngroups] - z0;
+    const int rowq = 16 * ldo / 4;
+    const int64_t total = static_cast<int64_t>(nz) * rowq;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + tid; i < total; i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+      const int node = node_perm[z0 + static_cast<int>(i / rowq)];
+      if (static_cast<unsigned>(node) < static_cast<unsigned>(nnodes)) st4(OUT + static_cast<int64_t>(node) * 16 * ldo + 4 * (i % rowq), zero4());
+    }
+  }
+  __syncthreads();
+
+  const int ntiles = sCum[ngw];
+  const int i1 = static_cast<int>(static_cast<int64_t>(ntiles) * (blockIdx.x + 1) / gridDim.x);
+  int i = static_cast<int>(static_cast<int64_t>(ntiles) * blockIdx.x / gridDim.x);
+  int g = 0, staged_g = -1, staged_l = -1;
+
+  while (i < i1) {
+    while (sCum[g + 1] <= i) ++g;
+    const int tg = (sCum[g + 1] - sCum[g]) / 16;  // node tiles of the group
+    const int l = l_of_m((i - sCum[g]) / tg);
+    const int nm = 2 * l + 1;
+    const int blk0 = sCum[g] + tg * l * l;        // first tile of (g, l): tile blk0 + t * nm + (m - l * l)
+    const int t_first = (i - blk0) / nm;
+    const int seg_end = min(min(i1, blk0 + tg * nm), blk0 + (t_first + kResSegNodeTiles) * nm);
+    const int t_count = (seg_end - 1 - blk0) / nm - t_first + 1;
+    const int off0 = sOff[g], off1 = sOff[g + 1];
+
+    __syncthreads();  // every wave is done with the previous segment
+    // Row numbers of the segment's node tiles.  A row beyond the end of the group (or an index outside the node range)
+    // stands in for the first row of its tile: it then computes that row's values once more and stores the same bits
+    // to the same place, so that no load or store of the tile loop is conditional.
+    for (int r = tid; r < 32 * t_count; r += kResWaves * kWave) {
+      const int p0 = off0 + 32 * (t_first + r / 32);
+      const int p = p0 + r % 32;
+      int node = node_perm ? node_perm[p < off1 ? p : p0] : (p < off1 ? p : p0);
+      if (static_cast<unsigned>(node) >= static_cast<unsigned>(nnodes)) node = node_perm ? node_perm[p0] : p0;
+      if (static_cast<unsigned>(node) >= static_cast<unsigned>(nnodes)) node = 0;
+      sId[r] = node;
+    }
+    if (g != staged_g || l != staged_l) {
+      // W^T[c0 + j, :] of block (g, l) -> three planes; inside every 16 k the two middle groups of four trade places, so
+      // that the 8 values a lane reads at 16 s + 8 half are k = 16 s + 4 half + {0..3, 8..11}
+      const float *Wg = WT + ((static_cast<int64_t>(g) * 4 + l) * ldo + c0) * K;
+      // all loads of a thread first (16 at 128 x 128), then the splits: one trip through L2 instead of one per piece
+      constexpr int kPieces = NOUT * (K / 4) / (kResWaves * kWave);
+      static_assert(NOUT * (K / 4) % (kResWaves * kWave) == 0, "weight staging map");
+      f4 wv[kPieces];
+#pragma unroll
+      for (int it = 0; it < kPieces; ++it) {
+        const int q = it * (kResWaves * kWave) + tid;
+        wv[it] = ld4(Wg + static_cast<int64_t>(q / (K / 4)) * K + 4 * (q % (K / 4)));
+      }
+#pragma unroll
+      for (int it = 0; it < kPieces; ++it) {
+        const int q = it * (kResWaves * kWave) + tid;
+        const int j = q / (K / 4), kq = q % (K / 4);
+        bf16x4 h, md, lw;
+        split3(wv[it], h, md, lw);
+        const int sub = kq & 3;
+        const int at = j * LD + 16 * (kq >> 2) + 4 * (sub == 1 ? 2 : (sub == 2 ? 1 : sub));
+        *reinterpret_cast<bf16x4 *>(sW + at) = h;
+        *reinterpret_cast<bf16x4 *>(sW + NOUT * LD + at) = md;
+        *reinterpret_cast<bf16x4 *>(sW + 2 * NOUT * LD + at) = lw;
+      }
+      staged_g = g;
+      staged_l = l;
+    }
+    __syncthreads();
+
+    // this wave's contiguous share of the segment
+    const int per = (seg_end - i + kResWaves - 1) / kResWaves;
+    const int wb = i + wave * per, we = min(seg_end, wb + per);
+    i = seg_end;
+    if (wb >= we) continue;
+
+    // Tile loop.  Every global access in it is issued from assembly in a fixed order and waited for by an explicit count
+    // (the compiler would sink part of a prefetch down to its use and then wait for everything that is in flight, the
+    // stores of the previous tile included):
+    //     tile i:  wait: all but the stores of tile i - 1 | landing registers -> working registers (times row_scale)
+    //              | issue the loads of tile i + 1 | multiply | output block by block through LDS, issue the stores
+    // The landing registers are accumulator-file registers (a load may write them directly; nothing else competes for
+    // them, so the compiler has no reason to move them while a load is in flight), the working set lives in ordinary
+    // registers.
+    // Loads are whole lines: one instruction fetches 128 bytes of each of 8 rows (lane = 16-byte piece opiece of row
+    // 8 rg + orow; in 32-byte pieces, which is what a lane feeds per k step, every line would be requested four times and
+    // the compute unit's queue of outstanding misses would hold a quarter of the bytes).  The landed values change to the
+    // operand layout through the wave's own corner of LDS, kChunk columns at a time.
+    constexpr int kLines = kChunk / 32;  // 128-byte lines of a row per chunk
+    constexpr int kChunks = K / kChunk;
+    static_assert(K % kChunk == 0 && kChunk % 32 == 0, "chunks of whole lines");
+    f4 land[2 * KS];                           // index (chunk * 4 + rg) * kLines + line
+    f4 sland[SCALED ? 2 * KS : 1];
+    float *stg = sStage + wave * kStageFloats;
+    const int orow = lane / 8, opiece = lane % 8;
+    auto issue = [&](int idx, int &m_of, int &tb_of) {
+      const int j = idx - blk0;
+      const int t = j / nm;
+      m_of = l * l + (j - t * nm);
+      tb_of = 32 * (t - t_first);
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int nd = sId[tb_of + 8 * rg + orow];
+        const float *xp = X + (static_cast<int64_t>(nd) * 16 + m_of) * K + 4 * opiece;
+#pragma unroll
+        for (int c = 0; c < kChunks; ++c)
+#pragma unroll
+          for (int ln = 0; ln < kLines; ++ln)
+            asm volatile("global_load_dwordx4 %0, %1, off offset:%2 nt" : "=a"(land[(c * 4 + rg) * kLines + ln]) : "v"(xp), "n"(4 * (c * kChunk + 32 * ln)) : "memory");
+        if constexpr (SCALED) {
+          const float *sp = row_scale + static_cast<int64_t>(nd) * K + 4 * opiece;
+#pragma unroll
+          for (int c = 0; c < kChunks; ++c)
+#pragma unroll
+            for (int ln = 0; ln < kLines; ++ln)
+              asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=a"(sland[(c * 4 + rg) * kLines + ln]) : "v"(sp), "n"(4 * (c * kChunk + 32 * ln)) : "memory");
+        }
+      }
+    };
+    const __bf16 *wl = sW + mrow * LD + 8 * half;
+    int m_next, tb_next;
+    issue(wb, m_next, tb_next);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (int idx = wb; idx < we; ++idx) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * NT) : "memory");
+      const int m_cur = m_next, tb_cur = tb_next;
+      f4 cur[2 * KS];
+#pragma unroll
+      for (int c = 0; c < kChunks; ++c) {
+        wave_lds_fence();
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg)
+#pragma unroll
+          for (int ln = 0; ln < kLines; ++ln) {
+            const int j = (c * 4 + rg) * kLines + ln;
+            asm volatile("" : "+a"(land[j]));
+            f4 v = land[j];
+            if constexpr (SCALED) {
+              asm volatile("" : "+a"(sland[j]));
+              v *= sland[j];
+            }
+            *reinterpret_cast<f4 *>(stg + (8 * rg + orow) * kTLd + 32 * ln + 4 * opiece) = v;
+          }
+        wave_lds_fence();
+        // k step s of the chunk: the lane's values are columns 16 s + 4 half + {0..3} and 16 s + 8 + 4 half + {0..3}
+#pragma unroll
+        for (int sc = 0; sc < kChunk / 16; ++sc) {
+          const int s = c * (kChunk / 16) + sc;
+          cur[2 * s] = *reinterpret_cast<const f4 *>(stg + mrow * kTLd + 16 * sc + 4 * half);
+          cur[2 * s + 1] = *reinterpret_cast<const f4 *>(stg + mrow * kTLd + 16 * sc + 8 + 4 * half);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 2 * KS; ++j) asm volatile("" : "+v"(cur[j]));
+      if (idx + 1 < we) issue(idx + 1, m_next, tb_next);
+
+      v16f acc[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+      // One wave per SIMD: nothing but this wave's own instruction stream can fill the issue slots between two matrix
+      // instructions (32 cycles apart), so the k loop is pipelined in the source: the pieces of X and the weight fragments of
+      // step s + 1 are prepared while the 6 NT matrix instructions of step s run, and the scheduler is told to weave them
+      // (per matrix instruction: three vector instructions, and an LDS read for the first 3 NT of them).
+      constexpr int kSplitOps = (64 + 6 * NT - 1) / (6 * NT);  // the split of a step is about 60 vector instructions
+      bf16x8 xq[2][3], wq[2][NT][3];
+      auto prepare = [&](int s, auto par) {
+        constexpr int P = decltype(par)::value;
+        bf16x4 h0, m0, l0, h1, m1, l1;
+        split3(cur[2 * s], h0, m0, l0);
+        split3(cur[2 * s + 1], h1, m1, l1);
+        xq[P][0] = __builtin_shufflevector(h0, h1, 0, 1, 2, 3, 4, 5, 6, 7);
+        xq[P][1] = __builtin_shufflevector(m0, m1, 0, 1, 2, 3, 4, 5, 6, 7);
+        xq[P][2] = __builtin_shufflevector(l0, l1, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int p = 0; p < 3; ++p) wq[P][t][p] = *reinterpret_cast<const bf16x8 *>(wl + p * NOUT * LD + 32 * t * LD + 16 * s);
+      };
+      auto step = [&](int s, auto par) {
+        constexpr int P = decltype(par)::value;
+        if (s + 1 < KS) prepare(s + 1, std::integral_constant<int, 1 - P>{});
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wq[P][t][0], xq[P][2], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wq[P][t][2], xq[P][0], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wq[P][t][1], xq[P][1], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wq[P][t][0], xq[P][1], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wq[P][t][1], xq[P][0], acc[t], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wq[P][t][0], xq[P][0], acc[t], 0, 0, 0);
+        if (s + 1 < KS) {
+#pragma unroll
+          for (int i = 0; i < 6 * NT; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one matrix instruction
+            if (i < 3 * NT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+            __builtin_amdgcn_sched_group_barrier(0x002, kSplitOps, 0);          // a share of the split arithmetic
+          }
+        }
+        // nothing else moves across k steps: fragment reads of later steps hoisted further would not fit the register file
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      prepare(0, std::integral_constant<int, 0>{});
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < KS; s += 2) {
+        step(s, std::integral_constant<int, 0>{});
+        if (s + 1 < KS) step(s + 1, std::integral_constant<int, 1>{});
+      }
+      // accumulator r of a lane: output column 32 t + 8 (r / 4) + 4 half + r % 4 of row mrow of the tile.  Stored from
+      // here a row would leave in 32-byte pieces; a block of 32 columns goes through the wave's own corner of LDS instead
+      // (rows padded to 9 x 16 bytes: conflict-free both ways) and leaves as whole 128-byte lines, 8 rows per store.
+      float *orows[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        orows[r] = OUT + (static_cast<int64_t>(sId[tb_cur + 8 * r + orow]) * 16 + m_cur) * ldo + c0 + 4 * opiece;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        wave_lds_fence();
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *reinterpret_cast<f4 *>(stg + mrow * kOutLd + 8 * q + 4 * half) = f4{acc[t][4 * q], acc[t][4 * q + 1], acc[t][4 * q + 2], acc[t][4 * q + 3]} * scale;
+        wave_lds_fence();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const f4 v = *reinterpret_cast<const f4 *>(stg + (8 * r + orow) * kOutLd + 4 * opiece);
+          // the two idle issue slots are what the compiler puts between a 16-byte store and an instruction that
+          // overwrites the registers it stores from; it does not see this store
+          asm volatile("global_store_dwordx4 %0, %1, off offset:%2\n\ts_nop 1" : : "v"(orows[r]), "v"(v), "n"(128 * t) : "memory");
+        }
+      }
+    }
+    // every landing register has been consumed: nothing this wave issued can still write a register
+  }
+}
+
+int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+template <int K, int NT>
+int launch_resident(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
+                    int zero_last_group, int Nout, float scale, const float *row_scale, float *OUT, hipStream_t st) {
+  // one workgroup per compute unit.  (The kernel can also split the columns over grid.y, 32 NT per workgroup: the
+  // workgroups that share X rows are then a multiple of 8 apart in launch order, i.e. on one XCD and its L2.  Measured at
+  // 192 = 2 x 96 and 256 = 4 x 64 columns it only equals the kernels above, because every column block splits the X rows
+  // again, so those widths are not routed here.)
+  const int ycount = Nout / (32 * NT);
+  const dim3 grid(static_cast<unsigned>(std::max(8, compute_units() / ycount / 8 * 8)), static_cast<unsigned>(ycount)), block(kResWaves * kWave);
+  if (row_scale)
+    hipLaunchKernelGGL((linear_resident_kernel<K, NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                       zero_last_group, Nout, scale, row_scale, OUT);
+  else
+    hipLaunchKernelGGL((linear_resident_kernel<K, NT, false>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                       zero_last_group, Nout, scale, row_scale, OUT);
+  return check_launch("cm_linear");
+}
+
 template <int NT>
 int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
            int zero_last_group, int ncomp, int K, float scale, const float *row_scale, const float *residual, float *OUT,
@@ -565,6 +905,17 @@ extern "C" int cm_linear(const float *X, const float *W_T, const int32_t *node_p
   if (nnodes == 0) return CM_OK;
   CM_REQUIRE(X && W_T && OUT, "cm_linear: NULL pointer");
   hipStream_t st = cm::as_stream(stream);
+  // 16 components per node, square weights up to 128 and enough rows to give every compute unit a few tiles: the
+  // kernel that keeps the weights in LDS (measured against the ring kernel at 25 000 nodes: 87 vs 102-112 us at 128
+  // channels, 58 vs 67-71 at 96, 42 vs 47 at 64; 360 vs 430 us at 100 000 x 128; equal at 2 500 nodes)
+  if (ncomp == 16 && K == Nout && !residual && ngroups <= cm::kResMaxGroups && nnodes >= cm::kResMinNodes) {
+    switch (K) {
+#define CM_CASE(K_, NT_) \
+      case K_: return cm::launch_resident<K_, NT_>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, Nout, scale, row_scale, OUT, st);
+      CM_CASE(64, 2) CM_CASE(96, 3) CM_CASE(128, 4)
+#undef CM_CASE
+    }
+  }
   switch (Nout / 32) {
     case 1: return cm::launch<1>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);
     case 2: return cm::launch<2>(X, W_T, node_perm, group_offsets, nnodes, ngroups, zero_last_group, ncomp, K, scale, row_scale, residual, OUT, st);

@@ -330,6 +330,51 @@ def test_scalar_elemental_linear_and_zero_group(cabi, N, K, Nout, ne, seed):
     close(out16, ref16, 1e-5, 2e-6)
 
 
+@pytest.mark.parametrize("N,C,ne,seed", [(2048, 128, 1, 0), (2500, 128, 10, 1), (4099, 96, 5, 2), (3000, 64, 3, 3), (6000, 128, 130, 4)])
+def test_linear_many_rows(cabi, N, C, ne, seed):
+    """16-component features with at least 2048 nodes and 64 / 96 / 128 square weights run on the kernel that keeps the
+    weight block in LDS (one workgroup per compute unit walking 32-row tiles); more than 128 weight groups stay on the
+    tiled kernels.  Groups of very different sizes, an empty group, a group of one node, tiles that end inside a group,
+    rows of no group, with and without row_scale; twice, for the same bits."""
+    _say("linear_many_rows", N, C, ne, seed)
+    g = torch.Generator().manual_seed(seed)
+    X = torch.randn(N, 16, C, generator=g, dtype=torch.float64).float().double()
+    S = torch.randn(N, C, generator=g, dtype=torch.float64).float().double()
+    W = torch.randn(ne, 4, C, C, generator=g, dtype=torch.float64).float().double()
+    p = torch.rand(ne + 1, generator=g, dtype=torch.float64) ** 3 + 1e-3
+    elem = torch.multinomial(p, N, replacement=True, generator=g)  # value ne = "no element"
+    if ne >= 3:
+        elem[elem == 1] = 0  # an empty group
+        elem[elem == 2] = 0
+        elem[N // 2] = 2     # a group of one node
+    Xd, Sd = X.float().to(DEV), S.float().to(DEV)
+    WT = W.transpose(-1, -2).contiguous().float().to(DEV)
+    # one weight group for all nodes
+    close(cabi.linear(Xd, WT[0]), O.linear(X, W[0]), 1e-5, 2e-6)
+    close(cabi.linear(Xd, WT[0], row_scale=Sd), O.linear(X * S[:, None, :], W[0]), 1e-5, 2e-6)
+    # per-element weights, rows of the last key are zero
+    ref = torch.zeros(N, 16, C, dtype=torch.float64)
+    ref_s = torch.zeros(N, 16, C, dtype=torch.float64)
+    for e in range(ne):
+        rows = (elem == e).nonzero()[:, 0]
+        if rows.numel():
+            ref[rows] = O.linear(X[rows], W[e])
+            ref_s[rows] = O.linear(X[rows] * S[rows][:, None, :], W[e])
+    perm, off = cabi.stable_key_sort(elem.int().to(DEV), ne + 1)
+    out = cabi.linear(Xd, WT, perm, off, zero_last_group=True)
+    close(out, ref, 1e-5, 2e-6)
+    assert float(out[(elem == ne).to(DEV)].abs().sum()) == 0.0
+    out_s = cabi.linear(Xd, WT, perm, off, zero_last_group=True, row_scale=Sd)
+    close(out_s, ref_s, 1e-5, 2e-6)
+    assert torch.equal(out, cabi.linear(Xd, WT, perm, off, zero_last_group=True))
+    # every node in a group (no zero rows): the keys of the rows of no group move to the last element
+    elem2 = torch.where(elem == ne, torch.full_like(elem, ne - 1), elem)
+    rows = (elem == ne).nonzero()[:, 0]
+    ref[rows] = O.linear(X[rows], W[ne - 1])
+    perm2, off2 = cabi.stable_key_sort(elem2.int().to(DEV), ne)
+    close(cabi.linear(Xd, WT, perm2, off2), ref, 1e-5, 2e-6)
+
+
 # ------------------------------------------------------------------------------------------------
 # symmetric contraction with synthetic sparse tables
 # ------------------------------------------------------------------------------------------------
