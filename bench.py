@@ -64,10 +64,13 @@ def traffic_of(table, kernels):
     return None if any(p is None for p in parts) else sum(parts)
 
 
-def linear_kernel_name(C):
-    """The library runs the channel-mixing linear on its LDS-ring kernel for 64, 96, 128, 224 and 256 columns and on the
-    plain one otherwise."""
+def linear_kernel_name(C, N):
+    """The library runs the [N,16,C] channel-mixing linear on its kernel with LDS-resident weights for 64, 96 and 128
+    columns when there are at least 2 048 nodes, else on the LDS-ring kernel for 64, 96, 128, 224 and 256 columns and on
+    the plain one otherwise."""
     nt = C // 32
+    if nt in (2, 3, 4) and N >= 2048:
+        return "linear_resident_kernel<%d,%d,false>" % (C, nt)
     return ("linear_ring_kernel<%d,false>" if nt in (2, 3, 4, 7, 8) else "linear_kernel<%d,false>") % nt
 
 
@@ -171,7 +174,7 @@ def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=
              lambda: cabi.symcon_forward(G, eperm, eoff, m3d, m2d, T3, T2, T1, builtin=True)),
             ("symmetric contraction backward", "symcon_backward_kernel", 4 * 33 * N * C, lambda: cabi.symcon_backward(G, gN)),
             # channel-mixing linear [N,16,C] x [C,C] per l: reads X and the four weight blocks, writes OUT
-            ("linear [N,16,C] x [C,C]", linear_kernel_name(C), 4 * (32 * N * C + 4 * C * C), lambda: cabi.linear(G, WT)),
+            ("linear [N,16,C] x [C,C]", linear_kernel_name(C, N), 4 * (32 * N * C + 4 * C * C), lambda: cabi.linear(G, WT)),
         ]
     return cases
 
@@ -455,9 +458,9 @@ def main():
         if t_lin:
             flops = 32 * N * C * C
             tf = flops / (t_lin * 1e-3) / 1e12
-            others.append({"kernel": linear_kernel_name(C), "bound": "mfma", "achieved": round(tf, 1),
+            others.append({"kernel": linear_kernel_name(C, N), "bound": "mfma", "achieved": round(tf, 1),
                            "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
-                           "traffic": traffic_of(traffic["standalone"], linear_kernel_name(C)) if default_workload else None,
+                           "traffic": traffic_of(traffic["standalone"], linear_kernel_name(C, N)) if default_workload else None,
                            "algorithmic_flops_per_launch": flops, "avg_launch_ms": round(t_lin, 4),
                            "launches_timed": launches("linear"),
                            "note": "fp32-equivalent flops of the [N,16,C] x [C,C] channel mixing against the fp32 matrix "

@@ -533,9 +533,20 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
 // Contract of the hand-issued memory operations of the tile loop (the loads and the stores): a load names its landing
 // registers at issue time although the data arrives by the explicit wait that precedes their first use, which is
 // sound only while the compiler neither copies nor spills them in between; they are accumulator-file registers,
-// which nothing else in the kernel wants, and the build refuses scratch memory in this kernel.  A store is followed
-// by the two idle issue slots that the hardware needs before the stored registers may be overwritten (the compiler
-// inserts them for the stores it knows; without them the last lanes of the following block were stored instead).
+// which nothing else in the kernel wants, and the build refuses scratch memory in this kernel and any copy into the
+// accumulator file in its code.  A store is followed by the two idle issue slots that the hardware needs before the
+// stored registers may be overwritten (the compiler inserts them for the stores it knows; without them the last lanes of
+// the following block were stored instead).
+//
+// What was measured on the way (25 000 x 128, one box each): loads of 32 bytes per lane and row, which is what a lane
+// feeds per k step, request every line four times, and the kernel then ran at the rate of the compute unit's queue of
+// outstanding misses (118 us; whole lines: 99 us); stores under a branch make the compiler wait for everything in
+// flight at the top of the loop (hence no conditional rows, see the row numbers below); weaving the operand split of
+// the next k step between the matrix instructions took it to 87 us.  Without its matrix instructions the kernel takes
+// 62 us and without its loads and stores 72 us: what remains is that one wave per SIMD does its memory waits, its LDS
+// round trips and its matrix instructions one after the other.  Two waves per SIMD (eight waves, a tile landing in
+// chunks of 32 columns, no weaving) came out equal at this size and 7 % slower at 100 000 nodes; two tiles ahead
+// instead of one changes nothing (and 64 outstanding instructions per wave is where the counter ends).
 // -----------------------------------------------------------------------------------------------
 constexpr int kResWaves = 4;
 constexpr int kResMaxGroups = 128;

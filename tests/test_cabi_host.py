@@ -123,6 +123,28 @@ def test_build_refuses_scratch_in_hand_scheduled_kernels():
         build._check_no_scratch("mp.hip", ok)
 
 
+def test_build_refuses_copies_into_landing_registers():
+    """The resident-weights linear kernel lands its loads in accumulator-file registers named at issue time; the build
+    scans the device assembly and fails if the compiler copies into that file inside such a kernel."""
+    import importlib.util
+
+    import pytest
+
+    spec = importlib.util.spec_from_file_location("_cm_build", os.path.join(ROOT, "cuda-mace_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    ok = ["_ZN2cm13linear_kernelILi8ELb1EEE:  ; @x", "\tv_accvgpr_write_b32 a3, v7", ".Lfunc_end0:",
+          "_ZN2cm22linear_resident_kernelILi128ELi4ELb0EEE:  ; @y", "\tglobal_load_dwordx4 a[64:67], v[2:3], off nt",
+          "\tv_accvgpr_read_b32 v5, a64", "\tv_accvgpr_write_b32 a0, 0", ".Lfunc_end1:"]
+    build._scan_landing_registers("linear.hip", ok)  # other kernels may copy; a constant is no copy
+    with pytest.raises(RuntimeError, match="copies into the accumulator file"):
+        build._scan_landing_registers("linear.hip", ok[:5] + ["\tv_accvgpr_write_b32 a64, v84"] + ok[5:])
+    with pytest.raises(RuntimeError, match="copies into the accumulator file"):
+        build._scan_landing_registers("linear.hip", ok[:5] + ["\tv_accvgpr_mov_b32 a64, a12"] + ok[5:])
+    with pytest.raises(RuntimeError, match="no code found"):
+        build._scan_landing_registers("linear.hip", ok[:3])
+
+
 def test_header_is_valid_c_and_cpp(tmp_path):
     """The boundary is a C ABI: the header must compile as plain C (what cgo, a Fortran binding generator or LAMMPS'
     C glue would include) and as C++, on its own."""
