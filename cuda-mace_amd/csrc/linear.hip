@@ -686,6 +686,7 @@ __global__ __launch_bounds__(kResWaves *kWave, 1) void linear_resident_kernel(
     f4 sland[SCALED ? 2 * KS : 1];
     float *stg = sStage + wave * kStageFloats;
     const int orow = lane / 8, opiece = lane % 8;
+    int t_scales = -1;  // node tile whose row_scale rows are in (or on their way into) sland
     auto issue = [&](int idx, int &m_of, int &tb_of) {
       const int j = idx - blk0;
       const int t = j / nm;
@@ -700,13 +701,21 @@ __global__ __launch_bounds__(kResWaves *kWave, 1) void linear_resident_kernel(
 #pragma unroll
           for (int ln = 0; ln < kLines; ++ln)
             asm volatile("global_load_dwordx4 %0, %1, off offset:%2 nt" : "=a"(land[(c * 4 + rg) * kLines + ln]) : "v"(xp), "n"(4 * (c * kChunk + 32 * ln)) : "memory");
-        if constexpr (SCALED) {
-          const float *sp = row_scale + static_cast<int64_t>(nd) * K + 4 * opiece;
+      }
+      if constexpr (SCALED) {
+        // the 2 l + 1 tiles of a node tile follow each other and share their row_scale rows: fetched once (these loads
+        // are older than the stores the wait at the top of a tile lets stay out, whether they are issued or not)
+        if (t != t_scales) {
+          t_scales = t;
 #pragma unroll
-          for (int c = 0; c < kChunks; ++c)
+          for (int rg = 0; rg < 4; ++rg) {
+            const float *sp = row_scale + static_cast<int64_t>(sId[tb_of + 8 * rg + orow]) * K + 4 * opiece;
 #pragma unroll
-            for (int ln = 0; ln < kLines; ++ln)
-              asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=a"(sland[(c * 4 + rg) * kLines + ln]) : "v"(sp), "n"(4 * (c * kChunk + 32 * ln)) : "memory");
+            for (int c = 0; c < kChunks; ++c)
+#pragma unroll
+              for (int ln = 0; ln < kLines; ++ln)
+                asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=a"(sland[(c * 4 + rg) * kLines + ln]) : "v"(sp), "n"(4 * (c * kChunk + 32 * ln)) : "memory");
+          }
         }
       }
     };
