@@ -375,6 +375,41 @@ def test_linear_many_rows(cabi, N, C, ne, seed):
     close(cabi.linear(Xd, WT, perm2, off2), ref, 1e-5, 2e-6)
 
 
+@pytest.mark.parametrize("N,C", [(25000, 128), (100000, 192), (5000, 96)])
+def test_linear_at_benchmark_sizes(cabi, N, C):
+    """The channel mixing at the node and channel counts of benchmark configurations 4, 5 and 3, per-element weights
+    with row_scale (the backward launch of the model): 1 500 random rows against the fp64 oracle, and linearity in X
+    over the whole output (the kernel applied to a X1 + b X2 equals a out1 + b out2 to fp32 rounding)."""
+    _say("linear_at_benchmark_sizes", N, C)
+    ne = 10
+    g = torch.Generator(device=DEV).manual_seed(N + C)
+    X1 = torch.randn(N, 16, C, device=DEV, generator=g)
+    X2 = torch.randn(N, 16, C, device=DEV, generator=g)
+    S = torch.randn(N, C, device=DEV, generator=g)
+    WT = torch.randn(ne, 4, C, C, device=DEV, generator=g)
+    elem = torch.randint(0, ne, (N,), device=DEV, generator=g)
+    perm, off = cabi.stable_key_sort(elem.int(), ne)
+    out1 = cabi.linear(X1, WT, perm, off, row_scale=S)
+    rows = torch.randperm(N, device=DEV, generator=g)[:1500]
+    W = WT.transpose(-1, -2).double().cpu()
+    er, Xr, Sr = elem[rows].cpu(), X1[rows].double().cpu(), S[rows].double().cpu()
+    ref = torch.zeros(rows.numel(), 16, C, dtype=torch.float64)
+    for e in range(ne):
+        sel = (er == e).nonzero()[:, 0]
+        if sel.numel():
+            ref[sel] = O.linear(Xr[sel] * Sr[sel][:, None, :], W[e])
+    close(out1[rows], ref, 1e-5, 2e-6)
+    out2 = cabi.linear(X2, WT, perm, off, row_scale=S)
+    a, b = 0.75, -1.5  # exact in fp32, so the combined input is rounded once per element
+    out12 = cabi.linear(a * X1 + b * X2, WT, perm, off, row_scale=S)
+    scale = float(out1.abs().max())
+    assert float((out12 - (a * out1 + b * out2)).abs().max()) < 2e-5 * scale
+    del out12, out2, X2
+    # plain weights, no row_scale (the forward launch of the second layer)
+    outp = cabi.linear(X1, WT[0])
+    close(outp[rows], O.linear(Xr, W[0]), 1e-5, 2e-6)
+
+
 # ------------------------------------------------------------------------------------------------
 # symmetric contraction with synthetic sparse tables
 # ------------------------------------------------------------------------------------------------
