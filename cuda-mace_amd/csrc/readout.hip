@@ -13,8 +13,9 @@
 // optionally written to row feats_rows[n], for callers that keep their nodes in another order internally).  The
 // backward is then a scaling of those derivatives by the incoming gradient of e[n].
 //
-// Work split: a workgroup of 256 threads takes 16 nodes; their h2 rows are staged in LDS with coalesced loads and
-// W2a sits in LDS; thread (node, j) accumulates z_j over the channels, 16-lane shuffles reduce over j.
+// Work split: a workgroup of 256 threads keeps W2a and w1 in LDS and walks tiles of 16 nodes; a tile's rows of both
+// feature arrays are staged in LDS with coalesced 16-byte loads; thread (node, j) accumulates z_j over the channels,
+// 16-lane shuffles reduce over j.
 #include <cmath>
 
 #include "common.hpp"
@@ -26,6 +27,7 @@ constexpr int kNodes = 16;    // nodes per workgroup
 constexpr int kHidden = 16;   // threads per node = largest hidden width handled
 constexpr int kMaxC = 256;
 constexpr int kLdW = kHidden + 1;  // padded row stride of the weight tile in LDS (doubles)
+constexpr int kMaxGroups = 512; // workgroups of a forward launch
 constexpr int kLdS = kMaxC + 1;    // padded row stride of the feature tile: the four nodes of a wave hit different banks
 
 __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
@@ -34,69 +36,123 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     double *__restrict__ node_es, float *__restrict__ d2, double *__restrict__ feats64,
     const int32_t *__restrict__ feats_rows) {
   __shared__ double sW[kMaxC * kLdW];      // W2a [C, H], H padded to 16 columns with zeros
+  __shared__ double sw1[kMaxC];
+  __shared__ float s1[kNodes * kLdS];
   __shared__ float s2[kNodes * kLdS];
   __shared__ double sD[kNodes * kHidden];  // w2b[j] * act'(z_j) per node
   const int t = threadIdx.x;
-  const int node0 = blockIdx.x * kNodes;
-  const int rows = min(kNodes, nnodes - node0);
   for (int i = t; i < C * kHidden; i += blockDim.x) {
     const int c = i / kHidden, j = i % kHidden;
     sW[c * kLdW + j] = j < H ? W2a[c * H + j] : 0.0;
   }
-  for (int i = t; i < rows * C; i += blockDim.x) {
-    const int r = i / C, c = i % C;
-    const float b = h2[static_cast<int64_t>(node0 + r) * C + c];
-    const float a = feats64 ? h1[static_cast<int64_t>(node0 + r) * C + c] : 0.f;
-    s2[r * kLdS + c] = b;
-    if (feats64) {
-      const int row = feats_rows ? feats_rows[node0 + r] : node0 + r;
-      if (static_cast<unsigned>(row) < static_cast<unsigned>(nnodes)) {
-        feats64[static_cast<int64_t>(row) * (2 * C) + c] = a;
-        feats64[static_cast<int64_t>(row) * (2 * C) + C + c] = b;
+  for (int c = t; c < C; c += blockDim.x) sw1[c] = w1[c];
+  // a workgroup stages the weights once and then walks tiles of 16 nodes; the rows of its next tile are requested
+  // before the current one is worked on (one element per trip, each waited for, would cost a memory latency per trip)
+  const int ntiles = (nnodes + kNodes - 1) / kNodes;
+  constexpr int kTrips = kNodes * kMaxC / 4 / (kNodes * kHidden);  // 16-byte pieces per thread at the widest C
+  const bool wide = C % 4 == 0;
+  f4 a[kTrips], b[kTrips];
+  auto request = [&](int tile) {
+    const int node0 = tile * kNodes;
+    const int n4 = min(kNodes, nnodes - node0) * C / 4;
+    const float *p1 = h1 + static_cast<int64_t>(node0) * C, *p2 = h2 + static_cast<int64_t>(node0) * C;
+#pragma unroll
+    for (int u = 0; u < kTrips; ++u) {
+      const int q = t + u * (kNodes * kHidden);
+      a[u] = q < n4 ? ld4(p1 + 4 * q) : zero4();
+      b[u] = q < n4 ? ld4(p2 + 4 * q) : zero4();
+    }
+  };
+  if (wide && static_cast<int>(blockIdx.x) < ntiles) request(blockIdx.x);
+  for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    const int node0 = tile * kNodes;
+    const int rows = min(kNodes, nnodes - node0);
+    __syncthreads();  // the previous tile's rows and sD have been read (and, before the first tile, the weights are written)
+    // the tile's rows of both feature arrays -> LDS (and, on request, -> the fp64 concatenation)
+    if (wide) {
+      const int n4 = rows * C / 4;
+#pragma unroll
+      for (int u = 0; u < kTrips; ++u) {
+        const int q = t + u * (kNodes * kHidden);
+        if (q < n4) {
+          const int r = 4 * q / C, c = 4 * q % C;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            s1[r * kLdS + c + k] = a[u][k];
+            s2[r * kLdS + c + k] = b[u][k];
+          }
+          if (feats64) {
+            const int row = feats_rows ? feats_rows[node0 + r] : node0 + r;
+            if (static_cast<unsigned>(row) < static_cast<unsigned>(nnodes)) {
+              double *f = feats64 + static_cast<int64_t>(row) * (2 * C) + c;
+#pragma unroll
+              for (int k = 0; k < 4; ++k) {
+                f[k] = a[u][k];
+                f[C + k] = b[u][k];
+              }
+            }
+          }
+        }
+      }
+      if (tile + static_cast<int>(gridDim.x) < ntiles) request(tile + gridDim.x);
+    } else {
+      for (int i = t; i < rows * C; i += blockDim.x) {
+        const int r = i / C, c = i % C;
+        const float av = h1[static_cast<int64_t>(node0 + r) * C + c];
+        const float bv = h2[static_cast<int64_t>(node0 + r) * C + c];
+        s1[r * kLdS + c] = av;
+        s2[r * kLdS + c] = bv;
+        if (feats64) {
+          const int row = feats_rows ? feats_rows[node0 + r] : node0 + r;
+          if (static_cast<unsigned>(row) < static_cast<unsigned>(nnodes)) {
+            feats64[static_cast<int64_t>(row) * (2 * C) + c] = av;
+            feats64[static_cast<int64_t>(row) * (2 * C) + C + c] = bv;
+          }
+        }
       }
     }
-  }
-  __syncthreads();
-  const int r = t / kHidden, j = t % kHidden;
-  const bool live = r < rows;
-  // first readout: each of the node's 16 threads takes every 16th channel
-  double e1 = 0.0, z = 0.0;
-  if (live) {
-    const float *row1 = h1 + static_cast<int64_t>(node0 + r) * C;
-    for (int c = j; c < C; c += kHidden) e1 += static_cast<double>(row1[c]) * w1[c];
-    // four independent partial sums: the fp64 multiply-add chain is otherwise as long as the channel count
-    double z0 = 0.0, z1 = 0.0, z2 = 0.0, z3 = 0.0;
-    const float *srow = s2 + r * kLdS;
-    const double *wcol = sW + j;
-    int c = 0;
+    __syncthreads();
+    const int r = t / kHidden, j = t % kHidden;
+    const bool live = r < rows;
+    // first readout: each of the node's 16 threads takes every 16th channel
+    double e1 = 0.0, z = 0.0;
+    if (live) {
+      const float *row1 = s1 + r * kLdS;
+      for (int c = j; c < C; c += kHidden) e1 += static_cast<double>(row1[c]) * sw1[c];
+      // four independent partial sums: the fp64 multiply-add chain is otherwise as long as the channel count
+      double z0 = 0.0, z1 = 0.0, z2 = 0.0, z3 = 0.0;
+      const float *srow = s2 + r * kLdS;
+      const double *wcol = sW + j;
+      int c = 0;
 #pragma unroll 2
-    for (; c + 3 < C; c += 4) {
-      z0 += static_cast<double>(srow[c]) * wcol[c * kLdW];
-      z1 += static_cast<double>(srow[c + 1]) * wcol[(c + 1) * kLdW];
-      z2 += static_cast<double>(srow[c + 2]) * wcol[(c + 2) * kLdW];
-      z3 += static_cast<double>(srow[c + 3]) * wcol[(c + 3) * kLdW];
+      for (; c + 3 < C; c += 4) {
+        z0 += static_cast<double>(srow[c]) * wcol[c * kLdW];
+        z1 += static_cast<double>(srow[c + 1]) * wcol[(c + 1) * kLdW];
+        z2 += static_cast<double>(srow[c + 2]) * wcol[(c + 2) * kLdW];
+        z3 += static_cast<double>(srow[c + 3]) * wcol[(c + 3) * kLdW];
+      }
+      for (; c < C; ++c) z0 += static_cast<double>(srow[c]) * wcol[c * kLdW];
+      z = (z0 + z1) + (z2 + z3);
     }
-    for (; c < C; ++c) z0 += static_cast<double>(srow[c]) * wcol[c * kLdW];
-    z = (z0 + z1) + (z2 + z3);
-  }
-  double e2 = 0.0, dj = 0.0;
-  if (live && j < H) {
-    const double sig = 1.0 / (1.0 + exp(-z));
-    e2 = w2b[j] * act_cst * z * sig;
-    dj = w2b[j] * act_cst * (sig + z * sig * (1.0 - sig));
-  }
-  sD[t] = dj;
-  double e = e1 + e2;
+    double e2 = 0.0, dj = 0.0;
+    if (live && j < H) {
+      const double sig = 1.0 / (1.0 + exp(-z));
+      e2 = w2b[j] * act_cst * z * sig;
+      dj = w2b[j] * act_cst * (sig + z * sig * (1.0 - sig));
+    }
+    sD[t] = dj;
+    double e = e1 + e2;
 #pragma unroll
-  for (int off = kHidden / 2; off > 0; off >>= 1) e += __shfl_xor(e, off);
-  if (live && j == 0) node_es[node0 + r] = scale * e + shift;
-  __syncthreads();
-  for (int i = t; i < rows * C; i += blockDim.x) {
-    const int rr = i / C, c = i % C;
-    double acc = 0.0;
+    for (int off = kHidden / 2; off > 0; off >>= 1) e += __shfl_xor(e, off);
+    if (live && j == 0) node_es[node0 + r] = scale * e + shift;
+    __syncthreads();
+    for (int i = t; i < rows * C; i += blockDim.x) {
+      const int rr = i / C, c = i % C;
+      double acc = 0.0;
 #pragma unroll
-    for (int q = 0; q < kHidden; ++q) acc += sW[c * kLdW + q] * sD[rr * kHidden + q];
-    d2[static_cast<int64_t>(node0 + rr) * C + c] = static_cast<float>(scale * acc);
+      for (int q = 0; q < kHidden; ++q) acc += sW[c * kLdW + q] * sD[rr * kHidden + q];
+      d2[static_cast<int64_t>(node0 + rr) * C + c] = static_cast<float>(scale * acc);
+    }
   }
 }
 
@@ -121,7 +177,10 @@ extern "C" int cm_readout_forward(const float *h1, const float *h2, const double
   CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 2, "cm_readout_forward: nnodes out of range");
   if (nnodes == 0) return CM_OK;
   CM_REQUIRE(h1 && h2 && w1 && W2a && w2b && node_energies && d_h2, "cm_readout_forward: NULL pointer");
-  hipLaunchKernelGGL(cm::readout_forward_kernel, dim3(static_cast<unsigned>(cm::ceil_div(nnodes, cm::kNodes))),
+  // at most kMaxGroups workgroups (two per compute unit of a 256-unit device fit by their LDS): each stages the
+  // weights once and walks several tiles
+  const int64_t tiles = cm::ceil_div(nnodes, cm::kNodes);
+  hipLaunchKernelGGL(cm::readout_forward_kernel, dim3(static_cast<unsigned>(tiles < cm::kMaxGroups ? tiles : cm::kMaxGroups)),
                      dim3(cm::kNodes * cm::kHidden), 0, cm::as_stream(stream), h1, h2, w1, W2a, w2b, act_cst, scale, shift,
                      static_cast<int>(nnodes), channels, hidden, node_energies, d_h2, node_feats64, feats_rows);
   return cm::check_launch("cm_readout_forward");

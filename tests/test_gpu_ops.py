@@ -525,7 +525,7 @@ def test_edge_geometry(cabi, nnodes, avg, iso, seed):
 
 
 # ---- readouts ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("N,C,H,seed", [(1, 32, 16, 0), (1000, 128, 16, 1), (37, 96, 5, 2), (515, 256, 1, 3), (16, 64, 16, 4)])
+@pytest.mark.parametrize("N,C,H,seed", [(1, 32, 16, 0), (1000, 128, 16, 1), (37, 96, 5, 2), (515, 256, 1, 3), (16, 64, 16, 4), (50, 30, 7, 5), (20000, 128, 16, 6)])
 def test_readout_forward_backward(cabi, N, C, H, seed):
     g = torch.Generator().manual_seed(seed)
     h1 = torch.randn(N, C, generator=g).double()
