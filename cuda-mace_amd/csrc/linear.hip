@@ -39,18 +39,27 @@ constexpr int kTileNodes = 32 * kWaves;  // rows per workgroup (MFMA M = 32 per 
 constexpr int kKC = 32;                  // K columns staged per step
 constexpr int kLdH = kKC + 8;            // padded LDS row stride of a bf16 plane (elements; 80 bytes: conflict-free b128 reads)
 
-// a = hi + mid + lo with bf16 pieces (round to nearest at every step; the remainders are exact in fp32)
+// a = hi + mid + lo with bf16 pieces (round to nearest at every step; the remainders are exact in fp32).  Two values at a
+// time: the packed conversion rounds both and leaves the pieces in the order the matrix instruction takes them, and a
+// piece widens back to fp32 by a shift or a mask (11 instructions per pair; element by element the compiler converts
+// every value alone, widens it, and packs the pairs at the end with further conversions: 15).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f2 __attribute__((ext_vector_type(2)));
+typedef unsigned u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void split3_pair(float v0, float v1, unsigned &hi, unsigned &mid, unsigned &lo) {
+  hi = __builtin_bit_cast(unsigned, __builtin_convertvector(f2{v0, v1}, bf16x2));
+  const float r0 = v0 - __builtin_bit_cast(float, hi << 16), r1 = v1 - __builtin_bit_cast(float, hi & 0xffff0000u);
+  mid = __builtin_bit_cast(unsigned, __builtin_convertvector(f2{r0, r1}, bf16x2));
+  const float q0 = r0 - __builtin_bit_cast(float, mid << 16), q1 = r1 - __builtin_bit_cast(float, mid & 0xffff0000u);
+  lo = __builtin_bit_cast(unsigned, __builtin_convertvector(f2{q0, q1}, bf16x2));
+}
 __device__ __forceinline__ void split3(f4 v, bf16x4 &hi, bf16x4 &mid, bf16x4 &lo) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const __bf16 h = static_cast<__bf16>(v[j]);
-    const float r1 = v[j] - static_cast<float>(h);
-    const __bf16 m = static_cast<__bf16>(r1);
-    const float r2 = r1 - static_cast<float>(m);
-    hi[j] = h;
-    mid[j] = m;
-    lo[j] = static_cast<__bf16>(r2);
-  }
+  unsigned h0, m0, l0, h1, m1, l1;
+  split3_pair(v.x, v.y, h0, m0, l0);
+  split3_pair(v.z, v.w, h1, m1, l1);
+  hi = __builtin_bit_cast(bf16x4, u2{h0, h1});
+  mid = __builtin_bit_cast(bf16x4, u2{m0, m1});
+  lo = __builtin_bit_cast(bf16x4, u2{l0, l1});
 }
 
 // Nout = 32 * NT; SCALED: X is multiplied by row_scale on the way in

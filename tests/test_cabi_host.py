@@ -125,7 +125,7 @@ def test_build_refuses_scratch_in_hand_scheduled_kernels():
 
 def test_build_refuses_copies_into_landing_registers():
     """The resident-weights linear kernel lands its loads in accumulator-file registers named at issue time; the build
-    scans the device assembly and fails if the compiler copies into that file inside such a kernel."""
+    scans the device assembly and fails if anything but a load writes one of those registers inside such a kernel."""
     import importlib.util
 
     import pytest
@@ -135,14 +135,15 @@ def test_build_refuses_copies_into_landing_registers():
     spec.loader.exec_module(build)
     ok = ["_ZN2cm13linear_kernelILi8ELb1EEE:  ; @x", "\tv_accvgpr_write_b32 a3, v7", ".Lfunc_end0:",
           "_ZN2cm22linear_resident_kernelILi128ELi4ELb0EEE:  ; @y", "\tglobal_load_dwordx4 a[64:67], v[2:3], off nt",
-          "\tv_accvgpr_read_b32 v5, a64", "\tv_accvgpr_write_b32 a0, 0", ".Lfunc_end1:"]
-    build._scan_landing_registers("linear.hip", ok)  # other kernels may copy; a constant is no copy
-    with pytest.raises(RuntimeError, match="copies into the accumulator file"):
-        build._scan_landing_registers("linear.hip", ok[:5] + ["\tv_accvgpr_write_b32 a64, v84"] + ok[5:])
-    with pytest.raises(RuntimeError, match="copies into the accumulator file"):
-        build._scan_landing_registers("linear.hip", ok[:5] + ["\tv_accvgpr_mov_b32 a64, a12"] + ok[5:])
+          "\tv_accvgpr_read_b32 v5, a64", "\tv_accvgpr_write_b32 a0, 0", "\tv_accvgpr_write_b32 a130, v9", ".Lfunc_end1:"]
+    build._scan_landing_registers("linear.hip", ok)  # other kernels may copy; so may this one outside its landing registers
+    for bad in ("\tv_accvgpr_write_b32 a66, v84", "\tv_accvgpr_mov_b32 a64, a12"):
+        with pytest.raises(RuntimeError, match="copies into a landing register"):
+            build._scan_landing_registers("linear.hip", ok[:5] + [bad] + ok[5:])
     with pytest.raises(RuntimeError, match="no code found"):
         build._scan_landing_registers("linear.hip", ok[:3])
+    with pytest.raises(RuntimeError, match="no load into the accumulator file"):
+        build._scan_landing_registers("linear.hip", ok[:4] + ok[5:])
 
 
 def test_header_is_valid_c_and_cpp(tmp_path):
