@@ -542,8 +542,8 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
 // Contract of the hand-issued memory operations of the tile loop (the loads and the stores): a load names its landing
 // registers at issue time although the data arrives by the explicit wait that precedes their first use, which is
 // sound only while the compiler neither copies nor spills them in between; they are accumulator-file registers,
-// which nothing else in the kernel wants, and the build refuses scratch memory in this kernel and any copy into the
-// accumulator file in its code.  A store is followed by the two idle issue slots that the hardware needs before the
+// which nothing else in the kernel wants, and the build refuses scratch memory in this kernel and any instruction other
+// than a load that writes a register its loads land in.  A store is followed by the two idle issue slots that the hardware needs before the
 // stored registers may be overwritten (the compiler inserts them for the stores it knows; without them the last lanes of
 // the following block were stored instead).
 //
