@@ -3,7 +3,8 @@
 // one.  Nothing here computes; this file is the order of the launches and the layout of the workspace.
 //
 // Forward                                         Backward (seed -1 on every node energy: the chain delivers forces)
-//   vec        = pos[snd] - pos[rcv] + shift        g1, g2    = readout backward
+//   vec        = pos[snd] - pos[rcv] + shift        g1 = -scale w1 (every node), g2 = -dE/dh2 (never stored: the sign
+//                                                             goes into the scale of the linears that read dE/dh2)
 //   M1         = MP(X1, vec, spline 0)              gB2       = g2 . Wprod2^T
 //   A          = mix0(M1)        (per element)      gA        = (gB2 * grad2) . Wmix1^T      (contraction backward folded)
 //   B1, grad1  = contraction 0 (A)                  gX2, gv2  = MP backward(X2, vec, spline 1, gA)
@@ -78,6 +79,14 @@ __global__ void fill_f64_kernel(double *p, int64_t n, double value) {
     p[i] = value;
 }
 
+// g1[n, c] = -scale * w1[c]: the gradient of -sum(node energies) with respect to the first layer's features (the linear
+// readout), the same row for every node
+__global__ void seed_linear_readout_kernel(float *__restrict__ g1, const double *__restrict__ w1, double scale, int64_t total, int C) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    g1[i] = static_cast<float>(-1.0 * scale * w1[i % C]);
+}
+
 // a += b, 16 bytes per lane where the length allows
 __global__ void add_f32_kernel(float *__restrict__ a, const float *__restrict__ b, int64_t n) {
   const int64_t n4 = n / 4;
@@ -110,8 +119,7 @@ inline size_t align256(size_t n) { return (n + 255) & ~static_cast<size_t>(255);
 // Carves the workspace; the same walk sizes it (base == nullptr) and lays it out.
 struct Layout {
   float *vec, *len, *gv1, *gv2, *bufM1, *bufM2, *bufA, *edge_scratch;
-  float *B1, *h1, *sc, *X2, *B2, *h2, *d_h2, *g1, *g2, *gB, *gX2, *gh1a, *gh1;
-  double *seed;
+  float *B1, *h1, *sc, *X2, *B2, *h2, *d_h2, *g1, *gB, *gX2, *gh1a, *gh1;
   size_t bytes;
 
   Layout(void *base, int64_t N, int64_t E, int C) {
@@ -127,8 +135,7 @@ struct Layout {
     bufM1 = f(16 * NC), bufM2 = f(16 * NC), bufA = f(16 * NC);
     edge_scratch = f(E * C);
     B1 = f(NC), h1 = f(NC), sc = f(NC), X2 = f(NC), B2 = f(NC), h2 = f(NC), d_h2 = f(NC);
-    g1 = f(NC), g2 = f(NC), gB = f(NC), gX2 = f(NC), gh1a = f(NC), gh1 = f(NC);
-    seed = reinterpret_cast<double *>(take(static_cast<size_t>(N) * sizeof(double)));
+    g1 = f(NC), gB = f(NC), gX2 = f(NC), gh1a = f(NC), gh1 = f(NC);
     bytes = at;
   }
 };
@@ -247,16 +254,21 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
                      interaction_energy);
 
   // ---- backward: d(-sum of node energies) / d positions ----
-  hipLaunchKernelGGL(cm::fill_f64_kernel, dim3(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(N, 256), 1024))), dim3(256), 0,
-                     st, L.seed, N, -1.0);
-  CM_STAGE(13, cm_readout_backward(L.seed, w->w1, L.d_h2, w->scale, N, C, L.g1, L.g2, stream));
+  // The seed is -1 on every node energy, so the readouts' backward needs no pass of its own: the gradient with respect to
+  // the second layer's features is -d_h2 (the sign goes into the scale of the two linears that consume it, which is
+  // exact), the one with respect to the first layer's is a constant row.
+  {
+    cm::StageTimer timer_(st, 13, timing_mask);
+    hipLaunchKernelGGL(cm::seed_linear_readout_kernel, dim3(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(N * C, 256), 2048))),
+                       dim3(256), 0, st, L.g1, w->w1, w->scale, static_cast<int64_t>(N) * C, C);
+  }
   // layer 1 (second interaction)
-  CM_STAGE(14, cm_linear(L.g2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.gB, stream));
+  CM_STAGE(14, cm_linear(L.d_h2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, -1.0f, none, none, L.gB, stream));
   CM_STAGE(15, cm_linear(L.bufM2, w->mix_W[1], nullptr, nullptr, N, 1, 0, 16, C, C, w->mix_scale[1], L.gB, none, L.bufA, stream));
   CM_STAGE(16, cm_mp_edge_backward(L.X2, L.vec, w->r_knots, w->spline[1], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
                               g->first_occ, g->sender_perm, g->sender_offsets, N, E, C, L.gX2, L.gv2, L.edge_scratch, stream));
   CM_STAGE(17, cm_linear(L.gX2, w->up_W, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, L.g1, L.gh1a, stream));
-  CM_STAGE(18, cm_linear(L.g2, w->skip_W, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, w->skip_scale, none, L.gh1a, L.gh1, stream));
+  CM_STAGE(18, cm_linear(L.d_h2, w->skip_W, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, -w->skip_scale, none, L.gh1a, L.gh1, stream));
   // layer 0 (first interaction): its input features depend on the species alone, so no gradient with respect to them
   CM_STAGE(19, cm_linear(L.gh1, w->prod_W[0], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.gB, stream));
   CM_STAGE(20, cm_linear(L.bufM1, w->mix_W[0], oh_perm, oh_off, N, ne + 1, 1, 16, C, C, w->mix_scale[0], L.gB, none, L.bufA, stream));
