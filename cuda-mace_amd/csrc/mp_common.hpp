@@ -258,6 +258,13 @@ int launch_sender_pass(int channels, const float *gXe, const int32_t *perm, cons
                        int64_t nedges, float *gX, hipStream_t st, const float *live_vec = nullptr,
                        const float *live_r = nullptr, float r_max = 0.f);
 
+// Forward from edge vectors with the radial table in LDS, one degree and one 32-channel slice per workgroup (defined in
+// mp_sliced.hip): whether it takes a launch of this shape, and the launch.
+bool sliced_forward_applies(int64_t nnodes, int channels, int nknots);
+int launch_sliced_forward(const float *X, const float *vec, const float *knots, const float *coeffs, int nknots, float r_width,
+                          float r_max, const int32_t *sender, const int32_t *first_occ, int64_t nnodes, int64_t nedges,
+                          int channels, float *out, hipStream_t st);
+
 }  // namespace mp
 }  // namespace cm
 

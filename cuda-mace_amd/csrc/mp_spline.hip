@@ -495,6 +495,9 @@ extern "C" int cm_mp_edge_forward(const float *X, const float *vectors, const fl
   CM_REQUIRE(nedges == 0 || sender, "cm_mp_edge_forward: NULL edge operand");
   int rc = cm::check_spline("cm_mp_edge_forward", vectors, r_knots, coeffs, nknots, r_width, nedges, nnodes, channels);
   if (rc != CM_OK) return rc;
+  if (nedges > 0 && cm::mp::sliced_forward_applies(nnodes, channels, nknots))
+    return cm::mp::launch_sliced_forward(X, vectors, r_knots, coeffs, nknots, r_width, r_max, sender, first_occ, nnodes, nedges,
+                                         channels, out, cm::as_stream(stream));
   const cm::Spline sp{vectors, nullptr, r_knots, coeffs, nknots, r_width, r_max};
   rc = CM_EINVAL;
   CM_DISPATCH_C(channels, rc = (cm::launch_forward<C_, true>(X, nullptr, sp, sender, first_occ, nnodes, nedges, out, cm::as_stream(stream))));

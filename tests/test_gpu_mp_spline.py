@@ -146,3 +146,85 @@ def test_edges_beyond_cutoff_and_invalid_senders_cost_nothing_and_contribute_not
     gvec_only = cabi.mp_edge_backward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, d(G), snd.cuda(), fo, perm, off, nnodes,
                                       need_gX=False)[1]
     assert torch.equal(gvec_only, gvec)
+
+
+# ---- many receiver nodes: the forward from edge vectors runs on the kernel that keeps its part of the table in LDS ----
+def _edge_case(nnodes, avg, C, iso, seed, nknots=256, heavy=0):
+    """Receiver-sorted random graph with edge vectors of lengths 0.7 .. 5.3 (r_max = 5), a few senders out of range,
+    optionally one node with `heavy` extra edges (more edge blocks than the kernel's node sort tells apart)."""
+    snd, rcv = random_graph(nnodes, avg, seed, isolated_frac=iso)
+    if heavy:
+        g0 = torch.Generator().manual_seed(seed + 5)
+        node = nnodes // 3
+        extra = torch.randint(0, nnodes, (heavy,), generator=g0, dtype=torch.int32)
+        at = int(torch.searchsorted(rcv, torch.tensor(node, dtype=torch.int32)))
+        snd = torch.cat([snd[:at], extra, snd[at:]])
+        rcv = torch.cat([rcv[:at], torch.full((heavy,), node, dtype=torch.int32), rcv[at:]])
+    E = snd.numel()
+    g = torch.Generator().manual_seed(seed + 100)
+    X = torch.randn(nnodes, C, generator=g, dtype=torch.float64)
+    r = torch.rand(E, generator=g, dtype=torch.float64) * 4.6 + 0.7
+    vec = torch.randn(E, 3, generator=g, dtype=torch.float64)
+    vec = (vec / vec.norm(dim=1, keepdim=True) * r[:, None]).float().double()
+    snd = snd.clone()
+    bad = torch.randperm(E, generator=g)[:30]
+    snd[bad[:15]] = nnodes + 5
+    snd[bad[15:]] = -1
+    knots_np, h = np.linspace(1e-12, 6.0, nknots, retstep=True)
+    knots = torch.from_numpy(knots_np)
+    table = torch.sin(knots[:, None] * torch.linspace(0.5, 2.5, 4 * C, dtype=torch.float64)[None, :]) * torch.randn(
+        1, 4 * C, generator=g, dtype=torch.float64)
+    coeffs = O.spline_coefficients(knots, table).float().double()
+    return snd, rcv, X, vec, knots.float().double(), coeffs, float(np.float32(h))
+
+
+MANY_NODES = [
+    # nnodes, avg degree, channels, isolated fraction, seed, knots, extra edges of one node
+    (2100, 14, 32, 0.1, 0, 256, 0),
+    (2300, 9, 64, 0.0, 1, 256, 300),   # one node with more than 63 blocks of four edges
+    (2048, 21, 96, 0.05, 2, 200, 0),
+    (3000, 6, 160, 0.3, 3, 256, 0),
+    (2500, 3, 256, 0.0, 4, 272, 0),    # the largest table the kernel keeps in LDS
+]
+
+
+@pytest.mark.parametrize("case", MANY_NODES, ids=lambda c: "N%d_d%d_C%d_k%d" % (c[0], c[1], c[2], c[5]))
+def test_mp_edge_forward_many_nodes(cabi, case):
+    """Parity with the fp64 oracle (harmonics, spline, message-passing definition) on the live edges; edges beyond the
+    cutoff or with a sender out of range add nothing; nodes without edges come out as zeros; the result is the same
+    on a second call (which wave serves a node changes from run to run, the node's result must not)."""
+    print("mp_edge_forward many nodes", case, flush=True)
+    nnodes, C = case[0], case[2]
+    snd, rcv, X, vec, knots, coeffs, h = _edge_case(*case)
+    live = (vec.norm(dim=1).float() <= 5.0) & (snd >= 0) & (snd < nnodes)
+    Rv = O.spline_eval(vec[live].norm(dim=1), knots, coeffs, h, 5.0).view(-1, 4, C)
+    ref = O.mp_forward(X, O.spherical_harmonics(vec[live]), Rv, snd[live], rcv[live], nnodes)
+    d = lambda t: t.float().cuda()
+    fo = cabi.first_occurences(rcv.cuda(), nnodes)
+    out = cabi.mp_edge_forward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, snd.cuda(), fo, nnodes)
+    close(out, ref, 2e-5, 2e-6)
+    empty = torch.bincount(rcv.long(), minlength=nnodes) == 0
+    assert float(out[empty.cuda()].abs().max()) == 0.0 if bool(empty.any()) else True
+    again = cabi.mp_edge_forward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, snd.cuda(), fo, nnodes)
+    assert torch.equal(out, again)
+
+
+def test_mp_edge_forward_many_nodes_agrees_with_harmonics_and_lengths_path(cabi):
+    """40 000 receiver nodes at 256 channels: a workgroup of the LDS-table kernel sorts and serves its nodes in more than
+    one batch.  Checked against the kernel that takes harmonics and lengths (same radial table, same per-edge
+    arithmetic, another summation order), and against the oracle on a sample of nodes."""
+    nnodes, C = 40000, 256
+    snd, rcv, X, vec, knots, coeffs, h = _edge_case(nnodes, 3, C, 0.1, 9)
+    d = lambda t: t.float().cuda()
+    fo = cabi.first_occurences(rcv.cuda(), nnodes)
+    out = cabi.mp_edge_forward(d(X), d(vec), d(knots), d(coeffs), h, 5.0, snd.cuda(), fo, nnodes)
+    Y = cabi.sh_forward(d(vec))
+    length = d(vec).norm(dim=1)  # rounding of the length may differ from the kernel's in the last bit
+    other = cabi.mp_spline_forward(d(X), Y, length, d(knots), d(coeffs), h, 5.0, snd.cuda(), fo, nnodes)
+    close(out, other.double().cpu(), 1e-4, 1e-5)
+    nodes = torch.arange(0, nnodes, 997)
+    pick = torch.isin(rcv.long(), nodes)
+    live = pick & (vec.norm(dim=1).float() <= 5.0) & (snd >= 0) & (snd < nnodes)
+    Rv = O.spline_eval(vec[live].norm(dim=1), knots, coeffs, h, 5.0).view(-1, 4, C)
+    ref = O.mp_forward(X, O.spherical_harmonics(vec[live]), Rv, snd[live], rcv[live], nnodes)
+    close(out[nodes.cuda()], ref[nodes], 2e-5, 2e-6)
