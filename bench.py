@@ -64,6 +64,14 @@ def traffic_of(table, kernels):
     return None if any(p is None for p in parts) else sum(parts)
 
 
+def forward_kernel_name(C, N):
+    """Kernel that runs the fused forward from edge vectors at this shape (csrc/mp_spline.hip: cm_mp_edge_forward; the
+    benchmark's spline table has 256 knots)."""
+    if N >= 2048 and C % 16 == 0 and N * C < 2**30:
+        return "mp_edge_forward_sliced_kernel"
+    return "mp_spline_forward_kernel<%d,true>" % C
+
+
 def linear_kernel_name(C, N):
     """The library runs the [N,16,C] channel-mixing linear on its kernel with LDS-resident weights for 64, 96 and 128
     columns when there are at least 2 048 nodes, else on the LDS-ring kernel for 64, 96, 128, 224 and 256 columns and on
@@ -141,7 +149,7 @@ def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=
         ]
     if with_fused:
         cases += [
-            ("mp_edge_forward (fused harmonics + spline)", "mp_spline_forward_kernel<%d,true>" % C, fwd_fb,
+            ("mp_edge_forward (fused harmonics + spline)", forward_kernel_name(C, N), fwd_fb,
              lambda: cabi.mp_edge_forward(X, vec, knots, coeffs, float(h), 5.0, snd, fo, N)),
             ("mp_edge_backward grad_vectors (fused)", "mp_spline_backward_edge_kernel<%d,true,true,true,false>" % C, bwd_fb,
              lambda: cabi.mp_edge_backward(X, vec, knots, coeffs, float(h), 5.0, G, snd, fo, None, None, N, need_gX=False)),
@@ -432,19 +440,25 @@ def main():
     if fused:
         sh_b, spline_b = 88 * E, 4 * (8 * E * C + E)  # harmonics backward, spline backward (each operand once)
         sh_f, spline_f = 76 * E, 4 * (E + 8 * E * C)  # harmonics forward, spline forward (each operand once)
-        roofline = entry("mp_spline_forward_kernel<%d,true>" % C, fwd_fb, t_fwd, launches_timed=launches(fwd_name),
+        flops_fwd = 60 * E * C  # per edge and channel: the cubic of 4 degrees (12 FMA), 4 products, 16 accumulations
+        roofline = entry(forward_kernel_name(C, N), fwd_fb, t_fwd, launches_timed=launches(fwd_name),
                          note="dominant kernel of the step by total time (two launches per step). Harmonics and radial "
-                              "weights are evaluated in-kernel, so its own HBM operands are small: the radial coefficients "
-                              "come from the 2 MB spline table in L2 (16 loads of 16 B per lane and edge, texture-address "
-                              "units ~80% busy): bounded by L1 delivery, not HBM; see roofline_other_kernels for the "
-                              "HBM-bound message passing with tabulated R[E,4,C] and for the matrix-core linear",
+                              "weights are evaluated in-kernel, so its own HBM operands are small; a workgroup keeps its "
+                              "part of the spline table (two degrees x 16 channels, 130 KB) in LDS, so the coefficients "
+                              "no longer travel through L1 (the kernel it replaces pulled 8 KB per edge from L2 and ran "
+                              "at 0.37-0.46 ms): bounded by vector-instruction issue (counter summary: ~90% of the SIMDs' "
+                              "four-cycle issue slots with two waves per SIMD, LDS half busy), not by HBM; see "
+                              "roofline_other_kernels for the HBM-bound message passing with tabulated R[E,4,C] and for "
+                              "the matrix-core linear",
                          binding_resource={
-                             "resource": "vector-memory (L1) delivery: 17 loads of 16 B per lane and edge",
-                             "bytes": 68 * E * C, "achieved_GB/s": round(68 * E * C / (t_fwd * 1e-3) / 1e9, 1),
-                             "peak_GB/s": round(256 * 64 * 2.4, 1) * 1.0,
-                             "frac": round(68 * E * C / (t_fwd * 1e-3) / 1e9 / (256 * 64 * 2.4), 4),
-                             "meaning": "bytes the kernel pulls through the per-CU vector-memory path (coefficient table in "
-                                        "L2, sender rows) against 256 CUs x 64 B/clk x 2.4 GHz"},
+                             "resource": "fp32 vector arithmetic: per edge and channel the cubic of 4 degrees (12 FMA), 4 "
+                                         "products and 16 accumulations",
+                             "flops": flops_fwd, "achieved_TFLOP/s": round(flops_fwd / (t_fwd * 1e-3) / 1e12, 1),
+                             "peak_TFLOP/s": 157.3, "frac": round(flops_fwd / (t_fwd * 1e-3) / 1e12 / 157.3, 4),
+                             "meaning": "useful fp32 operations of the formulation against the vector peak; the kernel issues "
+                                        "about 1.8 instructions per useful one (edge set-up per quad of lanes, broadcasts of "
+                                        "the edge's values, addresses), and instructions with a cross-lane operand issue at "
+                                        "less than half the rate of plain ones on this device"},
                          unfused_equivalent={
                              "bytes": fwd_b + sh_f + spline_f,
                              "GB/s": round((fwd_b + sh_f + spline_f) / (t_fwd * 1e-3) / 1e9, 1),

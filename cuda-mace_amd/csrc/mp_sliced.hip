@@ -294,10 +294,20 @@ __global__ __launch_bounds__(kSlThreads) void mp_edge_forward_sliced_kernel(cons
   __shared__ int sNext;
 
   const int tid = threadIdx.x;
-  const int slice = blockIdx.x % p.nslices;
-  const int rest = blockIdx.x / p.nslices;
-  const int pair = rest & 1;
-  const int j = rest >> 1;  // place among the workgroups of the (pair, slice)
+  // Which (pair, slice) and which piece j of the node range.  Consecutive workgroups go to consecutive XCDs (eight of
+  // them, each with its own L2): where the pieces divide evenly among the XCDs, all workgroups of a piece sit on one XCD,
+  // so that the edge data and the X rows of a piece are fetched into one L2 only.
+  int type, j;
+  if (p.share % 8 == 0) {
+    const int xcd = blockIdx.x % 8, q = blockIdx.x / 8;
+    type = q % (2 * p.nslices);
+    j = xcd + 8 * (q / (2 * p.nslices));
+  } else {
+    type = blockIdx.x % (2 * p.nslices);
+    j = blockIdx.x / (2 * p.nslices);
+  }
+  const int slice = type >> 1;
+  const int pair = type & 1;
   const int lo = static_cast<int>(static_cast<int64_t>(p.nnodes) * j / p.share);
   const int hi = static_cast<int>(static_cast<int64_t>(p.nnodes) * (j + 1) / p.share);
 
