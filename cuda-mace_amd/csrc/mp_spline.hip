@@ -15,7 +15,8 @@
 // The FROM_VEC variants go one step further and take the fp32 edge vectors instead of Y and r: the 16 harmonics and the
 // length are computed per edge while the chunk is staged, and the backward turns the reduced gY and g_r of an edge
 // straight into the gradient with respect to its vector (harmonics Jacobian + radial part), so Y[16, E], grad_Y and
-// grad_r never exist either.
+// grad_r never exist either.  From 2 048 receiver nodes on the forward from edge vectors runs on the kernel of
+// mp_sliced.hip, which keeps a workgroup's part of the table in LDS (same arithmetic per edge, sums in list order).
 #include <type_traits>
 
 #include "mp_common.hpp"
