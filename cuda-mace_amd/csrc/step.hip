@@ -5,6 +5,8 @@
 // Forward                                         Backward (seed -1 on every node energy: the chain delivers forces)
 //   vec        = pos[snd] - pos[rcv] + shift        g1 = -scale w1 (every node), g2 = -dE/dh2 (never stored: the sign
 //                                                             goes into the scale of the linears that read dE/dh2)
+//   live       = edge ranges up to the last pair
+//                inside the cutoff (forward MP only)
 //   M1         = MP(X1, vec, spline 0)              gB2       = g2 . Wprod2^T
 //   A          = mix0(M1)        (per element)      gA        = (gB2 * grad2) . Wmix1^T      (contraction backward folded)
 //   B1, grad1  = contraction 0 (A)                  gX2, gv2  = MP backward(X2, vec, spline 1, gA)
@@ -20,6 +22,7 @@
 #include <vector>
 
 #include "common.hpp"
+#include "mp_common.hpp"
 
 namespace cm {
 namespace {
@@ -87,6 +90,28 @@ __global__ void seed_linear_readout_kernel(float *__restrict__ g1, const double 
     g1[i] = static_cast<float>(-1.0 * scale * w1[i % C]);
 }
 
+// Edge range of every receiver node cut back to its last edge inside the cutoff: live[n] = first_occ[n],
+// live[nnodes + n] = one past the last edge e of the node with |vec[e]| <= r_max (the node's first edge if there is
+// none).  The forward message passing skips the edges behind it, which contribute exact zeros (the backward keeps the
+// full range: it writes the zero gradients of those edges).  A Verlet list holds a third more pairs than the cutoff
+// takes in; the model orders each node's pairs with those of the skin shell last, nearest first, so that most of them
+// fall behind this mark.  The length is the one the message-passing kernels compute from the same fp32 vector.
+__global__ void live_range_kernel(const int32_t *__restrict__ first_occ, const float *__restrict__ vec, float r_max, int nnodes,
+                                  int64_t nedges, int32_t *__restrict__ live) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= nnodes) return;
+  int e0 = first_occ[n], e1 = first_occ[nnodes + n];
+  clamp_edge_range(e0, e1, nedges);
+  int e = e1;
+  while (e > e0) {
+    const int64_t q = e - 1;
+    if (mp::edge_length(vec[3 * q + 0], vec[3 * q + 1], vec[3 * q + 2]) <= r_max) break;
+    --e;
+  }
+  live[n] = e0;
+  live[nnodes + n] = e;
+}
+
 // a += b, 16 bytes per lane where the length allows
 __global__ void add_f32_kernel(float *__restrict__ a, const float *__restrict__ b, int64_t n) {
   const int64_t n4 = n / 4;
@@ -120,6 +145,7 @@ inline size_t align256(size_t n) { return (n + 255) & ~static_cast<size_t>(255);
 struct Layout {
   float *vec, *len, *gv1, *gv2, *bufM1, *bufM2, *bufA, *edge_scratch;
   float *B1, *h1, *sc, *X2, *B2, *h2, *d_h2, *g1, *gB, *gX2, *gh1a, *gh1;
+  int32_t *live;  // [2 N] edge ranges cut back to the last edge inside the cutoff
   size_t bytes;
 
   Layout(void *base, int64_t N, int64_t E, int C) {
@@ -136,6 +162,7 @@ struct Layout {
     edge_scratch = f(E * C);
     B1 = f(NC), h1 = f(NC), sc = f(NC), X2 = f(NC), B2 = f(NC), h2 = f(NC), d_h2 = f(NC);
     g1 = f(NC), gB = f(NC), gX2 = f(NC), gh1a = f(NC), gh1 = f(NC);
+    live = reinterpret_cast<int32_t *>(take(static_cast<size_t>(2 * N) * sizeof(int32_t)));
     bytes = at;
   }
 };
@@ -227,6 +254,10 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
 
   // ---- forward ----
   CM_STAGE(0, cm_edge_geometry_forward(positions, g->receiver, g->sender, shifts, g->node_rows, N, E, L.vec, L.len, stream));
+  if (E > 0)
+    hipLaunchKernelGGL(cm::live_range_kernel, dim3(static_cast<unsigned>(cm::ceil_div(N, 256))), dim3(256), 0, st, g->first_occ, L.vec,
+                       w->r_max, static_cast<int>(N), E, L.live);
+  const int32_t *fo_forward = E > 0 ? L.live : g->first_occ;
   const float *X[2] = {g->X1, L.X2};
   float *bufM[2] = {L.bufM1, L.bufM2};
   float *B[2] = {L.B1, L.B2};
@@ -237,7 +268,7 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
       CM_STAGE(5, cm_linear(L.h1, w->skip_WT, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, w->skip_scale, none, none, L.sc, stream));
       CM_STAGE(6, cm_linear(L.h1, w->up_WT, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.X2, stream));
     }
-    CM_STAGE(t == 0 ? 1 : 7, cm_mp_edge_forward(X[t], L.vec, w->r_knots, w->spline[t], w->nknots, w->r_width, w->r_max, g->sender, g->first_occ, N,
+    CM_STAGE(t == 0 ? 1 : 7, cm_mp_edge_forward(X[t], L.vec, w->r_knots, w->spline[t], w->nknots, w->r_width, w->r_max, g->sender, fo_forward, N,
                                E, C, bufM[t], stream));
     if (t == 0)
       CM_STAGE(2, cm_linear(bufM[t], w->mix_WT[t], oh_perm, oh_off, N, ne + 1, 1, 16, C, C, w->mix_scale[t], none, none, L.bufA, stream));

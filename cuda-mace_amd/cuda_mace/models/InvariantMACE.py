@@ -420,7 +420,8 @@ class OptimizedInvariantMACE(torch.nn.Module):
 
     def _spatial_order(self, data: Dict[str, torch.Tensor]):
         """Relabelling of one neighbour list: atoms sorted by (graph, 3-D bin of half the cutoff, lexicographic), edges
-        re-sorted by the new (row 0, row 1) labels.  Returns (perm new -> old [N], inverse [N], edge_perm new -> old [E],
+        re-sorted by the new row-0 label and, inside a row-0 segment, by the row-1 label with the pairs beyond the cutoff
+        last.  Returns (perm new -> old [N], inverse [N], edge_perm new -> old [E],
         relabelled edge_index [2, E], relabelled batch [N]).  Any permutation is valid; this one is cheap and keeps
         neighbours within a few hundred indices of each other."""
         pos = data["positions"].detach()
@@ -434,7 +435,20 @@ class OptimizedInvariantMACE(torch.nn.Module):
         inverse = torch.empty_like(perm)
         inverse[perm] = torch.arange(n, device=perm.device)
         row0, row1 = inverse[edge_index[0]], inverse[edge_index[1]]
-        edge_perm = torch.argsort(row0 * n + row1, stable=True)
+        # Inside a row-0 segment: the pairs within the cutoff by their row-1 label, then those beyond it (the skin shell
+        # of a Verlet list), nearest first.  The native step cuts every segment back to its last pair inside the cutoff
+        # before the forward message passing; with this order the pairs that drift inside between two list builds are
+        # the first of the shell, so the cut stays close to the pairs that count.  (Three stable sorts: by length, by
+        # the in-segment key, by segment.)
+        if "shifts" in data:
+            length = (pos[edge_index[1]] - pos[edge_index[0]] + data["shifts"].detach().to(pos.dtype)).norm(dim=1)
+            shell = length > float(self.r_max)
+            by_length = torch.argsort(torch.where(shell, length, torch.zeros_like(length)), stable=True)  # the rest stays put
+            inner_key = torch.where(shell, torch.full_like(row1, n), row1)[by_length]
+            by_inner = by_length[torch.argsort(inner_key, stable=True)]
+            edge_perm = by_inner[torch.argsort(row0[by_inner], stable=True)]
+        else:
+            edge_perm = torch.argsort(row0 * n + row1, stable=True)
         new_edges = torch.stack((row0[edge_perm], row1[edge_perm])).contiguous()
         return perm, inverse, edge_perm, new_edges, batch[perm].contiguous()
 

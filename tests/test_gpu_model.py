@@ -365,3 +365,35 @@ def test_native_step_equals_autograd_path(cabi, case):
     ref = M.energy_and_forces(up.export_params(), data)
     assert abs(float(a["energy"].sum()) - float(ref["energy"])) <= E_RTOL * abs(float(ref["energy"]))
     assert float((a["forces"].cpu() - ref["forces"]).abs().max()) <= F_ATOL
+
+
+@pytest.mark.parametrize("relabel", [True, False], ids=["shell_last", "shell_in_place"])
+def test_native_step_on_a_list_with_a_skin(cabi, relabel):
+    """A neighbour list built out to cutoff + skin, at a size where the forward runs the LDS-table kernel: the step walks
+    each receiver's edges only up to its last pair inside the cutoff (with relabelling the shell pairs sit at the end of
+    every segment, without it they stay where the list has them).  Features and node energies equal the autograd path's on
+    the same list bit for bit (a pair beyond the cutoff adds an exact zero there), energy and forces equal the exact
+    list's up to the order of the sums."""
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.utils.neighbour_list import neighbour_data
+
+    n, C = 2600, 64
+    base = to_device(make_system(n, 4, seed=21, density=0.1), "cuda")
+    avg = base["edge_index"].shape[1] / n
+    up = SyntheticInvariantMACE(channels=C, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=avg, seed=9)
+    kwargs = dict(spatial_order_min_atoms=0) if relabel else dict(spatial_order_min_atoms=None)
+    native = OptimizedInvariantMACE(up, device="cuda", native_step=True, **kwargs)
+    eager = OptimizedInvariantMACE(up, device="cuda", native_step=False, **kwargs)
+    pbc = (True, True, True)
+    wide = neighbour_data(base["positions"].clone(), base["node_attrs"], 5.6, pbc, base["cell"])
+    exact = neighbour_data(base["positions"].clone(), base["node_attrs"], 5.0, pbc, base["cell"])
+    assert wide["edge_index"].shape[1] > 1.3 * exact["edge_index"].shape[1]
+    a, b, c = native(dict(wide)), eager(dict(wide)), native(dict(exact))
+    assert native._native not in (None, False) and eager._native is None
+    _say("  skin list (%s): E %.12g, exact list %.12g" % ("relabelled" if relabel else "as built", float(a["energy"].sum()),
+                                                         float(c["energy"].sum())))
+    assert torch.equal(a["node_feats"], b["node_feats"].detach()) and torch.equal(a["node_energy"], b["node_energy"].detach())
+    fscale = float(c["forces"].abs().max())
+    torch.testing.assert_close(a["forces"], b["forces"].detach(), rtol=0, atol=5e-7 * fscale)
+    torch.testing.assert_close(a["energy"], c["energy"], rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(a["forces"], c["forces"], rtol=0, atol=2e-6 * fscale)
