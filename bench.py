@@ -541,10 +541,11 @@ def main():
     torch.cuda.synchronize()
     md_loop = None if not md_steps else {
                "ms_per_step": round(1e3 * (time.perf_counter() - t_md) / md_steps, 4), "steps": md_steps,
-               "list_rebuilds": calc.builds - builds0, "skin_A": 0.5, "move_per_step_A": 0.02,
+               "list_rebuilds": calc.builds - builds0, "steps_enqueued_twice": calc.dropped, "skin_A": 0.5, "move_per_step_A": 0.02,
                "hip_graph": calc.use_graph,
                "note": "energy+forces through DeviceCalculator incl. neighbour-list rebuilds on the device; the list holds "
-                       "(1 + skin/cutoff)^3 = 1.33x the pairs of the exact list"}
+                       "(1 + skin/cutoff)^3 = 1.33x the pairs of the exact list; the host reads the displacement test "
+                       "after it has enqueued the step (a step on a list found stale is enqueued again)"}
 
     configs = None
     if not args.no_extras:

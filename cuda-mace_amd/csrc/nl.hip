@@ -377,8 +377,47 @@ __global__ __launch_bounds__(256) void nl_rank_kernel(const int32_t *__restrict_
   }
 }
 
+// ---- the test a Verlet list needs before it is reused: how far has any atom moved since the list was built ----
+__global__ void clear_u64_kernel(unsigned long long *out) { *out = 0ull; }
+
+// Non-negative doubles order like their bit patterns, so the maximum over the grid is an integer atomic.
+__global__ __launch_bounds__(256) void max_displacement_kernel(const double *__restrict__ positions,
+                                                               const double *__restrict__ reference, int64_t nnodes,
+                                                               unsigned long long *__restrict__ out) {
+#pragma clang fp contract(off)  // squares and sums as written, like the accept test of the list itself
+  double worst = 0.0;
+  for (int64_t n = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; n < nnodes;
+       n += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const double d0 = positions[3 * n + 0] - reference[3 * n + 0];
+    const double d1 = positions[3 * n + 1] - reference[3 * n + 1];
+    const double d2 = positions[3 * n + 2] - reference[3 * n + 2];
+    const double r2 = d0 * d0 + d1 * d1 + d2 * d2;
+    worst = r2 > worst ? r2 : worst;  // a NaN coordinate is caught below
+    if (!(r2 == r2)) worst = __builtin_inf();
+  }
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    const double other = __shfl_down(worst, off);
+    worst = other > worst ? other : worst;
+  }
+  if (threadIdx.x % kWave == 0) atomicMax(out, static_cast<unsigned long long>(__double_as_longlong(worst)));
+}
+
 }  // namespace
 }  // namespace cm
+
+extern "C" int cm_max_displacement(const double *positions, const double *reference, int64_t nnodes, double *out_sq,
+                                   cm_stream_t stream) {
+  CM_REQUIRE(nnodes >= 0, "cm_max_displacement: negative size");
+  CM_REQUIRE(out_sq && (nnodes == 0 || (positions && reference)), "cm_max_displacement: NULL pointer");
+  hipStream_t st = cm::as_stream(stream);
+  unsigned long long *out = reinterpret_cast<unsigned long long *>(out_sq);
+  hipLaunchKernelGGL(cm::clear_u64_kernel, dim3(1), dim3(1), 0, st, out);
+  if (nnodes > 0) {
+    const unsigned blocks = static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(nnodes, 256), 1024));
+    hipLaunchKernelGGL(cm::max_displacement_kernel, dim3(blocks), dim3(256), 0, st, positions, reference, nnodes, out);
+  }
+  return cm::check_launch("cm_max_displacement");
+}
 
 extern "C" size_t cm_neighbour_list_workspace(int64_t nnodes, int64_t max_cells) {
   if (nnodes < 0 || max_cells < 1) return 0;

@@ -67,6 +67,7 @@ SIGNATURES = {
     "cm_neighbour_list_workspace": (_sz, [_i64, _i64]),
     "cm_neighbour_list_count": (_i32, [_p, _p, _i32, _i32, _i32, _f64, _i64, _i64, _p, _sz, _p, _p, _p]),
     "cm_neighbour_list_fill": (_i32, [_p, _f64, _i64, _i64, _p, _p, _i64, _p, _p, _p, _p, _p]),
+    "cm_max_displacement": (_i32, [_p, _p, _i64, _p, _p]),
     # the whole step: (weights struct *, graph struct *, positions, shifts, workspace, bytes, 4 outputs, stream)
     "cm_mace_step_timing": (_i32, [ctypes.c_uint]),
     "cm_mace_step_timing_read": (_i32, [_p, _p, _i32]),
@@ -555,6 +556,19 @@ def neighbour_list(positions, cell, pbc, cutoff: float, max_cells: int = 0):
             )
         )
     return row_i, row_j, S
+
+
+def max_displacement(positions, reference, out=None):
+    """fp64 [1] on the device: the largest squared distance between the rows of `positions` and `reference` (fp64
+    [N, 3]); nothing is read back here."""
+    N = positions.shape[0]
+    if reference.shape != positions.shape:
+        raise CudaMaceError("max_displacement: positions and reference differ in shape")
+    if out is None:
+        out = torch.empty(1, dtype=F64, device=positions.device)
+    _check(lib.cm_max_displacement(_dev(positions, F64, "positions"), _dev(reference, F64, "reference"), N,
+                                   _dev(out, F64, "out"), _stream()))
+    return out
 
 
 # ---- readouts -------------------------------------------------------------------------------------

@@ -376,6 +376,17 @@ int cm_neighbour_list_fill(const double *positions, double cutoff, int64_t nnode
                            const void *workspace, const int32_t *offsets, int64_t nedges, int32_t *edge_scratch,
                            int32_t *row_i, int32_t *row_j, int32_t *unit_shifts, cm_stream_t stream);
 
+/*
+ * The test a molecular-dynamics driver makes before it reuses a list built out to cutoff + skin: out_sq[0] (fp64,
+ * device memory) = the largest squared distance between an atom's row of `positions` and of `reference` (the
+ * positions the list was built from), both fp64 [nnodes, 3]; +inf when a coordinate is NaN, 0 without atoms.  The
+ * list stays valid while that is at most (skin / 2)^2.  No counterpart in the reference, which leaves the list to
+ * its callers (tests/test_utils.py:62-105 rebuild it on the host for every evaluation).  Two small launches, no
+ * workspace, nothing read back.
+ */
+int cm_max_displacement(const double *positions, const double *reference, int64_t nnodes, double *out_sq,
+                        cm_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Readouts of the two-layer invariant model, scale / shift and their derivative in one pass, fp64 arithmetic on the
  * fp32 node features.  Replaces the upstream readout modules the reference keeps in fp64 and the casts around them

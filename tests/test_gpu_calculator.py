@@ -43,6 +43,48 @@ def test_md_like_walk(cabi, use_graph):
     assert 1 < calc.builds < 25 and calc.steps == 25
 
 
+def test_running_ahead_of_the_displacement_test(cabi):
+    """The step is enqueued before the host has read how far the atoms have moved; a step that ran on a list which turns
+    out stale is enqueued again on a fresh one.  Small moves first (the calculator learns how fast the largest
+    displacement grows and starts to run ahead), then one atom jumps further than half the skin: the result of that
+    step equals the model's on an exact list, and one step was dropped.  With run_ahead=False nothing is dropped and the
+    results are the same."""
+    from cuda_mace.calculators import DeviceCalculator
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.utils.neighbour_list import neighbour_data
+    from cuda_mace.utils.synthetic import make_system, to_device
+
+    n = 300
+    data = to_device(make_system(n, 4, seed=5, density=0.1), "cuda")
+    upstream = SyntheticInvariantMACE(channels=32, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=data["edge_index"].shape[1] / n,
+                                      seed=6)
+    model = OptimizedInvariantMACE(upstream, device="cuda")
+    pbc = (True, True, True)
+    results = {}
+    for run_ahead in (True, False):
+        calc = DeviceCalculator(model, data["node_attrs"], cutoff=5.0, skin=0.4, pbc=pbc, cell=data["cell"], use_graph=False,
+                                run_ahead=run_ahead)
+        g = torch.Generator(device="cuda").manual_seed(3)
+        pos = data["positions"].clone()
+        outs = []
+        for it in range(6):
+            step = 1e-3 * torch.randn(pos.shape, device="cuda", dtype=pos.dtype, generator=g)
+            if it == 4:
+                step[17, 0] += 0.3  # further than skin / 2 in one step
+            pos = pos + step
+            got = calc.compute(pos)
+            exact = model(neighbour_data(pos.clone(), data["node_attrs"], 5.0, pbc, data["cell"]))
+            scale = float(exact["forces"].abs().max())
+            torch.testing.assert_close(got["energy"], exact["energy"].detach(), rtol=1e-7, atol=1e-7)
+            torch.testing.assert_close(got["forces"], exact["forces"].detach(), rtol=0, atol=2e-6 * scale)
+            outs.append((got["energy"].clone(), got["forces"].clone()))
+        assert calc.builds == 2 and calc.steps == 6
+        assert calc.dropped == (1 if run_ahead else 0)
+        results[run_ahead] = outs
+    for (ea, fa), (eb, fb) in zip(results[True], results[False]):
+        assert torch.equal(ea, eb) and torch.equal(fa, fb)
+
+
 class _Atoms:
     """The four accessors of ase.Atoms that a calculator reads."""
 

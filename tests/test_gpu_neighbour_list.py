@@ -111,3 +111,19 @@ def test_full_size_box_equals_host_list_and_feeds_the_model(cabi):
     out_dev = model(dev2)
     assert torch.equal(out_host["energy"], out_dev["energy"])
     assert torch.equal(out_host["forces"], out_dev["forces"])
+
+
+@pytest.mark.parametrize("n", [0, 1, 63, 1000, 300_001])
+def test_max_displacement(cabi, n):
+    """cm_max_displacement against the same maximum taken by torch in fp64 (bit-exact: squares and sums of three terms,
+    left to right without fused multiply-adds, then a maximum); a NaN coordinate gives +inf."""
+    g = torch.Generator(device="cuda").manual_seed(n)
+    ref = 20.0 * torch.rand(n, 3, device="cuda", dtype=torch.float64, generator=g)
+    pos = ref + 0.1 * torch.randn(n, 3, device="cuda", dtype=torch.float64, generator=g)
+    got = cabi.max_displacement(pos, ref)
+    d = pos - ref
+    want = (d[:, 0] * d[:, 0] + d[:, 1] * d[:, 1] + d[:, 2] * d[:, 2]).max() if n else torch.zeros((), dtype=torch.float64)
+    assert got.shape == (1,) and float(got[0]) == float(want)
+    if n:
+        pos[n // 2, 1] = float("nan")
+        assert float(cabi.max_displacement(pos, ref, out=got)[0]) == float("inf")
