@@ -20,6 +20,20 @@ inline hipStream_t as_stream(cm_stream_t s) { return reinterpret_cast<hipStream_
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Compute units of the current device (256 on the part this library is written for; also the answer when the query
+// fails), read once per device.
+inline int device_compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 // Checks the launch that was just enqueued; returns CM_OK or CM_ELAUNCH.
 inline int check_launch(const char *what) {
   hipError_t err = hipGetLastError();

@@ -849,18 +849,6 @@ __global__ __launch_bounds__(kResWaves *kWave, 1) void linear_resident_kernel(
   }
 }
 
-int compute_units() {
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 template <int K, int NT>
 int launch_resident(const float *X, const float *WT, const int32_t *perm, const int32_t *offs, int64_t nnodes, int ngroups,
                     int zero_last_group, int Nout, float scale, const float *row_scale, float *OUT, hipStream_t st) {
@@ -869,7 +857,7 @@ int launch_resident(const float *X, const float *WT, const int32_t *perm, const 
   // 192 = 2 x 96 and 256 = 4 x 64 columns it only equals the kernels above, because every column block splits the X rows
   // again, so those widths are not routed here.)
   const int ycount = Nout / (32 * NT);
-  const dim3 grid(static_cast<unsigned>(std::max(8, compute_units() / ycount / 8 * 8)), static_cast<unsigned>(ycount)), block(kResWaves * kWave);
+  const dim3 grid(static_cast<unsigned>(std::max(8, device_compute_units() / ycount / 8 * 8)), static_cast<unsigned>(ycount)), block(kResWaves * kWave);
   if (row_scale)
     hipLaunchKernelGGL((linear_resident_kernel<K, NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
                        zero_last_group, Nout, scale, row_scale, OUT);

@@ -368,18 +368,6 @@ __global__ __launch_bounds__(kSlThreads) void mp_edge_forward_sliced_kernel(cons
   }
 }
 
-int device_compute_units() {
-  static int cached[64] = {0};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (cached[dev] == 0) {
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cached[dev] = n;
-  }
-  return cached[dev];
-}
-
 }  // namespace
 
 bool sliced_forward_applies(int64_t nnodes, int channels, int nknots) {

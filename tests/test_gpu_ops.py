@@ -245,7 +245,10 @@ def test_sh_forward_backward(cabi, E, seed):
 # ------------------------------------------------------------------------------------------------
 # spline
 # ------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("E,J,seed", [(1, 128, 0), (777, 384, 1), (5000, 512, 2), (300, 768, 3)])
+# from 32 768 edges on the forward without derivative and the backward run on their LDS-table kernels: full rows of
+# slices, a last slice of 8 of 32 outputs, and more edges than one pass of chunks holds (256 workgroups x 8 192)
+@pytest.mark.parametrize("E,J,seed", [(1, 128, 0), (777, 384, 1), (5000, 512, 2), (300, 768, 3), (40_000, 512, 4),
+                                      (70_001, 72, 5), (2_200_003, 8, 6)])
 def test_spline_forward_backward(cabi, E, J, seed):
     _say("spline", E, J, seed)
     g = torch.Generator().manual_seed(seed)
@@ -269,8 +272,10 @@ def test_spline_forward_backward(cabi, E, J, seed):
     assert torch.equal(val, val_only)
     close(val, val_ref, 2e-5, 2e-6)
     close(der, der_ref, 2e-5, 5e-6)
-    # a sum of J signed terms: the error bound scales with the sum of their magnitudes
-    bound = 2e-6 * (gR.abs() * der_ref.abs()).sum(-1) + 1e-30
+    # a sum of J signed terms: the error bound scales with the sum of their magnitudes (5e-6: over millions of edges with
+    # only 8 outputs the cancellations inside b + 2 c x + 3 d x^2, x in fp32, reach 2.1 times the 2e-6 that a few
+    # thousand edges stay within, in the direct kernel and in the LDS-table kernel alike)
+    bound = 5e-6 * (gR.abs() * der_ref.abs()).sum(-1) + 1e-30
     assert bool(((gr.double().cpu() - gr_ref).abs() <= bound).all())
     assert float(val[(r32 > r_max).to(DEV)].abs().sum()) == 0.0
 
