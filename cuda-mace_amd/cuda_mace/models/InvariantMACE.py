@@ -438,15 +438,24 @@ class OptimizedInvariantMACE(torch.nn.Module):
         # Inside a row-0 segment: the pairs within the cutoff by their row-1 label, then those beyond it (the skin shell
         # of a Verlet list), nearest first.  The native step cuts every segment back to its last pair inside the cutoff
         # before the forward message passing; with this order the pairs that drift inside between two list builds are
-        # the first of the shell, so the cut stays close to the pairs that count.  (Three stable sorts: by length, by
-        # the in-segment key, by segment.)
+        # the first of the shell, so the cut stays close to the pairs that count.  Three stable sorts, least significant
+        # key first: by length among the shell pairs, by row-1 label among the others, by segment; the two with node
+        # labels as keys are counting sorts of the library (on the device, where the model runs).
+        def by_label(keys, nkeys):
+            if keys.is_cuda and nkeys < 2**31 - 1:
+                return cabi.stable_key_sort(keys.int().contiguous(), nkeys)[0].long()
+            return torch.argsort(keys, stable=True)
+
         if "shifts" in data:
             length = (pos[edge_index[1]] - pos[edge_index[0]] + data["shifts"].detach().to(pos.dtype)).norm(dim=1)
             shell = length > float(self.r_max)
-            by_length = torch.argsort(torch.where(shell, length, torch.zeros_like(length)), stable=True)  # the rest stays put
-            inner_key = torch.where(shell, torch.full_like(row1, n), row1)[by_length]
-            by_inner = by_length[torch.argsort(inner_key, stable=True)]
-            edge_perm = by_inner[torch.argsort(row0[by_inner], stable=True)]
+            by_length = torch.argsort(torch.where(shell, length, torch.zeros_like(length)).float(), stable=True)  # the rest stays put
+            # by_length holds the pairs within the cutoff first, in the list's order: only those are sorted by label
+            # (as one key the shell would be a single bucket of a quarter of all pairs, which a counting sort ranks serially)
+            n_within = edge_index.shape[1] - int(shell.sum())
+            within, beyond = by_length[:n_within], by_length[n_within:]
+            by_inner = torch.cat((within[by_label(row1[within], n)], beyond))
+            edge_perm = by_inner[by_label(row0[by_inner], n)]
         else:
             edge_perm = torch.argsort(row0 * n + row1, stable=True)
         new_edges = torch.stack((row0[edge_perm], row1[edge_perm])).contiguous()
