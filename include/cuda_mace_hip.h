@@ -74,6 +74,10 @@ int cm_receiver_list_status(const int32_t *receiver, int64_t nedges, int64_t nno
  * jit_elemental_linear (jit_wrappers/src/linear_wrapper.cpp:137-145).
  *   keys int32 [n] in [0, nkeys); perm int32 [n]; offsets int32 [nkeys + 1];
  *   workspace: cm_stable_key_sort_workspace(n, nkeys) bytes of device memory.
+ * Cost: linear in n up to 64 keys (any bucket size).  Above 64 keys the items of a bucket are ranked by comparing
+ * them with each other, so the cost also grows with the square of the largest bucket: meant for neighbour lists,
+ * where a bucket is one atom's edges (tens of items; 1.3 million edges over 25 000 senders take 0.1 ms), not for
+ * keys that put a large part of the items into one bucket (430 000 of 1.7 million items in one bucket: 25 ms).
  */
 size_t cm_stable_key_sort_workspace(int64_t n, int64_t nkeys);
 int cm_stable_key_sort(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm,
