@@ -458,7 +458,11 @@ def main():
                                          "products and 16 accumulations",
                              "flops": flops_fwd, "achieved_TFLOP/s": round(flops_fwd / (t_fwd * 1e-3) / 1e12, 1),
                              "peak_TFLOP/s": 157.3, "frac": round(flops_fwd / (t_fwd * 1e-3) / 1e12 / 157.3, 4),
-                             "meaning": "useful fp32 operations of the formulation against the vector peak; the kernel issues "
+                             "frac_of_unpacked_rate": round(flops_fwd / (t_fwd * 1e-3) / 1e12 / 78.65, 4),
+                             "meaning": "useful fp32 operations of the formulation against the vector peak (which counts "
+                                        "two-wide packed fp32 instructions; this library is built without them, so one "
+                                        "FMA per lane and four cycles, 78.65 TFLOP/s, is the rate its instructions can "
+                                        "reach: frac_of_unpacked_rate); the kernel issues "
                                         "about 1.8 instructions per useful one (edge set-up per quad of lanes, broadcasts of "
                                         "the edge's values, addresses), and instructions with a cross-lane operand issue at "
                                         "less than half the rate of plain ones on this device"},
