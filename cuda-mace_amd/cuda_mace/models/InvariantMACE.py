@@ -476,7 +476,10 @@ class OptimizedInvariantMACE(torch.nn.Module):
         # Without strain the positions stay in the caller's order: the geometry kernels read them (and write the forces)
         # through the row map.  The strain path transforms positions per graph and works on a gathered copy.
         direct = not (compute_virials or compute_stress or compute_displacement)
-        inner["positions"] = data["positions"].detach() if direct else data["positions"].detach().index_select(0, perm)
+        # With compute_force=False the caller differentiates the returned energies itself (a wrapper that sums the
+        # energies of some atoms only): the positions then stay attached to the caller's tensor.
+        own = data["positions"].detach() if compute_force else data["positions"]
+        inner["positions"] = own if direct else own.index_select(0, perm)
         inner["edge_index"], inner["batch"] = edge_index, batch
         inner["node_attrs"] = _cached_for(data["edge_index"], "_cm_spatial_attrs", data["node_attrs"],
                                           lambda: data["node_attrs"].index_select(0, perm))

@@ -78,8 +78,11 @@ def contraction_nested(X, elem, W3, W2, W1, U3, U2):
 
 
 def energy_and_forces(params: Dict[str, object], data: Dict[str, torch.Tensor], dtype=torch.float64,
-                      compute_forces: bool = True, edge_chunk: Optional[int] = None):
-    """Returns dict(energy [1], interaction_energy [1], node_energy [N], forces [N, 3], node_feats [N, 2C])."""
+                      compute_forces: bool = True, edge_chunk: Optional[int] = None,
+                      node_weights: Optional[torch.Tensor] = None):
+    """Returns dict(energy [1], interaction_energy [1], node_energy [N], forces [N, 3], node_feats [N, 2C]).
+    With node_weights [N] the forces are minus the gradient of sum_n node_weights[n] * node_energy[n] (what a rank of
+    a domain-decomposed MD code reports: weight 1 for its own atoms, 0 for ghosts); energies are unweighted."""
     C = int(params["channels"])
     ne = int(params["num_elements"])
     pos = data["positions"].detach().to(dtype).clone().requires_grad_(compute_forces)
@@ -127,7 +130,8 @@ def energy_and_forces(params: Dict[str, object], data: Dict[str, torch.Tensor], 
     inter_e = node_inter.sum().view(1)
     forces = None
     if compute_forces:
-        (g,) = torch.autograd.grad(inter_e.sum(), pos)
+        seeded = inter_e.sum() if node_weights is None else (node_inter * node_weights.to(dtype)).sum()
+        (g,) = torch.autograd.grad(seeded, pos)
         forces = -g
     return dict(energy=(node_e0.sum() + inter_e).detach(), interaction_energy=inter_e.detach(),
                 node_energy=(node_e0 + node_inter).detach(), forces=forces,

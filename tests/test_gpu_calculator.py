@@ -85,6 +85,45 @@ def test_running_ahead_of_the_displacement_test(cabi):
         assert torch.equal(ea, eb) and torch.equal(fa, fb)
 
 
+@pytest.mark.parametrize("relabel", [False, True], ids=["as_given", "relabelled"])
+def test_lammps_style_wrapper(cabi, relabel):
+    """LAMMPS_MACE (upstream's interface for a domain-decomposed MD code): the energy of the rank's own atoms and minus
+    its gradient with respect to every atom, ghosts included, against the fp64 reference model seeded with the same
+    mask; with every atom local it equals the model's own energy, forces and virials."""
+    from oracle import mace_model as M
+
+    from cuda_mace.calculators import LAMMPS_MACE
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.utils.synthetic import make_system, to_device
+
+    n = 320
+    data = make_system(n, 4, seed=31, density=0.1)
+    upstream = SyntheticInvariantMACE(channels=32, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=data["edge_index"].shape[1] / n,
+                                      seed=32, atomic_energies=torch.linspace(-2.0, -1.0, 4, dtype=torch.float64))
+    params = upstream.export_params()
+    model = OptimizedInvariantMACE(upstream, device="cuda", spatial_order_min_atoms=0 if relabel else None)
+    wrapper = LAMMPS_MACE(model)
+    dev = to_device(data, "cuda")
+    local = (torch.rand(n, generator=torch.Generator().manual_seed(33)) < 0.6).double()
+    got = wrapper(dict(dev), local.cuda())
+    ref = M.energy_and_forces(params, data, node_weights=local)
+    e_ref = float((ref["node_energy"] * local).sum())
+    assert abs(float(got["total_energy_local"].sum()) - e_ref) <= 1e-5 * abs(e_ref)
+    assert float((got["forces"].double().cpu() - ref["forces"]).abs().max()) <= 1e-4
+    assert float((got["node_energy"].double().cpu() - ref["node_energy"]).abs().max()) <= 1e-5 * float(ref["node_energy"].abs().max())
+    # the masked forces are not the forces of the whole system (the mask matters) ...
+    whole = M.energy_and_forces(params, data)
+    assert float((ref["forces"] - whole["forces"]).abs().max()) > 1e-2
+    # ... and with every atom local the wrapper reproduces the model's own outputs
+    every = wrapper(dict(dev), torch.ones(n, device="cuda"), compute_virials=True)
+    own = model(dict(dev), compute_virials=True)
+    scale = float(own["forces"].abs().max())
+    torch.testing.assert_close(every["total_energy_local"], own["energy"].detach(), rtol=1e-9, atol=1e-9)
+    torch.testing.assert_close(every["forces"], own["forces"].detach(), rtol=0, atol=2e-6 * scale)
+    torch.testing.assert_close(every["virials"], own["virials"].detach(), rtol=0, atol=2e-6 * float(own["virials"].abs().max()))
+    assert got["virials"] is None and every["virials"].shape == (1, 3, 3)
+
+
 class _Atoms:
     """The four accessors of ase.Atoms that a calculator reads."""
 
