@@ -82,12 +82,20 @@ __global__ void fill_f64_kernel(double *p, int64_t n, double value) {
     p[i] = value;
 }
 
-// g1[n, c] = -scale * w1[c]: the gradient of -sum(node energies) with respect to the first layer's features (the linear
-// readout), the same row for every node
-__global__ void seed_linear_readout_kernel(float *__restrict__ g1, const double *__restrict__ w1, double scale, int64_t total, int C) {
+// g1[n, c] = -weight[n] * scale * w1[c]: the gradient of -sum(weight * node energies) with respect to the first layer's
+// features (the linear readout); without weights the same row for every node
+__global__ void seed_linear_readout_kernel(float *__restrict__ g1, const double *__restrict__ w1, double scale,
+                                           const double *__restrict__ node_weights, int64_t total, int C) {
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x)
-    g1[i] = static_cast<float>(-1.0 * scale * w1[i % C]);
+    g1[i] = static_cast<float>(-1.0 * scale * w1[i % C] * (node_weights ? node_weights[i / C] : 1.0));
+}
+
+// rows of x [nnodes, C] times the node's weight (the second readout's derivative, when node energies carry weights)
+__global__ void weight_rows_kernel(float *__restrict__ x, const double *__restrict__ node_weights, int64_t total, int C) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    x[i] = static_cast<float>(static_cast<double>(x[i]) * node_weights[i / C]);
 }
 
 // Edge range of every receiver node cut back to its last edge inside the cutoff: live[n] = first_occ[n],
@@ -124,12 +132,12 @@ __global__ void add_f32_kernel(float *__restrict__ a, const float *__restrict__ 
 // out[g] = sum of x over the nodes ptr[g] .. ptr[g + 1]: one workgroup per graph, every thread a strided partial sum, a
 // tree over the partials: the same order on every run.
 constexpr int kSumThreads = 1024;
-__global__ __launch_bounds__(kSumThreads) void segment_sum_f64_kernel(const double *__restrict__ x, const int32_t *__restrict__ ptr,
-                                                                     double *__restrict__ out) {
+__global__ __launch_bounds__(kSumThreads) void segment_sum_f64_kernel(const double *__restrict__ x, const double *__restrict__ weights,
+                                                                     const int32_t *__restrict__ ptr, double *__restrict__ out) {
   __shared__ double part[kSumThreads];
   const int lo = ptr[blockIdx.x], hi = ptr[blockIdx.x + 1];
   double s = 0.0;
-  for (int i = lo + threadIdx.x; i < hi; i += kSumThreads) s += x[i];
+  for (int i = lo + threadIdx.x; i < hi; i += kSumThreads) s += weights ? weights[i] * x[i] : x[i];
   part[threadIdx.x] = s;
   __syncthreads();
   for (int d = kSumThreads / 2; d > 0; d >>= 1) {
@@ -281,17 +289,21 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   }
   CM_STAGE(11, cm_readout_forward(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden, node_energy,
                              L.d_h2, node_feats, g->node_rows, stream));
-  hipLaunchKernelGGL(cm::segment_sum_f64_kernel, dim3(g->ngraphs), dim3(cm::kSumThreads), 0, st, node_energy, g->graph_ptr,
-                     interaction_energy);
+  hipLaunchKernelGGL(cm::segment_sum_f64_kernel, dim3(g->ngraphs), dim3(cm::kSumThreads), 0, st, node_energy, g->node_weights,
+                     g->graph_ptr, interaction_energy);
 
   // ---- backward: d(-sum of node energies) / d positions ----
-  // The seed is -1 on every node energy, so the readouts' backward needs no pass of its own: the gradient with respect to
-  // the second layer's features is -d_h2 (the sign goes into the scale of the two linears that consume it, which is
-  // exact), the one with respect to the first layer's is a constant row.
+  // The seed is -1 on every node energy (-weight[n] with node weights), so the readouts' backward needs no pass of its
+  // own: the gradient with respect to the second layer's features is -d_h2 (the sign goes into the scale of the two
+  // linears that consume it, which is exact; node weights scale its rows first), the one with respect to the first
+  // layer's is a constant row (times the node's weight).
   {
     cm::StageTimer timer_(st, 13, timing_mask);
-    hipLaunchKernelGGL(cm::seed_linear_readout_kernel, dim3(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(N * C, 256), 2048))),
-                       dim3(256), 0, st, L.g1, w->w1, w->scale, static_cast<int64_t>(N) * C, C);
+    const dim3 grid(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(N * C, 256), 2048)));
+    hipLaunchKernelGGL(cm::seed_linear_readout_kernel, grid, dim3(256), 0, st, L.g1, w->w1, w->scale, g->node_weights,
+                       static_cast<int64_t>(N) * C, C);
+    if (g->node_weights)
+      hipLaunchKernelGGL(cm::weight_rows_kernel, grid, dim3(256), 0, st, L.d_h2, g->node_weights, static_cast<int64_t>(N) * C, C);
   }
   // layer 1 (second interaction)
   CM_STAGE(14, cm_linear(L.d_h2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, -1.0f, none, none, L.gB, stream));

@@ -8,8 +8,9 @@ code adds the ghosts' shares back to their owners).  This is the wrapper upstrea
 (mace/calculators/lammps_mace.py, class LAMMPS_MACE: same constructor, call signature and result keys); the reference
 itself stops at the model (tools/model_surgery.py:217-229) and has no counterpart.
 
-The backward seed is a per-atom mask, not one per graph, so the step goes through the autograd path of the model (the
-library's one-call step seeds every node energy alike).
+With this package's model the mask travels as data["node_weights"], which the library's one-call step takes as the
+seed of every node energy, so the wrapper costs what the plain model costs.  Any other model with the same forward
+signature (upstream's own) is driven as upstream's wrapper drives it: node energies out, autograd from here.
 """
 from __future__ import annotations
 
@@ -38,6 +39,11 @@ class LAMMPS_MACE(torch.nn.Module):
         num_graphs = data["ptr"].numel() - 1
         if self.head is not None:
             data["head"] = torch.full((num_graphs,), int(self.head), dtype=torch.int64, device=data["positions"].device)
+        if getattr(self.model, "supports_node_weights", False):
+            data["node_weights"] = local_or_ghost.to(torch.float64)
+            out = self.model(data, training=False, compute_force=True, compute_virials=compute_virials, compute_stress=False)
+            return {"total_energy_local": out["energy"].detach(), "node_energy": out["node_energy"].detach(),
+                    "forces": out["forces"].detach(), "virials": out["virials"].detach() if compute_virials else None}
         positions = data["positions"]
         if not positions.requires_grad:
             positions = positions.detach().requires_grad_(True)

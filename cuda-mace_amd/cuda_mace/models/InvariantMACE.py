@@ -303,6 +303,9 @@ class _WeightsToken:
 
 
 class OptimizedInvariantMACE(torch.nn.Module):
+    # forward() honours data["node_weights"] (see _forward_ordered); wrappers that need per-atom seeds check for this
+    supports_node_weights = True
+
     def __init__(self, mace_model: torch.nn.Module, device="cuda", num_spline_knots: int = 256, fused_radial: bool = True,
                  fused_readout: bool = True, fused_contraction: bool = True, spatial_order_min_atoms: Optional[int] = 8192,
                  native_step: bool = True):
@@ -487,6 +490,9 @@ class OptimizedInvariantMACE(torch.nn.Module):
             if name in data:
                 t = data[name]
                 inner[name] = _cached_for(data["edge_index"], "_cm_spatial_" + name, t, lambda t=t: t.index_select(0, edge_perm))
+        if data.get("node_weights") is not None:
+            t = data["node_weights"]
+            inner["node_weights"] = _cached_for(data["edge_index"], "_cm_spatial_node_weights", t, lambda: t.index_select(0, perm))
         rows = _cached(data["edge_index"], "_cm_spatial_rows32", None, lambda: (perm.int(), inverse))
         out = self._forward_ordered(inner, training, compute_force, compute_virials, compute_stress, compute_displacement,
                                     node_rows=rows, positions_in_caller_order=direct)
@@ -529,7 +535,14 @@ class OptimizedInvariantMACE(torch.nn.Module):
 
         e0_per_head, node_feats_up = _cached_for(node_attrs, "_cm_species_only", self._weights_token, species_only)
         node_e0 = _select_head(e0_per_head, zero_heads if node_heads is None else node_heads)
-        if num_graphs == 1 and node_heads is None:
+        # data["node_weights"] [N] (optional): every node energy enters the graph's energy, and hence the quantity the
+        # forces, virials and stress derive from, with this weight (1 for a rank's own atoms, 0 for ghost copies in a
+        # domain-decomposed MD code); node_energy itself stays unweighted.
+        node_weights = data.get("node_weights")
+        if node_weights is not None:
+            node_weights = node_weights.detach().to(torch.float64)
+            e0 = scatter_sum(src=node_e0 * node_weights, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
+        elif num_graphs == 1 and node_heads is None:
             # one graph: the sum of the atomic reference energies is a function of the species tensor alone, too
             e0 = _cached_for(node_attrs, "_cm_e0_sum", self._weights_token, lambda: node_e0.sum(dim=0, keepdim=True))
         else:
@@ -554,6 +567,10 @@ class OptimizedInvariantMACE(torch.nn.Module):
                 handle = _cached_for(edge_index, "_cm_native_graph_%d" % id(self._weights_token), node_attrs,
                                      lambda: native.graph(edge_index, receiver, sender, node_attrs32, atom_types, data["ptr"],
                                                           node_feats_up, rows32))
+                if node_weights is not None:
+                    plain = handle
+                    handle = _cached_for(data["node_weights"], "_cm_native_graph_weighted_%d" % id(self._weights_token), plain,
+                                         lambda: plain.with_node_weights(node_weights))
                 res = native(handle, positions, shifts)
                 inter_e = res["interaction_energy"]
                 return {
@@ -607,7 +624,8 @@ class OptimizedInvariantMACE(torch.nn.Module):
                 node_feats_out = node_feats_out.index_select(0, node_rows[1])
             node_inter_es = torch.sum(torch.stack(node_es_list, dim=0), dim=0)
             node_inter_es = self.scale_shift(node_inter_es, zero_heads if node_heads is None else node_heads)
-        inter_e = scatter_sum(src=node_inter_es.double(), index=batch, dim=-1, dim_size=num_graphs, ptr=data["ptr"])
+        weighted_es = node_inter_es.double() if node_weights is None else node_inter_es.double() * node_weights
+        inter_e = scatter_sum(src=weighted_es, index=batch, dim=-1, dim_size=num_graphs, ptr=data["ptr"])
 
         total_energy = e0 + inter_e
         node_energy = node_e0 + node_inter_es

@@ -37,7 +37,7 @@ class _Graph(ctypes.Structure):
         ("nnodes", ctypes.c_int64), ("nedges", ctypes.c_int64), ("ngraphs", ctypes.c_int),
         ("receiver", _fp), ("sender", _fp), ("first_occ", _fp), ("sender_perm", _fp), ("sender_offsets", _fp),
         ("elem_perm", _fp), ("elem_offsets", _fp), ("onehot_perm", _fp), ("onehot_offsets", _fp),
-        ("node_rows", _fp), ("graph_ptr", _fp), ("X1", _fp),
+        ("node_rows", _fp), ("graph_ptr", _fp), ("X1", _fp), ("node_weights", _fp),
     ]
 
 
@@ -117,6 +117,7 @@ class NativeStep:
         g.onehot_perm, g.onehot_offsets = _ptr(operm, I32, "onehot_perm"), _ptr(ooff, I32, "onehot_offsets")
         g.node_rows = _ptr(node_rows, I32, "node_rows") if node_rows is not None else None
         g.graph_ptr, g.X1 = _ptr(ptr32, I32, "graph_ptr"), _ptr(X1, torch.float32, "X1")
+        g.node_weights = None
         return _GraphHandle(g, (receiver, sender, first_occ, sperm, soff, eperm, eoff, operm, ooff, ptr32, X1, node_rows))
 
     def __call__(self, handle: "_GraphHandle", positions: torch.Tensor, shifts: torch.Tensor, want_feats: bool = True) -> Dict[str, torch.Tensor]:
@@ -146,3 +147,14 @@ class NativeStep:
 class _GraphHandle:
     def __init__(self, struct, keep):
         self.struct, self._keep = struct, keep
+
+    def with_node_weights(self, weights: torch.Tensor) -> "_GraphHandle":
+        """The same index structures with a weight per node energy (fp64 [nnodes], in the order of the lists): the step
+        then returns sum_n weights[n] * node_energy[n] per graph and minus its gradient."""
+        if weights.shape != (int(self.struct.nnodes),):
+            raise cabi.CudaMaceError("node weights must be [%d]" % int(self.struct.nnodes))
+        g = _Graph()
+        ctypes.memmove(ctypes.addressof(g), ctypes.addressof(self.struct), ctypes.sizeof(_Graph))
+        w = weights.detach().to(torch.float64).contiguous()
+        g.node_weights = _ptr(w, torch.float64, "node_weights")
+        return _GraphHandle(g, (self._keep, w))

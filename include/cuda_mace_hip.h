@@ -440,9 +440,13 @@ int cm_readout_backward(const double *grad_node_energies, const double *w1, cons
  *   node_rows int32 [nnodes] or NULL: atom n of the lists is row node_rows[n] of positions / forces / node_feats
  *   graph_ptr int32 [ngraphs + 1]: node range of every graph of the batch, in the order of the lists
  *   X1 fp32 [nnodes, C]: linear_up(node_embedding(species)) of the first layer
- * Per call: positions fp64 [nnodes, 3], shifts fp64 [nedges, 3]; outputs interaction_energy fp64 [ngraphs] (sum of the
- * node energies of each graph, in a fixed order), node_energy fp64 [nnodes] (interaction part, in list order), forces
- * fp64 [nnodes, 3] = -d(sum of energies)/d positions (rows of the caller when node_rows is given), node_feats fp64
+ *   node_weights fp64 [nnodes] (in the order of the lists) or NULL: weight of every node energy in interaction_energy
+ *     and in the quantity the forces derive from, sum_n node_weights[n] * node_energy[n]; what the rank of a
+ *     domain-decomposed MD code needs (1 for its own atoms, 0 for ghost copies: upstream MACE's LAMMPS wrapper,
+ *     mace/calculators/lammps_mace.py; the reference has no counterpart).  NULL is all ones, bit for bit.
+ * Per call: positions fp64 [nnodes, 3], shifts fp64 [nedges, 3]; outputs interaction_energy fp64 [ngraphs] ((weighted) sum
+ * of the node energies of each graph, in a fixed order), node_energy fp64 [nnodes] (interaction part, unweighted, in
+ * list order), forces fp64 [nnodes, 3] = -d(sum of interaction_energy)/d positions (rows of the caller when node_rows is given), node_feats fp64
  * [nnodes, 2C] or NULL.  workspace: cm_mace_step_workspace(nnodes, nedges, channels) bytes, 256-byte aligned; its
  * contents are scratch.  Nothing is allocated, so the call can be captured into a HIP graph.
  */
@@ -471,6 +475,7 @@ typedef struct cm_mace_graph {
   const int32_t *elem_perm, *elem_offsets, *onehot_perm, *onehot_offsets;
   const int32_t *node_rows, *graph_ptr;
   const float *X1;
+  const double *node_weights;
 } cm_mace_graph;
 
 /* Per-stage timing of cm_mace_step (off by default): with bit s of stage_mask set, stage s of every later step is

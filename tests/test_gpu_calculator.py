@@ -106,6 +106,19 @@ def test_lammps_style_wrapper(cabi, relabel):
     dev = to_device(data, "cuda")
     local = (torch.rand(n, generator=torch.Generator().manual_seed(33)) < 0.6).double()
     got = wrapper(dict(dev), local.cuda())
+    assert model._native not in (None, False)  # the mask went into the library's one-call step as node weights
+    # the route for models that know nothing of node weights (upstream's own): node energies out, autograd in the wrapper
+    model.supports_node_weights = False
+    try:
+        generic = wrapper(dict(dev), local.cuda())
+    finally:
+        del model.supports_node_weights
+    torch.testing.assert_close(generic["total_energy_local"], got["total_energy_local"], rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(generic["forces"], got["forces"], rtol=0, atol=5e-7 * float(got["forces"].abs().max()))
+    # all-ones weights are the unweighted step bit for bit
+    ones = dict(dev, node_weights=torch.ones(n, dtype=torch.float64, device="cuda"))
+    a, b = model(ones), model(dict(dev))
+    assert torch.equal(a["forces"], b["forces"]) and torch.equal(a["energy"], b["energy"])
     ref = M.energy_and_forces(params, data, node_weights=local)
     e_ref = float((ref["node_energy"] * local).sum())
     assert abs(float(got["total_energy_local"].sum()) - e_ref) <= 1e-5 * abs(e_ref)
