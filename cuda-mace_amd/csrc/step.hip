@@ -147,13 +147,76 @@ __global__ __launch_bounds__(kSumThreads) void segment_sum_f64_kernel(const doub
   if (threadIdx.x == 0) out[blockIdx.x] = part[0];
 }
 
+// Virials from the per-edge gradients the backward chain ends with: under a symmetric strain every edge vector becomes
+// vec + vec . strain, so -dE/d strain = 1/2 sum_e (vec_e (x) gv_e + gv_e (x) vec_e) with gv_e = -dE/d vec_e, which is what
+// the chain delivers.  Two levels, both in a fixed order: per receiver node (eight lanes share a node's edges), then per
+// graph.  node_virial [nnodes, 6]: xx, yy, zz, yz, xz, xy.
+__global__ __launch_bounds__(256) void node_virial_kernel(const float *__restrict__ vec, const float *__restrict__ gv,
+                                                          const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges,
+                                                          double *__restrict__ node_virial) {
+  const int64_t t = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  const int n = static_cast<int>(t >> 3), sub = static_cast<int>(t & 7);
+  double acc[6] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+  if (n < nnodes) {
+    int e0 = first_occ[n], e1 = first_occ[nnodes + n];
+    clamp_edge_range(e0, e1, nedges);
+    for (int64_t e = e0 + sub; e < e1; e += 8) {
+      const double v0 = vec[3 * e + 0], v1 = vec[3 * e + 1], v2 = vec[3 * e + 2];
+      const double g0 = gv[3 * e + 0], g1 = gv[3 * e + 1], g2 = gv[3 * e + 2];
+      acc[0] += v0 * g0, acc[1] += v1 * g1, acc[2] += v2 * g2;
+      acc[3] += 0.5 * (v1 * g2 + v2 * g1), acc[4] += 0.5 * (v0 * g2 + v2 * g0), acc[5] += 0.5 * (v0 * g1 + v1 * g0);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 6; ++k) {
+    acc[k] += __shfl_xor(acc[k], 1);
+    acc[k] += __shfl_xor(acc[k], 2);
+    acc[k] += __shfl_xor(acc[k], 4);
+  }
+  if (n < nnodes && sub == 0) {
+#pragma unroll
+    for (int k = 0; k < 6; ++k) node_virial[6 * static_cast<int64_t>(n) + k] = acc[k];
+  }
+}
+
+// virials[g] (3 x 3, symmetric) = sum of node_virial over the graph's nodes; one workgroup per graph, strided partial sums
+// and a tree over them
+__global__ __launch_bounds__(kSumThreads) void graph_virial_kernel(const double *__restrict__ node_virial,
+                                                                   const int32_t *__restrict__ ptr, double *__restrict__ virials) {
+  __shared__ double part[6][kSumThreads];
+  const int lo = ptr[blockIdx.x], hi = ptr[blockIdx.x + 1];
+  double s[6] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+  for (int i = lo + threadIdx.x; i < hi; i += kSumThreads) {
+#pragma unroll
+    for (int k = 0; k < 6; ++k) s[k] += node_virial[6 * static_cast<int64_t>(i) + k];
+  }
+#pragma unroll
+  for (int k = 0; k < 6; ++k) part[k][threadIdx.x] = s[k];
+  __syncthreads();
+  for (int d = kSumThreads / 2; d > 0; d >>= 1) {
+    if (threadIdx.x < d) {
+#pragma unroll
+      for (int k = 0; k < 6; ++k) part[k][threadIdx.x] += part[k][threadIdx.x + d];
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    double *o = virials + 9 * static_cast<int64_t>(blockIdx.x);
+    o[0] = part[0][0], o[4] = part[1][0], o[8] = part[2][0];
+    o[5] = o[7] = part[3][0];
+    o[2] = o[6] = part[4][0];
+    o[1] = o[3] = part[5][0];
+  }
+}
+
 inline size_t align256(size_t n) { return (n + 255) & ~static_cast<size_t>(255); }
 
 // Carves the workspace; the same walk sizes it (base == nullptr) and lays it out.
 struct Layout {
   float *vec, *len, *gv1, *gv2, *bufM1, *bufM2, *bufA, *edge_scratch;
   float *B1, *h1, *sc, *X2, *B2, *h2, *d_h2, *g1, *gB, *gX2, *gh1a, *gh1;
-  int32_t *live;  // [2 N] edge ranges cut back to the last edge inside the cutoff
+  int32_t *live;         // [2 N] edge ranges cut back to the last edge inside the cutoff
+  double *node_virial;   // [N, 6]
   size_t bytes;
 
   Layout(void *base, int64_t N, int64_t E, int C) {
@@ -171,6 +234,7 @@ struct Layout {
     B1 = f(NC), h1 = f(NC), sc = f(NC), X2 = f(NC), B2 = f(NC), h2 = f(NC), d_h2 = f(NC);
     g1 = f(NC), gB = f(NC), gX2 = f(NC), gh1a = f(NC), gh1 = f(NC);
     live = reinterpret_cast<int32_t *>(take(static_cast<size_t>(2 * N) * sizeof(int32_t)));
+    node_virial = reinterpret_cast<double *>(take(static_cast<size_t>(6 * N) * sizeof(double)));
     bytes = at;
   }
 };
@@ -222,7 +286,7 @@ extern "C" int cm_mace_step_timing_read(double *total_ms, int64_t *launches, int
 
 extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, const double *positions, const double *shifts,
                             void *workspace, size_t workspace_bytes, double *interaction_energy, double *node_energy,
-                            double *forces, double *node_feats, cm_stream_t stream) {
+                            double *forces, double *node_feats, double *virials, cm_stream_t stream) {
   CM_REQUIRE(w && g, "cm_mace_step: NULL weights or graph");
   const int64_t N = g->nnodes, E = g->nedges;
   const int C = w->channels, ne = w->nelements;
@@ -238,6 +302,8 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   }
   if (N == 0) {
     hipLaunchKernelGGL(cm::fill_f64_kernel, dim3(1), dim3(64), 0, st, interaction_energy, static_cast<int64_t>(g->ngraphs), 0.0);
+    if (virials)
+      hipLaunchKernelGGL(cm::fill_f64_kernel, dim3(1), dim3(64), 0, st, virials, static_cast<int64_t>(9) * g->ngraphs, 0.0);
     return cm::check_launch("cm_mace_step");
   }
   CM_REQUIRE(positions && node_energy && forces, "cm_mace_step: NULL positions or output");
@@ -322,5 +388,11 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
                        dim3(256), 0, st, L.gv1, L.gv2, 3 * E);
   CM_STAGE(23, cm_edge_geometry_backward(positions, g->receiver, g->sender, shifts, g->node_rows, g->first_occ, g->sender_perm,
                                     g->sender_offsets, L.gv1, nullptr, N, E, forces, nullptr, stream));
+  if (virials) {
+    if (N > 0)
+      hipLaunchKernelGGL(cm::node_virial_kernel, dim3(static_cast<unsigned>(cm::ceil_div(8 * N, 256))), dim3(256), 0, st, L.vec, L.gv1,
+                       g->first_occ, static_cast<int>(N), E, L.node_virial);
+    hipLaunchKernelGGL(cm::graph_virial_kernel, dim3(g->ngraphs), dim3(cm::kSumThreads), 0, st, L.node_virial, g->graph_ptr, virials);
+  }
   return cm::check_launch("cm_mace_step");
 }

@@ -42,8 +42,11 @@ class DeviceCalculator:
         self.cell = None if cell is None else cell.detach().double().reshape(3, 3).contiguous()
         if use_graph is None:
             use_graph = node_attrs.shape[0] <= 8192
-        self.use_graph = bool(use_graph) and not compute_stress  # the strain path re-derives shifts from the cell
         self.compute_stress = bool(compute_stress)
+        # Stress comes out of the library's one-call step without a strain tensor and replays like the forces; only the
+        # autograd path (a model that cannot take the one-call step) re-derives the shifts from a strained cell.
+        one_call = bool(getattr(model, "native_step", False)) and getattr(model, "_native_step_of", lambda: None)() is not None
+        self.use_graph = bool(use_graph) and (one_call or not self.compute_stress)
         self.run_ahead = bool(run_ahead)
         self.builds = 0
         self.steps = 0
@@ -69,7 +72,10 @@ class DeviceCalculator:
             "ptr": torch.tensor([0, n], dtype=torch.int64, device=dev),
         }
         self._ref_positions = pos.clone()
-        self._graph = GraphedStep(self.model, self._data, warmup=1) if self.use_graph else None
+        self._graph = None
+        if self.use_graph:
+            self._graph = GraphedStep(self.model, self._data, warmup=1, compute_virials=self.compute_stress,
+                                      compute_stress=self.compute_stress)
         self._moved = 0.0
         self.builds += 1
 

@@ -400,6 +400,14 @@ class OptimizedInvariantMACE(torch.nn.Module):
             object.__setattr__(self, "_native", NativeStep(self) if NativeStep.supported(self) else False)
         return self._native or None
 
+    def _native_step_for(self, data, training: bool, compute_force: bool, compute_displacement: bool):
+        """The library's one-call step, if this evaluation can run on it: inference with forces (virials and stress come
+        from the same per-edge gradients), one head, positions on the GPU, no strain tensor asked for."""
+        if not (self.native_step and not training and compute_force and not compute_displacement and "head" not in data
+                and data["positions"].is_cuda):
+            return None
+        return self._native_step_of()
+
     def _fold_contraction_tables(self):
         """Per layer: the packed coupling tables regrouped into monomials (host, once) and folded with the per-element
         weights into coefficient tables on the device."""
@@ -477,8 +485,10 @@ class OptimizedInvariantMACE(torch.nn.Module):
                                                               lambda: self._spatial_order(data))
         inner = dict(data)
         # Without strain the positions stay in the caller's order: the geometry kernels read them (and write the forces)
-        # through the row map.  The strain path transforms positions per graph and works on a gathered copy.
-        direct = not (compute_virials or compute_stress or compute_displacement)
+        # through the row map.  The strain path transforms positions per graph and works on a gathered copy; the
+        # one-call step needs no strain for virials and stress.
+        direct = (not (compute_virials or compute_stress or compute_displacement)
+                  or self._native_step_for(data, training, compute_force, compute_displacement) is not None)
         # With compute_force=False the caller differentiates the returned energies itself (a wrapper that sums the
         # energies of some atoms only): the positions then stay attached to the caller's tensor.
         own = data["positions"].detach() if compute_force else data["positions"]
@@ -518,8 +528,11 @@ class OptimizedInvariantMACE(torch.nn.Module):
         shifts = data["shifts"]
         cell = data.get("cell")
 
+        native = None
+        if node_rows is None or positions_in_caller_order:
+            native = self._native_step_for(data, training, compute_force, compute_displacement)
         displacement = _constant(0.0, (num_graphs, 3, 3), positions.dtype, positions.device)  # replaced below when strained
-        if compute_virials or compute_stress or compute_displacement:
+        if native is None and (compute_virials or compute_stress or compute_displacement):
             positions, shifts, displacement, cell = get_symmetric_displacement(
                 positions=positions, unit_shifts=data["unit_shifts"], cell=cell, edge_index=data["edge_index"],
                 num_graphs=num_graphs, batch=batch)
@@ -558,26 +571,29 @@ class OptimizedInvariantMACE(torch.nn.Module):
         node_attrs32, atom_types = _cached(node_attrs, "_cm_species", None,
                                            lambda: (node_attrs.detach().float(), node_attrs.detach().argmax(dim=-1).int()))
 
-        strained = compute_virials or compute_stress or compute_displacement
-        if (self.native_step and not training and compute_force and not strained and node_heads is None
-                and positions.is_cuda and (node_rows is None or positions_in_caller_order)):
-            native = self._native_step_of()
-            if native is not None:
-                rows32 = None if node_rows is None else node_rows[0]
-                handle = _cached_for(edge_index, "_cm_native_graph_%d" % id(self._weights_token), node_attrs,
-                                     lambda: native.graph(edge_index, receiver, sender, node_attrs32, atom_types, data["ptr"],
-                                                          node_feats_up, rows32))
-                if node_weights is not None:
-                    plain = handle
-                    handle = _cached_for(data["node_weights"], "_cm_native_graph_weighted_%d" % id(self._weights_token), plain,
-                                         lambda: plain.with_node_weights(node_weights))
-                res = native(handle, positions, shifts)
-                inter_e = res["interaction_energy"]
-                return {
-                    "energy": e0 + inter_e, "node_energy": node_e0 + res["node_energy"], "interaction_energy": inter_e,
-                    "forces": res["forces"].to(data["positions"].dtype), "virials": None, "stress": None, "hessian": None,
-                    "displacement": displacement, "node_feats": res["node_feats"], "edge_forces": None,
-                }
+        if native is not None:
+            rows32 = None if node_rows is None else node_rows[0]
+            handle = _cached_for(edge_index, "_cm_native_graph_%d" % id(self._weights_token), node_attrs,
+                                 lambda: native.graph(edge_index, receiver, sender, node_attrs32, atom_types, data["ptr"],
+                                                      node_feats_up, rows32))
+            if node_weights is not None:
+                plain = handle
+                handle = _cached_for(data["node_weights"], "_cm_native_graph_weighted_%d" % id(self._weights_token), plain,
+                                     lambda: plain.with_node_weights(node_weights))
+            want_virials = compute_virials or compute_stress
+            res = native(handle, positions, shifts, want_virials=want_virials)
+            inter_e = res["interaction_energy"]
+            virials = res["virials"].to(positions.dtype) if want_virials else None
+            stress = None
+            if compute_stress and cell is not None:
+                c3 = cell.view(-1, 3, 3).to(virials.dtype)  # the volume as a triple product: a few element-wise launches
+                volume = (c3[:, 0] * torch.linalg.cross(c3[:, 1], c3[:, 2], dim=-1)).sum(dim=-1).abs()
+                stress = -virials / volume.view(-1, 1, 1)
+            return {
+                "energy": e0 + inter_e, "node_energy": node_e0 + res["node_energy"], "interaction_energy": inter_e,
+                "forces": res["forces"].to(data["positions"].dtype), "virials": virials, "stress": stress, "hessian": None,
+                "displacement": displacement, "node_feats": res["node_feats"], "edge_forces": None,
+            }
 
         # vectors = positions[edge_index[1]] - positions[edge_index[0]] + shifts in fp64, rounded once to fp32
         vectors32, lengths32 = EdgeGeometryAutograd.apply(positions, shifts, receiver, sender,

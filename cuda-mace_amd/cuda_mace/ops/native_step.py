@@ -120,7 +120,8 @@ class NativeStep:
         g.node_weights = None
         return _GraphHandle(g, (receiver, sender, first_occ, sperm, soff, eperm, eoff, operm, ooff, ptr32, X1, node_rows))
 
-    def __call__(self, handle: "_GraphHandle", positions: torch.Tensor, shifts: torch.Tensor, want_feats: bool = True) -> Dict[str, torch.Tensor]:
+    def __call__(self, handle: "_GraphHandle", positions: torch.Tensor, shifts: torch.Tensor, want_feats: bool = True,
+                 want_virials: bool = False) -> Dict[str, torch.Tensor]:
         g = handle.struct
         N, E, C = int(g.nnodes), int(g.nedges), self.channels
         dev = positions.device
@@ -137,11 +138,14 @@ class NativeStep:
         node_energy = torch.empty(N, dtype=F64, device=dev)
         forces = torch.empty(N, 3, dtype=F64, device=dev)
         feats = torch.empty(N, 2 * C, dtype=F64, device=dev) if want_feats else None
+        virials = torch.empty(int(g.ngraphs), 3, 3, dtype=F64, device=dev) if want_virials else None
         cabi._check(cabi.lib.cm_mace_step(
             ctypes.addressof(self.weights), ctypes.addressof(g), _ptr(pos64, F64, "positions"), _ptr(sh64, F64, "shifts"),
             ws.data_ptr(), ws.numel(), _ptr(energy, F64, "energy"), _ptr(node_energy, F64, "node_energy"),
-            _ptr(forces, F64, "forces"), _ptr(feats, F64, "node_feats") if want_feats else None, cabi._stream()))
-        return {"interaction_energy": energy, "node_energy": node_energy, "forces": forces, "node_feats": feats}
+            _ptr(forces, F64, "forces"), _ptr(feats, F64, "node_feats") if want_feats else None,
+            _ptr(virials, F64, "virials") if want_virials else None, cabi._stream()))
+        return {"interaction_energy": energy, "node_energy": node_energy, "forces": forces, "node_feats": feats,
+                "virials": virials}
 
 
 class _GraphHandle:

@@ -447,7 +447,10 @@ int cm_readout_backward(const double *grad_node_energies, const double *w1, cons
  * Per call: positions fp64 [nnodes, 3], shifts fp64 [nedges, 3]; outputs interaction_energy fp64 [ngraphs] ((weighted) sum
  * of the node energies of each graph, in a fixed order), node_energy fp64 [nnodes] (interaction part, unweighted, in
  * list order), forces fp64 [nnodes, 3] = -d(sum of interaction_energy)/d positions (rows of the caller when node_rows is given), node_feats fp64
- * [nnodes, 2C] or NULL.  workspace: cm_mace_step_workspace(nnodes, nedges, channels) bytes, 256-byte aligned; its
+ * [nnodes, 2C] or NULL, virials fp64 [ngraphs, 3, 3] or NULL = minus the derivative of each graph's energy with respect to a
+ * symmetric strain of its positions and cell (what models/InvariantMACE.py:273-285 obtains by differentiating through
+ * get_symmetric_displacement), formed from the per-edge gradients as 1/2 sum_e (vec_e (x) g_e + g_e (x) vec_e), g_e =
+ * -dE/d vec_e.  workspace: cm_mace_step_workspace(nnodes, nedges, channels) bytes, 256-byte aligned; its
  * contents are scratch.  Nothing is allocated, so the call can be captured into a HIP graph.
  */
 typedef struct cm_mace_weights {
@@ -492,7 +495,7 @@ int cm_mace_step_timing_read(double *total_ms, int64_t *launches, int capacity);
 size_t cm_mace_step_workspace(int64_t nnodes, int64_t nedges, int channels);
 int cm_mace_step(const cm_mace_weights *weights, const cm_mace_graph *graph, const double *positions, const double *shifts,
                  void *workspace, size_t workspace_bytes, double *interaction_energy, double *node_energy, double *forces,
-                 double *node_feats, cm_stream_t stream);
+                 double *node_feats, double *virials, cm_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -85,6 +85,37 @@ def test_running_ahead_of_the_displacement_test(cabi):
         assert torch.equal(ea, eb) and torch.equal(fa, fb)
 
 
+def test_stress_replays_with_the_forces(cabi):
+    """With stress asked for, the calculator still replays the step as one HIP graph (the one-call step forms the virials
+    from the per-edge gradients, no strain tensor in the way): energy, forces and stress of every step of a short walk
+    equal the model's on an exact list."""
+    from cuda_mace.calculators import DeviceCalculator
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.utils.neighbour_list import neighbour_data
+    from cuda_mace.utils.synthetic import make_system, to_device
+
+    n = 350
+    data = to_device(make_system(n, 4, seed=41, density=0.1), "cuda")
+    upstream = SyntheticInvariantMACE(channels=64, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=data["edge_index"].shape[1] / n,
+                                      seed=42)
+    model = OptimizedInvariantMACE(upstream, device="cuda")
+    pbc = (True, True, True)
+    calc = DeviceCalculator(model, data["node_attrs"], cutoff=5.0, skin=0.4, pbc=pbc, cell=data["cell"], use_graph=True,
+                            compute_stress=True)
+    assert calc.use_graph
+    g = torch.Generator(device="cuda").manual_seed(2)
+    pos = data["positions"].clone()
+    for _ in range(8):
+        pos = pos + 0.04 * torch.randn(pos.shape, device="cuda", dtype=pos.dtype, generator=g)
+        got = calc.compute(pos)
+        assert calc._graph is not None
+        exact = model(neighbour_data(pos.clone(), data["node_attrs"], 5.0, pbc, data["cell"]), compute_stress=True)
+        torch.testing.assert_close(got["energy"], exact["energy"].detach(), rtol=1e-7, atol=1e-7)
+        torch.testing.assert_close(got["forces"], exact["forces"].detach(), rtol=0, atol=2e-6 * float(exact["forces"].abs().max()))
+        torch.testing.assert_close(got["stress"], exact["stress"].detach(), rtol=0, atol=2e-6 * float(exact["stress"].abs().max()))
+    assert calc.builds >= 2
+
+
 @pytest.mark.parametrize("relabel", [False, True], ids=["as_given", "relabelled"])
 def test_lammps_style_wrapper(cabi, relabel):
     """LAMMPS_MACE (upstream's interface for a domain-decomposed MD code): the energy of the rank's own atoms and minus
