@@ -60,10 +60,17 @@ def get_symmetric_displacement(positions, unit_shifts, cell, edge_index, num_gra
     displacement = torch.zeros((num_graphs, 3, 3), dtype=positions.dtype, device=positions.device)
     displacement.requires_grad_(True)
     symmetric = 0.5 * (displacement + displacement.transpose(-1, -2))
-    positions = positions + torch.einsum("be,bec->bc", positions, symmetric[batch])
     cell = cell.view(-1, 3, 3)
     cell = cell + torch.matmul(cell, symmetric)
-    shifts = torch.einsum("be,bec->bc", unit_shifts, cell[batch[sender]])
+    if num_graphs == 1:
+        # one graph: products with the one matrix broadcast, whose backward is a sum over the rows (the gathered form
+        # below makes autograd add every atom's and every edge's 3 x 3 contribution into the one strain / cell with
+        # atomics: 0.5 s at 1.3 million edges; as a matrix product the backward is a 3 x E by E x 3 GEMM, 37 ms there)
+        positions = positions + (positions.unsqueeze(-1) * symmetric[0].unsqueeze(0)).sum(dim=1)
+        shifts = (unit_shifts.to(cell.dtype).unsqueeze(-1) * cell[0].unsqueeze(0)).sum(dim=1)
+    else:
+        positions = positions + torch.einsum("be,bec->bc", positions, symmetric[batch])
+        shifts = torch.einsum("be,bec->bc", unit_shifts, cell[batch[sender]])
     return positions, shifts, displacement, cell
 
 
