@@ -51,6 +51,23 @@ def get_edge_vectors_and_lengths(positions, edge_index, shifts) -> Tuple[torch.T
     return vectors, torch.linalg.norm(vectors, dim=-1, keepdim=True)
 
 
+class _RowsOfSortedIndex(torch.autograd.Function):
+    """src[index] for a non-decreasing index whose segment boundaries are `offsets` (offsets[g] = first position with
+    index g).  The backward is one reduction per segment (a slice each); the plain gather's backward adds every row into
+    the few rows of src with atomics, which serialises when thousands of rows share one, and torch.segment_reduce gives a
+    segment to a single thread."""
+
+    @staticmethod
+    def forward(ctx, src, index, offsets):
+        ctx.bounds = [int(v) for v in offsets.tolist()]
+        return src.index_select(0, index)
+
+    @staticmethod
+    def backward(ctx, grad):
+        b = ctx.bounds
+        return torch.stack([grad[b[g]:b[g + 1]].sum(dim=0) for g in range(len(b) - 1)]), None, None
+
+
 def get_symmetric_displacement(positions, unit_shifts, cell, edge_index, num_graphs, batch):
     """Applies a symmetric strain (zero, but differentiable) to positions and cell so that
     d energy / d displacement gives the virial."""
@@ -69,8 +86,16 @@ def get_symmetric_displacement(positions, unit_shifts, cell, edge_index, num_gra
         positions = positions + (positions.unsqueeze(-1) * symmetric[0].unsqueeze(0)).sum(dim=1)
         shifts = (unit_shifts.to(cell.dtype).unsqueeze(-1) * cell[0].unsqueeze(0)).sum(dim=1)
     else:
-        positions = positions + torch.einsum("be,bec->bc", positions, symmetric[batch])
-        shifts = torch.einsum("be,bec->bc", unit_shifts, cell[batch[sender]])
+        graphs = torch.arange(num_graphs + 1, device=batch.device, dtype=batch.dtype)
+        edge_graph = batch[sender]
+        sorted_lists = bool((batch[1:] >= batch[:-1]).all()) and bool((edge_graph[1:] >= edge_graph[:-1]).all())
+        if sorted_lists:  # atoms and edges graph by graph, as every collated batch has them
+            per_atom = _RowsOfSortedIndex.apply(symmetric, batch, torch.searchsorted(batch, graphs))
+            per_edge = _RowsOfSortedIndex.apply(cell, edge_graph, torch.searchsorted(edge_graph, graphs))
+        else:
+            per_atom, per_edge = symmetric[batch], cell[edge_graph]
+        positions = positions + torch.einsum("be,bec->bc", positions, per_atom)
+        shifts = torch.einsum("be,bec->bc", unit_shifts.to(cell.dtype), per_edge)
     return positions, shifts, displacement, cell
 
 
