@@ -561,6 +561,20 @@ def main():
                        "(1 + skin/cutoff)^3 = 1.33x the pairs of the exact list; the host reads the displacement test "
                        "after it has enqueued the step (a step on a list found stale is enqueued again)"}
 
+    # the same step with virials and stress (formed from the per-edge gradients in the same library call)
+    with_stress = None
+    if not args.no_extras and fused:
+        for _ in range(3):
+            model(dict(data), compute_stress=True)
+        torch.cuda.synchronize()
+        t_s = time.perf_counter()
+        for _ in range(20):
+            out_s = model(dict(data), compute_stress=True)
+        torch.cuda.synchronize()
+        with_stress = {"ms_per_step": round(1e3 * (time.perf_counter() - t_s) / 20, 4), "steps": 20,
+                       "stress_finite": bool(torch.isfinite(out_s["stress"]).all()),
+                       "note": "energy + forces + virials + stress in one library call"}
+
     configs = None
     if not args.no_extras:
         del calc
@@ -597,7 +611,7 @@ def main():
                                "l_max 3, correlation 3, %d elements, random-init weights (seed 0)" % (N, E, C, ne),
                    "atoms": N, "edges": E, "channels": C, "radial": "fused spline" if fused else "tabulated"},
         "roofline": roofline, "roofline_other_kernels": others, "cpu_baseline": cpu_baseline,
-        "neighbour_list": neighbour_list, "md_loop": md_loop, "other_configs": configs,
+        "neighbour_list": neighbour_list, "md_loop": md_loop, "with_stress": with_stress, "other_configs": configs,
     }
     if cpu_baseline:
         line["speedup_vs_cpu_baseline"] = round(value / cpu_baseline["value"], 1)

@@ -15,9 +15,11 @@
 //   X2         = h1 . Wup                           gA        = (gB1 * grad1) . Wmix0^T      (per element)
 //   M2         = MP(X2, vec, spline 1)              gv1       = MP backward(X1, vec, spline 0, gA)   (no gX: X1 is constant)
 //   A          = mix1(M2)                           forces    = geometry backward(gv1 + gv2)
-//   B2, grad2  = contraction 1 (A)
-//   h2         = B2 . Wprod2 + sc
+//   B2, grad2  = contraction 1 (A)                  virials   = 1/2 sum_e (vec (x) gv + gv (x) vec), per node, then per graph
+//   h2         = B2 . Wprod2 + sc                               (on request)
 //   E_n, dE/dh2, feats = readouts(h1, h2);  E_graph = sum over the graph's nodes
+// With node weights (cm_mace_graph.node_weights) E_graph = sum_n weight[n] E_n and the seed of node n is -weight[n]: g1's
+// rows and the rows of dE/dh2 are multiplied by the node's weight before the chain starts.
 #include <mutex>
 #include <vector>
 
