@@ -139,11 +139,15 @@ def test_lammps_style_wrapper(cabi, relabel):
     got = wrapper(dict(dev), local.cuda())
     assert model._native not in (None, False)  # the mask went into the library's one-call step as node weights
     # the route for models that know nothing of node weights (upstream's own): node energies out, autograd in the wrapper
+    got_v = wrapper(dict(dev), local.cuda(), compute_virials=True)  # virials of the masked energy, from the same call
     model.supports_node_weights = False
     try:
         generic = wrapper(dict(dev), local.cuda())
+        generic_v = wrapper(dict(dev), local.cuda(), compute_virials=True)  # by autograd through the strain
     finally:
         del model.supports_node_weights
+    assert torch.equal(got_v["forces"], got["forces"])
+    torch.testing.assert_close(got_v["virials"], generic_v["virials"], rtol=0, atol=2e-6 * float(generic_v["virials"].abs().max()))
     torch.testing.assert_close(generic["total_energy_local"], got["total_energy_local"], rtol=1e-12, atol=1e-12)
     torch.testing.assert_close(generic["forces"], got["forces"], rtol=0, atol=5e-7 * float(got["forces"].abs().max()))
     # all-ones weights are the unweighted step bit for bit
