@@ -144,8 +144,11 @@ __global__ void symcon_forward_kernel(const S *__restrict__ X, const int32_t *__
 
 // Specialised forward for the l_max = 3 structure known at build time: the monomial lists are unrolled, so a
 // thread (= one channel) keeps its 77 + 16 + 1 coefficients, the node's 16 inputs and 16 gradient accumulators in
-// registers and streams over kNodesPerBlock nodes of one element.  No LDS; loads and stores are coalesced rows.
-constexpr int kNodesPerBlock = 16;
+// registers and streams over `npb` nodes of one element.  No LDS; loads and stores are coalesced rows.  npb is 16 where
+// that still gives every SIMD two waves (the coefficient loads are then a fifth of a wave's loads), fewer for fewer
+// nodes, down to 2: at 5 000 nodes x 96 channels 16 nodes per wave leave the device at 0.6 waves per SIMD (29 us per
+// launch, the time of one wave's 16 nodes).
+constexpr int kMaxNodesPerBlock = 16;
 
 template <typename S, bool GRAD>
 __global__ __launch_bounds__(kWave) void symcon_lmax3_kernel(const S *__restrict__ X,
@@ -153,16 +156,16 @@ __global__ __launch_bounds__(kWave) void symcon_lmax3_kernel(const S *__restrict
                                                             const int32_t *__restrict__ group_offsets,
                                                             const S *__restrict__ T3, const S *__restrict__ T2,
                                                             const S *__restrict__ T1, int nnodes, int ne, int C,
-                                                            S *__restrict__ out, S *__restrict__ grad) {
+                                                            int npb, S *__restrict__ out, S *__restrict__ grad) {
   const int c = blockIdx.y * kWave + threadIdx.x;
   int tile = blockIdx.x;
   int e = 0, pos0 = 0, gend = 0;
   bool found = false;
   for (e = 0; e < ne; ++e) {
     const int lo = group_offsets[e], hi = group_offsets[e + 1];
-    const int tiles = (hi - lo + kNodesPerBlock - 1) / kNodesPerBlock;
+    const int tiles = (hi - lo + npb - 1) / npb;
     if (tile < tiles) {
-      pos0 = lo + tile * kNodesPerBlock;
+      pos0 = lo + tile * npb;
       gend = hi;
       found = true;
       break;
@@ -170,7 +173,7 @@ __global__ __launch_bounds__(kWave) void symcon_lmax3_kernel(const S *__restrict
     tile -= tiles;
   }
   if (!found || c >= C) return;
-  const int nb = min(kNodesPerBlock, gend - pos0);
+  const int nb = min(npb, gend - pos0);
 
   S t3[CM_SYMCON_N3], t2[CM_SYMCON_N2];
 #pragma unroll
@@ -298,14 +301,16 @@ int forward(const char *what, const S *X, const int32_t *node_perm, const int32_
                "%s: built-in structure has %d cubic and %d quadratic monomials, got %d and %d", what, CM_SYMCON_N3,
                CM_SYMCON_N2, n3, n2);
     CM_REQUIRE(T3 && T2, "%s: NULL table", what);
-    const dim3 grid(static_cast<unsigned>(ceil_div(nnodes, kNodesPerBlock) + nelements),
-                    static_cast<unsigned>(ceil_div(channels, kWave)));
+    const int64_t column_blocks = ceil_div(channels, kWave);
+    const int64_t two_waves_per_simd = static_cast<int64_t>(device_compute_units()) * 4 * 2;
+    const int npb = static_cast<int>(std::max<int64_t>(2, std::min<int64_t>(kMaxNodesPerBlock, nnodes * column_blocks / two_waves_per_simd)));
+    const dim3 grid(static_cast<unsigned>(ceil_div(nnodes, npb) + nelements), static_cast<unsigned>(column_blocks));
     if (grad)
       hipLaunchKernelGGL((symcon_lmax3_kernel<S, true>), grid, dim3(kWave), 0, st, X, node_perm, group_offsets, T3, T2, T1,
-                         static_cast<int>(nnodes), nelements, channels, out, grad);
+                         static_cast<int>(nnodes), nelements, channels, npb, out, grad);
     else
       hipLaunchKernelGGL((symcon_lmax3_kernel<S, false>), grid, dim3(kWave), 0, st, X, node_perm, group_offsets, T3, T2, T1,
-                         static_cast<int>(nnodes), nelements, channels, out, grad);
+                         static_cast<int>(nnodes), nelements, channels, npb, out, grad);
     return check_launch(what);
   }
   // LDS per workgroup is held to 32 KB in fp32, 64 KB in fp64 (two [NB][16][C] arrays) so that several fit a CU
