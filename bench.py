@@ -299,6 +299,15 @@ def other_configs(torch, make_system, to_device, OptimizedInvariantMACE, Synthet
     res["c1"] = run("21-atom cluster in an 8 A cube, {H,C,N,O}, 64x0e (fp32 kernels; the fp64 CPU reference is the parity "
                     "oracle of this configuration)", make_system(21, 4, seed=0, density=None, cluster_box=8.0), 64,
                     (1, 6, 7, 8), 20, 200, graph=True)
+    # how configuration 1 is served when throughput matters: many such structures in one batch, one library call
+    from cuda_mace.utils.synthetic import collate
+
+    nbatch = 512
+    many = run("%d clusters of configuration 1 in one batch (different seeds), one step for all of them" % nbatch,
+               collate([make_system(21, 4, seed=s, density=None, cluster_box=8.0) for s in range(nbatch)]), 64, (1, 6, 7, 8), 10, 50)
+    many["structures"] = nbatch
+    many["us_per_structure"] = round(1e3 * many["ms_per_step"] / nbatch, 3)
+    res["c1"]["batched"] = many
     res["c3"] = run("5 000-atom periodic box, 96x0e, 10 elements", make_system(5000, 10, seed=0, density=0.1), 96,
                     tuple(range(1, 11)), 10, 50)
     res["c5"] = run("100 000-atom periodic box, 192x0e, 10 elements", make_system(100000, 10, seed=0, density=0.1), 192,
