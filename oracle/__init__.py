@@ -23,6 +23,13 @@ Pin status of each function (what fixes it besides its own formula):
                           U_matrix_real is PARITY UNPINNED (upstream package
                           is not available offline; only matters for trained
                           checkpoints, not for random-init weights)
+  readout_energies        scalar python loops over nodes, channels and hidden
+                          units; special cases (dead hidden layer, one hidden
+                          unit without layer-1 features, saturated gate); the
+                          shift added after the scale; and, in the model, the
+                          two-atom chain carried by hand through both layers
+                          to the node energies (fan-in folds, gate constant,
+                          scale, shift, E0)
   neighbour_list          scipy cKDTree (periodic, box > 2 cutoff), explicit
                           replication of the cell into a non-periodic cluster
                           searched by a non-periodic cKDTree (small cells,

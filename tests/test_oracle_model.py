@@ -238,10 +238,13 @@ def test_single_atom_energy_is_closed_form():
 
 def test_two_atom_energy_is_closed_form():
     """Two atoms at distance d along z, one channel per l that matters: with Y(z-axis) known in closed form (Y_l0 =
-    sqrt(2l+1), every other component 0) the whole first layer is a hand-computable scalar chain.  Checks the chain
-    radial basis -> MLP -> message -> 1/avg_num_neighbors -> linear -> per-element linear -> contraction -> product
-    linear -> linear readout, with independent arithmetic (numpy, explicit loops over the 16 components)."""
-    model = SyntheticInvariantMACE(channels=32, atomic_numbers=(1, 6), avg_num_neighbors=3.0, seed=5)
+    sqrt(2l+1), every other component 0) both layers are a hand-computable scalar chain.  Checks the chain
+    radial basis -> MLP -> message -> 1/avg_num_neighbors -> linear -> per-element linear (on the message in layer 1,
+    as skip connection in layer 2) -> contraction -> product linear -> both readouts -> scale, shift, E0, with
+    independent arithmetic (numpy, explicit loops over the 16 components, the hidden units and the channels)."""
+    scale, shift = 1.7, -0.4
+    model = SyntheticInvariantMACE(channels=32, atomic_numbers=(1, 6), avg_num_neighbors=3.0, seed=5, scale=scale,
+                                   shift=shift, atomic_energies=torch.tensor([-1.25, 3.5]))
     p = model.export_params()
     C, ne, d = 32, 2, 1.7
     attrs = torch.tensor([[1.0, 0.0], [0.0, 1.0]], dtype=torch.float64)
@@ -253,42 +256,70 @@ def test_two_atom_energy_is_closed_form():
     from oracle.u_tensors import u_tensors
 
     U1, U2, U3 = u_tensors()
-    lay = p["layers"][0]
     r_max, nb, pw = float(p["r_max"]), int(p["num_bessel"]), int(p["p"])
     x = d / r_max
     env = 1 - (pw + 1) * (pw + 2) / 2 * x ** pw + pw * (pw + 2) * x ** (pw + 1) - pw * (pw + 1) / 2 * x ** (pw + 2)
     basis = np.array([math.sqrt(2 / r_max) * math.sin(n * math.pi * d / r_max) / d * env for n in range(1, nb + 1)])
-    z = basis
-    mlp = [W.double().numpy() for W in lay["mlp"]]
-    for i, W in enumerate(mlp):
-        z = z @ W / math.sqrt(W.shape[0])
-        if i + 1 < len(mlp):
-            z = M.SILU_2MOM * z / (1 + np.exp(-z))
-    R = z.reshape(4, C)
     h0 = (attrs @ p["W_emb"].double() / math.sqrt(ne)).numpy()
-    u = h0 @ lay["W_up"].double().numpy() / math.sqrt(C)
-    h1 = np.zeros((2, C))
-    W_lin, W_skip = lay["W_lin"].double().numpy(), lay["W_skip"].double().numpy()
-    for rcv, snd, sign in ((1, 0, +1.0), (0, 1, -1.0)):  # edge vector = pos[rcv] - pos[snd] = +-d along the 3rd axis
-        # harmonics of +-z in the oracle's component order, taken from the scipy-pinned routine
-        Y = O.spherical_harmonics(torch.tensor([[0.0, 0.0, sign * d]], dtype=torch.float64))[:, 0].numpy()
-        A = np.zeros((16, C))
-        for m in range(16):
-            l = int(math.isqrt(m))
-            msg = u[snd] * Y[m] * R[l]
-            A[m] = (msg @ W_lin[l]) / math.sqrt(C) / 3.0
-            A[m] = (A[m] @ W_skip[l][:, rcv, :]) / math.sqrt(C * ne)  # element of atom rcv is rcv
-        e = rcv
-        B = np.zeros(C)
-        W3, W2, W1 = (lay[k].double().numpy()[e] for k in ("W3", "W2", "W1"))
-        for c in range(C):
-            a = A[:, c]
-            B[c] = np.einsum("ijkp,p,i,j,k->", U3, W3[:, c], a, a, a) + np.einsum("ijp,p,i,j->", U2, W2[:, c], a, a) + W1[0, c] * a[0]
-        h1[rcv] = B @ lay["W_prod"].double().numpy() / math.sqrt(C)
-    e1 = h1 @ p["w_read0"].double().numpy()[:, 0] / math.sqrt(C)
-    got1 = out["node_feats"][:, :C].numpy()
-    np.testing.assert_allclose(got1, h1, rtol=1e-10, atol=1e-13)
-    assert np.abs(h1).max() > 1e-4 and np.abs(e1).max() > 1e-6
+
+    def layer_by_hand(t, h_in):
+        lay = p["layers"][t]
+        z = basis
+        mlp = [W.double().numpy() for W in lay["mlp"]]
+        for i, W in enumerate(mlp):
+            z = z @ W / math.sqrt(W.shape[0])
+            if i + 1 < len(mlp):
+                z = M.SILU_2MOM * z / (1 + np.exp(-z))
+        R = z.reshape(4, C)
+        u = h_in @ lay["W_up"].double().numpy() / math.sqrt(C)
+        h_out = np.zeros((2, C))
+        W_lin, W_skip = lay["W_lin"].double().numpy(), lay["W_skip"].double().numpy()
+        for rcv, snd, sign in ((1, 0, +1.0), (0, 1, -1.0)):  # edge vector = pos[rcv] - pos[snd] = +-d along the 3rd axis
+            # harmonics of +-z in the oracle's component order, taken from the scipy-pinned routine
+            Y = O.spherical_harmonics(torch.tensor([[0.0, 0.0, sign * d]], dtype=torch.float64))[:, 0].numpy()
+            A = np.zeros((16, C))
+            for m in range(16):
+                l = int(math.isqrt(m))
+                msg = u[snd] * Y[m] * R[l]
+                A[m] = (msg @ W_lin[l]) / math.sqrt(C) / 3.0
+                if t == 0:  # the first layer's per-element linear acts on the message; element of atom rcv is rcv
+                    A[m] = (A[m] @ W_skip[l][:, rcv, :]) / math.sqrt(C * ne)
+            e = rcv
+            B = np.zeros(C)
+            W3, W2, W1 = (lay[k].double().numpy()[e] for k in ("W3", "W2", "W1"))
+            for c in range(C):
+                a = A[:, c]
+                B[c] = (np.einsum("ijkp,p,i,j,k->", U3, W3[:, c], a, a, a) + np.einsum("ijp,p,i,j->", U2, W2[:, c], a, a)
+                        + W1[0, c] * a[0])
+            h_out[rcv] = B @ lay["W_prod"].double().numpy() / math.sqrt(C)
+            if t == 1:  # the second layer's per-element linear is the skip connection on the incoming scalars
+                h_out[rcv] += h_in[rcv] @ W_skip[0][:, rcv, :] / math.sqrt(C * ne)
+        return h_out
+
+    h1 = layer_by_hand(0, h0)
+    h2 = layer_by_hand(1, h1)
+    np.testing.assert_allclose(out["node_feats"][:, :C].numpy(), h1, rtol=1e-10, atol=1e-13)
+    np.testing.assert_allclose(out["node_feats"][:, C:].numpy(), h2, rtol=1e-9, atol=1e-13)
+    # readouts, scale and shift with scalar arithmetic: linear readout of layer 1; layer 2 through 16 hidden units
+    # with the normalised silu gate; every weight divided by the square root of its fan-in; E0 of the element
+    w0 = p["w_read0"].double().numpy()[:, 0]
+    Wa, wb = p["W_read1"].double().numpy(), p["w_read2"].double().numpy()[:, 0]
+    hidden = Wa.shape[1]
+    assert hidden == 16 and abs(scale - 1.0) > 0.1 and abs(shift) > 0.1
+    e_node = np.zeros(2)
+    for n in range(2):
+        e1 = sum(h1[n, c] * w0[c] for c in range(C)) / math.sqrt(C)
+        e2 = 0.0
+        for k in range(hidden):
+            zk = sum(h2[n, c] * Wa[c, k] for c in range(C)) / math.sqrt(C)
+            e2 += wb[k] * M.SILU_2MOM * zk / (1 + math.exp(-zk))
+        e2 /= math.sqrt(hidden)
+        e_node[n] = float(p["E0"][n]) + scale * (e1 + e2) + shift
+        assert abs(e1) > 1e-6 and abs(e2) > 1e-6
+    np.testing.assert_allclose(out["node_energy"].numpy(), e_node, rtol=1e-10, atol=1e-13)
+    assert abs(float(out["energy"]) - e_node.sum()) < 1e-12 * max(1.0, abs(e_node.sum()))
+    # the comparison has teeth: a 1 % error in the gate constant or in 1/sqrt(hidden) is 1e6 tolerances away
+    assert np.abs(out["node_energy"].numpy() - e_node).max() < 1e-3 * abs(scale * 0.01 * e2)
 
 
 def test_carving_is_exact_on_the_reference_itself():

@@ -286,3 +286,74 @@ def test_neighbour_list_oracle_cluster_and_self_images():
     # a single atom in a 3 A cubic cell with a 3.5 A cutoff sees its 6 nearest images only (next shell at 4.24 A)
     ei, S = O.neighbour_list(np.array([[0.3, 0.2, 0.1]]), np.eye(3) * 3.0, (1, 1, 1), 3.5)
     assert ei.shape[1] == 6 and sorted(map(tuple, S)) == sorted([(1, 0, 0), (-1, 0, 0), (0, 1, 0), (0, -1, 0), (0, 0, 1), (0, 0, -1)])
+
+
+# ---- readouts, scale and shift --------------------------------------------------------------------
+def _readout_case(seed, n=7, C=5, H=3):
+    g = np.random.default_rng(seed)
+    return (g.normal(size=(n, C)), g.normal(size=(n, C)), g.normal(size=C), g.normal(size=(C, H)),
+            g.normal(size=H), 1.37, 0.8, -0.35)
+
+
+def _readout_loops(h1, h2, w1, W2a, w2b, act, scale, shift):
+    """Scalar arithmetic, one node and one hidden unit at a time: layer-1 energy is a dot product, layer-2 energy
+    a sum over hidden units of weight * act * z / (1 + exp(-z)); the sum of the two is scaled, then shifted."""
+    out = np.zeros(h1.shape[0])
+    for n in range(h1.shape[0]):
+        e = 0.0
+        for c in range(h1.shape[1]):
+            e += h1[n, c] * w1[c]
+        for k in range(W2a.shape[1]):
+            z = 0.0
+            for c in range(h2.shape[1]):
+                z += h2[n, c] * W2a[c, k]
+            e += w2b[k] * act * z / (1.0 + math.exp(-z))
+        out[n] = scale * e + shift
+    return out
+
+
+def test_readout_energies_explicit_loops():
+    case = _readout_case(0)
+    got = O.readout_energies(*(torch.from_numpy(a) if isinstance(a, np.ndarray) else a for a in case)).numpy()
+    np.testing.assert_allclose(got, _readout_loops(*case), rtol=1e-13, atol=1e-14)
+
+
+def test_readout_energies_special_cases():
+    h1, h2, w1, W2a, w2b, act, scale, shift = _readout_case(1)
+    t = torch.from_numpy
+    # a dead hidden layer (silu(0) = 0) leaves the linear readout alone: scale * h1.w1 + shift
+    got = O.readout_energies(t(h1), t(h2), t(w1), t(np.zeros_like(W2a)), t(w2b), act, scale, shift).numpy()
+    np.testing.assert_allclose(got, scale * (h1 @ w1) + shift, rtol=1e-13)
+    # no layer-1 features, one hidden unit: a scalar chain per node
+    W1u, w2u = W2a[:, :1], w2b[:1]
+    got = O.readout_energies(t(np.zeros_like(h1)), t(h2), t(w1), t(W1u), t(w2u), act, scale, shift).numpy()
+    for n in range(h2.shape[0]):
+        z = float(h2[n] @ W1u[:, 0])
+        assert abs(got[n] - (scale * w2u[0] * act * z / (1 + math.exp(-z)) + shift)) < 1e-13
+    # the shift is added after the scale, not scaled with it; the scale multiplies both readouts
+    a = O.readout_energies(t(h1), t(h2), t(w1), t(W2a), t(w2b), act, 1.0, 0.0).numpy()
+    b = O.readout_energies(t(h1), t(h2), t(w1), t(W2a), t(w2b), act, 3.0, 0.5).numpy()
+    np.testing.assert_allclose(b, 3.0 * a + 0.5, rtol=1e-13)
+    # large pre-activations: the gate is the identity times act for z >> 0 and 0 for z << 0
+    big = O.readout_energies(t(np.zeros((2, 1))), t(np.array([[40.0], [-40.0]])), t(np.zeros(1)), t(np.ones((1, 1))),
+                             t(np.ones(1)), act, 1.0, 0.0).numpy()
+    np.testing.assert_allclose(big, [act * 40.0, 0.0], rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("which", ["act", "scale", "shift_scaled", "w2b", "w1"])
+def test_readout_pin_has_teeth(which):
+    """A 1 % error in the activation constant, the scale, either weight fold, or a shift that is scaled with the sum
+    moves the loop value by far more than the tolerance of the comparison above."""
+    h1, h2, w1, W2a, w2b, act, scale, shift = _readout_case(2)
+    ref = _readout_loops(h1, h2, w1, W2a, w2b, act, scale, shift)
+    if which == "act":
+        bad = _readout_loops(h1, h2, w1, W2a, w2b, act * 1.01, scale, shift)
+    elif which == "scale":
+        bad = _readout_loops(h1, h2, w1, W2a, w2b, act, scale * 1.01, shift)
+    elif which == "shift_scaled":
+        bad = _readout_loops(h1, h2, w1, W2a, w2b, act, scale, shift * scale)
+    elif which == "w2b":
+        bad = _readout_loops(h1, h2, w1, W2a, w2b * 1.01, act, scale, shift)
+    else:
+        bad = _readout_loops(h1, h2, w1 * 1.01, W2a, w2b, act, scale, shift)
+    assert np.abs(bad - ref).max() > 1e-4
