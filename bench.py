@@ -28,6 +28,20 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_25k_atoms_128ch.json"
 KERNEL_SOURCES = os.path.join(ROOT, "cuda-mace_amd", "csrc")
 
 
+# stages of cm_mace_step (include/cuda_mace_hip.h), in the order they run
+STAGE_NAMES = {
+    0: "00 edge geometry + live ranges", 1: "01 mp forward L0", 2: "02 channel mixing L0 [N,16,C]", 3: "03 contraction L0",
+    4: "04 product linear L0 (+ skip, linear_up when chained)", 5: "05 skip connection", 6: "06 linear_up",
+    7: "07 mp forward L1", 8: "08 channel mixing L1 [N,16,C]", 9: "09 contraction L1", 10: "10 product linear L1 + skip",
+    11: "11 readouts", 12: "12 energy sums", 13: "13 backward seeds", 14: "14 product linear L1 backward",
+    15: "15 channel mixing L1 backward (+ contraction backward)", 16: "16 mp backward L1 (edge pass + sender pass)",
+    17: "17 linear_up backward (+ skip, product linear L0 backward when chained)", 18: "18 skip backward",
+    19: "19 product linear L0 backward", 20: "20 channel mixing L0 backward (+ contraction backward)",
+    21: "21 mp backward L0 (edge pass, onto L1's vector gradient)", 22: "22 sum of vector gradients",
+    23: "23 edge geometry backward (forces)", 24: "24 virials",
+}
+
+
 def kernel_sources_digest():
     """sha256 over the kernel sources (names and contents, sorted): ties a counter measurement to the code it was made on."""
     import hashlib
@@ -308,6 +322,18 @@ def other_configs(torch, make_system, to_device, OptimizedInvariantMACE, Synthet
     many["structures"] = nbatch
     many["us_per_structure"] = round(1e3 * many["ms_per_step"] / nbatch, 3)
     res["c1"]["batched"] = many
+    # the reference's own benchmark workload (tools/model_surgery.py:145-233: a cubic diamond supercell of size^3 cells with
+    # 0.05 A of noise, default size 3 = 216 atoms), here with a 128-channel model
+    from cuda_mace.tools.model_surgery import test_batch
+
+    class _Table:
+        atomic_numbers, r_max = (1, 6, 7, 8), 5.0
+
+    for size in (3, 4):
+        batch = {k: (v.cpu() if hasattr(v, "cpu") else v) for k, v in test_batch(_Table, size).items()}
+        res["diamond_%d" % (8 * size ** 3)] = run(
+            "the reference's benchmark structure: diamond supercell --size %d (%d atoms, noise 0.05 A), 128x0e" % (size, 8 * size ** 3),
+            batch, 128, (1, 6, 7, 8), 50, 100, graph=True)
     res["c3"] = run("5 000-atom periodic box, 96x0e, 10 elements", make_system(5000, 10, seed=0, density=0.1), 96,
                     tuple(range(1, 11)), 10, 50)
     res["c5"] = run("100 000-atom periodic box, 192x0e, 10 elements", make_system(100000, 10, seed=0, density=0.1), 192,
@@ -421,6 +447,21 @@ def main():
         cabi._check(min(cabi.lib.cm_mace_step_timing_read(ctypes.addressof(stage_ms), ctypes.addressof(stage_n), 32), 0))
         cabi._check(cabi.lib.cm_mace_step_timing(0))
 
+    # every stage of the step, bracketed by events in a few more steps outside the timed region (the brackets cost a
+    # few microseconds of launch gaps per stage, so the sum sits slightly above ms_per_step)
+    stages_us, stages_sum_ms, launches_per_step = None, None, None
+    if native:
+        all_ms, all_n = (ctypes.c_double * 32)(), (ctypes.c_int64 * 32)()
+        cabi._check(cabi.lib.cm_mace_step_timing((1 << 25) - 1))
+        nsteps_all = 10
+        for _ in range(nsteps_all):
+            step()
+        torch.cuda.synchronize()
+        cabi._check(min(cabi.lib.cm_mace_step_timing_read(ctypes.addressof(all_ms), ctypes.addressof(all_n), 32), 0))
+        cabi._check(cabi.lib.cm_mace_step_timing(0))
+        stages_us = {STAGE_NAMES[i]: round(1e3 * all_ms[i] / nsteps_all, 1) for i in range(25) if all_n[i]}
+        stages_sum_ms = round(sum(all_ms[i] for i in range(25)) / nsteps_all, 4)
+
     ms_per_step = 1e3 * elapsed / args.steps
     value = N * args.steps / elapsed
     assert bool(torch.isfinite(energy).all()) and bool(torch.isfinite(forces).all())
@@ -488,16 +529,14 @@ def main():
         if t_lin:
             flops = 32 * N * C * C
             tf = flops / (t_lin * 1e-3) / 1e12
-            others.append({"kernel": linear_kernel_name(C, N), "bound": "mfma", "achieved": round(tf, 1),
-                           "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
-                           "traffic": traffic_of(traffic["standalone"], linear_kernel_name(C, N)) if default_workload else None,
-                           "algorithmic_flops_per_launch": flops, "avg_launch_ms": round(t_lin, 4),
-                           "launches_timed": launches("linear"),
-                           "note": "fp32-equivalent flops of the [N,16,C] x [C,C] channel mixing against the fp32 matrix "
-                                   "peak; the kernel computes them as six bf16 piece products per fp32 product on "
-                                   "v_mfma_f32_32x32x16_bf16 (6x the instruction flops: %.0f TFLOP/s of the 2500 TFLOP/s "
-                                   "bf16 peak) and is bound by its %d MB of memory traffic per launch"
-                                   % (6 * tf, 4 * (32 * N * C + 4 * C * C) // 10**6)})
+            lin_bytes = 4 * (32 * N * C + 4 * C * C)
+            others.append(entry(linear_kernel_name(C, N), lin_bytes, t_lin, launches_timed=launches("linear"),
+                                matrix_cores={"fp32_equivalent_TFLOP/s": round(tf, 1), "instruction_TFLOP/s_bf16": round(6 * tf, 1),
+                                              "frac_of_bf16_peak": round(6 * tf / 2500.0, 4)},
+                                note="[N,16,C] x [C,C] channel mixing: bound by its memory traffic, not by the matrix cores "
+                                     "(every fp32 product is six bf16 piece products on v_mfma_f32_32x32x16_bf16, which "
+                                     "keeps the pipes about a third busy)"))
+            others[-1]["traffic"] = traffic_of(traffic["standalone"], linear_kernel_name(C, N)) if default_workload else None
     else:
         # The model drives the tabulated ops through the TorchScript classes, which the Python-side brackets above do not
         # see: the two message-passing kernels are then timed on their own, on the step's edge list with random operands.
@@ -510,12 +549,28 @@ def main():
                          note="timed stand-alone on the step's edge list" if not launches(bwd_name) else "timed inside the step")
         others = [entry("mp_forward_kernel<%d>" % C, fwd_b, t_fwd)]
 
+    # two control figures that tell boxes of the pool apart: a streaming kernel (message passing with tabulated R at the
+    # step's shape, HBM-bound) and a loop of plain fp32 multiply-adds (VALU-bound)
+    rcv32 = data["edge_index"][0].int().contiguous()
+    snd32 = data["edge_index"][1].int().contiguous()
+    probe_out = torch.zeros(1, device="cuda")
+    wgs, iters = 256 * 8 * 4, 4096
+    t_probe = _time_ms(torch, lambda: cabi._check(cabi.lib.cm_probe_fma(probe_out.data_ptr(), wgs, iters, cabi._stream())), 5)
+    mp_case = op_cases(torch, cabi, N, E, C, ne, rcv32, snd32, with_fused=False, with_node_ops=False)[0]
+    t_stream = _time_ms(torch, mp_case[3], 5)
+    controls = {
+        "valu_fp32_fma_TFLOP/s": round(2 * 8 * iters * 256 * wgs / (t_probe * 1e-3) / 1e12, 1),
+        "valu_note": "plain v_fma_f32 loop, 8 independent chains per lane, 32 waves per compute unit, built without packed fp32 "
+                     "instructions like the rest of the library",
+        "hbm_stream_kernel": mp_case[1], "hbm_stream_GB/s": round(mp_case[2] / (t_stream * 1e-3) / 1e9, 1),
+        "hbm_stream_ms": round(t_stream, 4),
+    }
+    del mp_case
+
     # every stand-alone op of the path (the reference's op list: message passing with tabulated R[E,4,C] incl. the full
     # backward, harmonics, spline, contraction, linear) at the same shape, and configuration 2, each timed on its own
     standalone, config2 = None, None
     if not args.no_extras:
-        rcv32 = data["edge_index"][0].int().contiguous()
-        snd32 = data["edge_index"][1].int().contiguous()
         standalone, config2 = standalone_rooflines(torch, cabi, N, E, C, ne, rcv32, snd32)
         for row in standalone:
             row["traffic"] = traffic_of(traffic["standalone"], row["kernel"]) if default_workload else None
@@ -619,7 +674,8 @@ def main():
         "config": {"workload": "invariant MACE energy+forces, %d-atom periodic box at 0.1 atoms/A^3, %d edges, %dx0e, "
                                "l_max 3, correlation 3, %d elements, random-init weights (seed 0)" % (N, E, C, ne),
                    "atoms": N, "edges": E, "channels": C, "radial": "fused spline" if fused else "tabulated"},
-        "roofline": roofline, "roofline_other_kernels": others, "cpu_baseline": cpu_baseline,
+        "roofline": roofline, "stages_us": stages_us, "stages_sum_ms": stages_sum_ms, "controls": controls,
+        "roofline_other_kernels": others, "cpu_baseline": cpu_baseline,
         "neighbour_list": neighbour_list, "md_loop": md_loop, "with_stress": with_stress, "other_configs": configs,
     }
     if cpu_baseline:

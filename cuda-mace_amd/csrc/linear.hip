@@ -26,41 +26,15 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "mfma_split.hpp"
 
 namespace cm {
 namespace {
-
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 4;
 constexpr int kTileNodes = 32 * kWaves;  // rows per workgroup (MFMA M = 32 per wave)
 constexpr int kKC = 32;                  // K columns staged per step
 constexpr int kLdH = kKC + 8;            // padded LDS row stride of a bf16 plane (elements; 80 bytes: conflict-free b128 reads)
-
-// a = hi + mid + lo with bf16 pieces (round to nearest at every step; the remainders are exact in fp32).  Two values at a
-// time: the packed conversion rounds both and leaves the pieces in the order the matrix instruction takes them, and a
-// piece widens back to fp32 by a shift or a mask (11 instructions per pair; element by element the compiler converts
-// every value alone, widens it, and packs the pairs at the end with further conversions: 15).
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f2 __attribute__((ext_vector_type(2)));
-typedef unsigned u2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void split3_pair(float v0, float v1, unsigned &hi, unsigned &mid, unsigned &lo) {
-  hi = __builtin_bit_cast(unsigned, __builtin_convertvector(f2{v0, v1}, bf16x2));
-  const float r0 = v0 - __builtin_bit_cast(float, hi << 16), r1 = v1 - __builtin_bit_cast(float, hi & 0xffff0000u);
-  mid = __builtin_bit_cast(unsigned, __builtin_convertvector(f2{r0, r1}, bf16x2));
-  const float q0 = r0 - __builtin_bit_cast(float, mid << 16), q1 = r1 - __builtin_bit_cast(float, mid & 0xffff0000u);
-  lo = __builtin_bit_cast(unsigned, __builtin_convertvector(f2{q0, q1}, bf16x2));
-}
-__device__ __forceinline__ void split3(f4 v, bf16x4 &hi, bf16x4 &mid, bf16x4 &lo) {
-  unsigned h0, m0, l0, h1, m1, l1;
-  split3_pair(v.x, v.y, h0, m0, l0);
-  split3_pair(v.z, v.w, h1, m1, l1);
-  hi = __builtin_bit_cast(bf16x4, u2{h0, h1});
-  mid = __builtin_bit_cast(bf16x4, u2{m0, m1});
-  lo = __builtin_bit_cast(bf16x4, u2{l0, l1});
-}
 
 // Nout = 32 * NT; SCALED: X is multiplied by row_scale on the way in
 template <int NT, bool SCALED>
@@ -120,10 +94,13 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
   __syncthreads();
 
   if (zero_last_group && g == ngroups - 1) {
-    // rows that belong to no weight group: defined as zero
+    // rows that belong to no weight group: the product is defined as zero (a residual still passes through)
     for (int i = tid; i < kTileNodes * NOUT; i += kWaves * kWave) {
       const int node = sNode[i / NOUT];
-      if (node >= 0) OUT[(static_cast<int64_t>(node) * ncomp + m) * NOUT + i % NOUT] = 0.f;
+      if (node >= 0) {
+        const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + i % NOUT;
+        OUT[at] = residual ? residual[at] : 0.f;
+      }
     }
     return;
   }
@@ -332,7 +309,10 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
   if (zero_last_group && g == ngroups - 1) {
     for (int i = tid; i < kTileNodes * NOUT; i += kWaves * kWave) {
       const int node = sNode[i / NOUT];
-      if (node >= 0) OUT[(static_cast<int64_t>(node) * ncomp + m) * NOUT + i % NOUT] = 0.f;
+      if (node >= 0) {
+        const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + i % NOUT;
+        OUT[at] = residual ? residual[at] : 0.f;
+      }
     }
     return;
   }
@@ -601,7 +581,7 @@ __global__ __launch_bounds__(kResWaves *kWave, 1) void linear_resident_kernel(
     sCum[ngw] = cum;
   }
   if (zero_last_group && blockIdx.y == 0) {
-    // rows that belong to no weight group: defined as zero
+    // rows that belong to no weight group: the product is defined as zero (a residual still passes through)
     const int z0 = group_offsets[ngroups - 1], nz = group_offsets[ngroups] - z0;
     const int rowq = 16 * ldo / 4;
     const int64_t total = static_cast<int64_t>(nz) * rowq;

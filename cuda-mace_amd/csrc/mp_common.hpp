@@ -265,6 +265,12 @@ int launch_sliced_forward(const float *X, const float *vec, const float *knots, 
                           float r_max, const int32_t *sender, const int32_t *first_occ, int64_t nnodes, int64_t nedges,
                           int channels, float *out, hipStream_t st);
 
+// The spline-fused backward edge pass from edge vectors without gX, writing (this layer's vector gradient + addend[e])
+// (defined in mp_spline.hip; operands as cm_mp_edge_backward, already checked by the caller).
+int edge_backward_onto(const float *X, const float *vectors, const float *r_knots, const float *coeffs, int nknots, float r_width,
+                       float r_max, const float *grad_out, const int32_t *sender, const int32_t *first_occ, int64_t nnodes,
+                       int64_t nedges, int channels, float *grad_vectors, const float *addend, hipStream_t st);
+
 }  // namespace mp
 }  // namespace cm
 

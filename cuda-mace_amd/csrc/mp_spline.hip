@@ -249,9 +249,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
         if (lane_is_dead) {
           const int64_t e = pass_base + lane;
           if constexpr (FROM_VEC) {
-            gY[3 * e + 0] = 0.f;
-            gY[3 * e + 1] = 0.f;
-            gY[3 * e + 2] = 0.f;
+            gY[3 * e + 0] = g_r ? g_r[3 * e + 0] : 0.f;
+            gY[3 * e + 1] = g_r ? g_r[3 * e + 1] : 0.f;
+            gY[3 * e + 2] = g_r ? g_r[3 * e + 2] : 0.f;
           } else {
             if constexpr (WANT_GY) {
 #pragma unroll
@@ -370,9 +370,17 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
           for (int m = 0; m < 16; ++m) gy[m] = sGY[m * kChunk + lane];
           sh::vjp(d, gy, gin);
           const float gr = sGr[lane];
-          gY[3 * e + 0] = gin[0] + gr * d.y;
-          gY[3 * e + 1] = gin[1] + gr * d.z;
-          gY[3 * e + 2] = gin[2] + gr * d.x;
+          float o0 = gin[0] + gr * d.y, o1 = gin[1] + gr * d.z, o2 = gin[2] + gr * d.x;
+          if (g_r) {
+            // g_r doubles as an optional [E, 3] addend in this variant (another layer's gradient of the same vectors);
+            // the sum is formed from the rounded value, as a separate addition pass would form it
+            o0 = __fadd_rn(o0, g_r[3 * e + 0]);
+            o1 = __fadd_rn(o1, g_r[3 * e + 1]);
+            o2 = __fadd_rn(o2, g_r[3 * e + 2]);
+          }
+          gY[3 * e + 0] = o0;
+          gY[3 * e + 1] = o1;
+          gY[3 * e + 2] = o2;
         } else {
           if constexpr (WANT_GY) {
 #pragma unroll
@@ -401,7 +409,8 @@ void launch_edge(const float *X, const float *Y, const Spline &sp, const float *
                      dim3(kWave), 0, st, X, Y, sp, G, sender, first_occ, static_cast<int>(nnodes), nedges, gY, g_r, gXe);
 }
 
-// gY / g_r: outputs of the Y-and-r variant; in the FROM_VEC variant gY is the [E, 3] vector gradient and g_r is unused.
+// gY / g_r: outputs of the Y-and-r variant; in the FROM_VEC variant gY is the [E, 3] vector gradient and g_r, when given,
+// an [E, 3] addend to it (read only).
 template <int C, bool FROM_VEC>
 int launch_backward(const float *X, const float *Y, const Spline &sp, const float *G, const int32_t *sender,
                     const int32_t *first_occ, const int32_t *perm, const int32_t *offsets, int64_t nnodes, int64_t nedges,
@@ -504,6 +513,25 @@ extern "C" int cm_mp_edge_forward(const float *X, const float *vectors, const fl
   CM_DISPATCH_C(channels, rc = (cm::launch_forward<C_, true>(X, nullptr, sp, sender, first_occ, nnodes, nedges, out, cm::as_stream(stream))));
   return rc;
 }
+
+namespace cm {
+namespace mp {
+
+// cm_mp_edge_backward without gX whose vector gradient is written as (this layer's gradient + addend[e]): saves the pass
+// that adds two layers' gradients of the same edge vectors.  Arguments as checked by the caller (cm_mace_step).
+int edge_backward_onto(const float *X, const float *vectors, const float *r_knots, const float *coeffs, int nknots, float r_width,
+                       float r_max, const float *grad_out, const int32_t *sender, const int32_t *first_occ, int64_t nnodes,
+                       int64_t nedges, int channels, float *grad_vectors, const float *addend, hipStream_t st) {
+  if (nnodes == 0) return CM_OK;
+  const Spline sp{vectors, nullptr, r_knots, coeffs, nknots, r_width, r_max};
+  int rc = CM_EINVAL;
+  CM_DISPATCH_C(channels, rc = (launch_backward<C_, true>(X, nullptr, sp, grad_out, sender, first_occ, nullptr, nullptr, nnodes, nedges,
+                                                          nullptr, grad_vectors, const_cast<float *>(addend), nullptr, st)));
+  return rc;
+}
+
+}  // namespace mp
+}  // namespace cm
 
 extern "C" int cm_mp_edge_backward(const float *X, const float *vectors, const float *r_knots, const float *coeffs, int nknots,
                                    float r_width, float r_max, const float *grad_out, const int32_t *sender,

@@ -239,7 +239,13 @@ void *static_scratch_of_current_device() {
 }  // namespace
 }  // namespace cm
 
-extern "C" size_t cm_stable_key_sort_static_capacity(void) { return CM_SORT_STATIC_BYTES; }
+// Also the set-up call: looks the buffer's address up for the current device (when there is one), so that a later
+// cm_stable_key_sort_static on this device makes no runtime query and can be recorded into a stream capture.
+extern "C" size_t cm_stable_key_sort_static_capacity(void) {
+  int count = 0;
+  if (hipGetDeviceCount(&count) == hipSuccess && count > 0) (void)cm::static_scratch_of_current_device();
+  return CM_SORT_STATIC_BYTES;
+}
 
 extern "C" int cm_stable_key_sort_static(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm,
                                          int32_t *offsets, cm_stream_t stream) {

@@ -30,7 +30,7 @@ namespace cm {
 namespace {
 
 // ---- optional per-stage timing: events on the launch stream around chosen stages of the step --------------------
-constexpr int kStages = 24;
+constexpr int kStages = 25;
 struct Pending {
   int stage;
   hipEvent_t start, stop;
@@ -122,15 +122,6 @@ __global__ void live_range_kernel(const int32_t *__restrict__ first_occ, const f
   live[nnodes + n] = e;
 }
 
-// a += b, 16 bytes per lane where the length allows
-__global__ void add_f32_kernel(float *__restrict__ a, const float *__restrict__ b, int64_t n) {
-  const int64_t n4 = n / 4;
-  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n4;
-       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
-    st4(a + 4 * i, ld4(a + 4 * i) + ld4(b + 4 * i));
-  if (blockIdx.x == 0 && threadIdx.x < n - 4 * n4) a[4 * n4 + threadIdx.x] += b[4 * n4 + threadIdx.x];
-}
-
 // out[g] = sum of x over the nodes ptr[g] .. ptr[g + 1]: one workgroup per graph, every thread a strided partial sum, a
 // tree over the partials: the same order on every run.
 constexpr int kSumThreads = 1024;
@@ -211,6 +202,23 @@ __global__ __launch_bounds__(kSumThreads) void graph_virial_kernel(const double 
   }
 }
 
+// A fixed amount of dependent-free fp32 multiply-adds per lane, nothing else: what a box's vector ALUs deliver, for
+// telling boxes apart when the step's VALU-bound kernels differ between runs.
+__global__ __launch_bounds__(256) void probe_fma_kernel(float *out, int iters) {
+  float a[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) a[k] = 1.0f + 0.001f * static_cast<float>(threadIdx.x + k);
+  const float m = 0.999f, c = 0.0005f;
+  for (int i = 0; i < iters; ++i) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) a[k] = fmaf(a[k], m, c);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) sum += a[k];
+  if (sum == 123.456f) out[0] = sum;  // never true: keeps the loop
+}
+
 inline size_t align256(size_t n) { return (n + 255) & ~static_cast<size_t>(255); }
 
 // Carves the workspace; the same walk sizes it (base == nullptr) and lays it out.
@@ -243,6 +251,12 @@ struct Layout {
 
 }  // namespace
 }  // namespace cm
+
+extern "C" int cm_probe_fma(float *out, int workgroups, int iters, cm_stream_t stream) {
+  CM_REQUIRE(out && workgroups > 0 && iters > 0, "cm_probe_fma: NULL output or empty launch");
+  hipLaunchKernelGGL(cm::probe_fma_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(256), 0, cm::as_stream(stream), out, iters);
+  return cm::check_launch("cm_probe_fma");
+}
 
 extern "C" size_t cm_mace_step_workspace(int64_t nnodes, int64_t nedges, int channels) {
   if (nnodes < 0 || nedges < 0 || channels <= 0) return 0;
@@ -302,6 +316,11 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
     std::lock_guard<std::mutex> lock(cm::g_timing_mutex);
     timing_mask = cm::g_timing_mask;
   }
+  if (timing_mask != 0) {
+    // events recorded into a capture cannot be read back: a captured step is not timed
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) timing_mask = 0;
+  }
   if (N == 0) {
     hipLaunchKernelGGL(cm::fill_f64_kernel, dim3(1), dim3(64), 0, st, interaction_energy, static_cast<int64_t>(g->ngraphs), 0.0);
     if (virials)
@@ -329,17 +348,23 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   const float *none = nullptr;
 
   // ---- forward ----
-  CM_STAGE(0, cm_edge_geometry_forward(positions, g->receiver, g->sender, shifts, g->node_rows, N, E, L.vec, L.len, stream));
-  if (E > 0)
-    hipLaunchKernelGGL(cm::live_range_kernel, dim3(static_cast<unsigned>(cm::ceil_div(N, 256))), dim3(256), 0, st, g->first_occ, L.vec,
-                       w->r_max, static_cast<int>(N), E, L.live);
+  {
+    cm::StageTimer timer_(st, 0, timing_mask);
+    const int rc_ = cm_edge_geometry_forward(positions, g->receiver, g->sender, shifts, g->node_rows, N, E, L.vec, L.len, stream);
+    if (rc_ != CM_OK) return rc_;
+    if (E > 0)
+      hipLaunchKernelGGL(cm::live_range_kernel, dim3(static_cast<unsigned>(cm::ceil_div(N, 256))), dim3(256), 0, st, g->first_occ,
+                         L.vec, w->r_max, static_cast<int>(N), E, L.live);
+  }
   const int32_t *fo_forward = E > 0 ? L.live : g->first_occ;
   const float *X[2] = {g->X1, L.X2};
   float *bufM[2] = {L.bufM1, L.bufM2};
   float *B[2] = {L.B1, L.B2};
   float *h[2] = {L.h1, L.h2};
+  // the three [N, C] products between the layers (and their three transposes in the backward) as one launch each
+  const bool glue = cm_node_glue_supported(C) != 0;
   for (int t = 0; t < 2; ++t) {
-    if (t == 1) {
+    if (t == 1 && !glue) {
       // residual skip connection per element and linear_up, both of the first layer's output
       CM_STAGE(5, cm_linear(L.h1, w->skip_WT, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, w->skip_scale, none, none, L.sc, stream));
       CM_STAGE(6, cm_linear(L.h1, w->up_WT, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.X2, stream));
@@ -353,23 +378,31 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
     // the contraction's gradient table takes the place of the message, which is no longer needed
     CM_STAGE(t == 0 ? 3 : 9, cm_symcon_forward(L.bufA, el_perm, el_off, w->mono3[t], w->n3[t], w->mono2[t], w->n2[t], w->T3[t], w->T2[t], w->T1[t], N,
                               ne, C, B[t], bufM[t], stream));
-    CM_STAGE(t == 0 ? 4 : 10, cm_linear(B[t], w->prod_WT[t], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, t == 1 ? L.sc : none, h[t], stream));
+    if (t == 0 && glue)
+      CM_STAGE(4, cm_node_glue_forward(L.B1, w->prod_WT[0], w->skip_WT, w->up_WT, oh_perm, oh_off, N, ne + 1, C, w->skip_scale, L.h1, L.sc,
+                                       L.X2, stream));
+    else
+      CM_STAGE(t == 0 ? 4 : 10, cm_linear(B[t], w->prod_WT[t], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, t == 1 ? L.sc : none, h[t], stream));
   }
   CM_STAGE(11, cm_readout_forward(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden, node_energy,
                              L.d_h2, node_feats, g->node_rows, stream));
-  hipLaunchKernelGGL(cm::segment_sum_f64_kernel, dim3(g->ngraphs), dim3(cm::kSumThreads), 0, st, node_energy, g->node_weights,
-                     g->graph_ptr, interaction_energy);
+  {
+    cm::StageTimer timer_(st, 12, timing_mask);
+    hipLaunchKernelGGL(cm::segment_sum_f64_kernel, dim3(g->ngraphs), dim3(cm::kSumThreads), 0, st, node_energy, g->node_weights,
+                       g->graph_ptr, interaction_energy);
+  }
 
   // ---- backward: d(-sum of node energies) / d positions ----
   // The seed is -1 on every node energy (-weight[n] with node weights), so the readouts' backward needs no pass of its
   // own: the gradient with respect to the second layer's features is -d_h2 (the sign goes into the scale of the two
   // linears that consume it, which is exact; node weights scale its rows first), the one with respect to the first
   // layer's is a constant row (times the node's weight).
-  {
+  if (!glue || g->node_weights) {
     cm::StageTimer timer_(st, 13, timing_mask);
     const dim3 grid(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(N * C, 256), 2048)));
-    hipLaunchKernelGGL(cm::seed_linear_readout_kernel, grid, dim3(256), 0, st, L.g1, w->w1, w->scale, g->node_weights,
-                       static_cast<int64_t>(N) * C, C);
+    if (!glue)  // the glue kernel forms the constant rows itself
+      hipLaunchKernelGGL(cm::seed_linear_readout_kernel, grid, dim3(256), 0, st, L.g1, w->w1, w->scale, g->node_weights,
+                         static_cast<int64_t>(N) * C, C);
     if (g->node_weights)
       hipLaunchKernelGGL(cm::weight_rows_kernel, grid, dim3(256), 0, st, L.d_h2, g->node_weights, static_cast<int64_t>(N) * C, C);
   }
@@ -378,19 +411,23 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   CM_STAGE(15, cm_linear(L.bufM2, w->mix_W[1], nullptr, nullptr, N, 1, 0, 16, C, C, w->mix_scale[1], L.gB, none, L.bufA, stream));
   CM_STAGE(16, cm_mp_edge_backward(L.X2, L.vec, w->r_knots, w->spline[1], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
                               g->first_occ, g->sender_perm, g->sender_offsets, N, E, C, L.gX2, L.gv2, L.edge_scratch, stream));
-  CM_STAGE(17, cm_linear(L.gX2, w->up_W, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, L.g1, L.gh1a, stream));
-  CM_STAGE(18, cm_linear(L.d_h2, w->skip_W, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, -w->skip_scale, none, L.gh1a, L.gh1, stream));
   // layer 0 (first interaction): its input features depend on the species alone, so no gradient with respect to them
-  CM_STAGE(19, cm_linear(L.gh1, w->prod_W[0], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.gB, stream));
+  if (glue) {
+    CM_STAGE(17, cm_node_glue_backward(L.gX2, L.d_h2, w->up_W, w->skip_W, w->prod_W[0], w->w1, w->scale, g->node_weights, oh_perm, oh_off, N,
+                                       ne + 1, C, w->skip_scale, L.gB, stream));
+  } else {
+    CM_STAGE(17, cm_linear(L.gX2, w->up_W, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, L.g1, L.gh1a, stream));
+    CM_STAGE(18, cm_linear(L.d_h2, w->skip_W, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, -w->skip_scale, none, L.gh1a, L.gh1, stream));
+    CM_STAGE(19, cm_linear(L.gh1, w->prod_W[0], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.gB, stream));
+  }
   CM_STAGE(20, cm_linear(L.bufM1, w->mix_W[0], oh_perm, oh_off, N, ne + 1, 1, 16, C, C, w->mix_scale[0], L.gB, none, L.bufA, stream));
-  CM_STAGE(21, cm_mp_edge_backward(g->X1, L.vec, w->r_knots, w->spline[0], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
-                              g->first_occ, nullptr, nullptr, N, E, C, nullptr, L.gv1, nullptr, stream));
-  if (E > 0)
-    hipLaunchKernelGGL(cm::add_f32_kernel, dim3(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(3 * E, 4 * 256), 2048))),
-                       dim3(256), 0, st, L.gv1, L.gv2, 3 * E);
+  // its vector gradient is written onto the second layer's: gv1 = (this layer's) + gv2
+  CM_STAGE(21, cm::mp::edge_backward_onto(g->X1, L.vec, w->r_knots, w->spline[0], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
+                                         g->first_occ, N, E, C, L.gv1, L.gv2, st));
   CM_STAGE(23, cm_edge_geometry_backward(positions, g->receiver, g->sender, shifts, g->node_rows, g->first_occ, g->sender_perm,
                                     g->sender_offsets, L.gv1, nullptr, N, E, forces, nullptr, stream));
   if (virials) {
+    cm::StageTimer timer_(st, 24, timing_mask);
     if (N > 0)
       hipLaunchKernelGGL(cm::node_virial_kernel, dim3(static_cast<unsigned>(cm::ceil_div(8 * N, 256))), dim3(256), 0, st, L.vec, L.gv1,
                        g->first_occ, static_cast<int>(N), E, L.node_virial);

@@ -64,12 +64,16 @@ SIGNATURES = {
     "cm_symcon_backward": (_i32, [_p, _p, _i64, _i32, _p, _p]),
     "cm_readout_forward": (_i32, [_p] * 5 + [_f64, _f64, _f64, _i64, _i32, _i32, _p, _p, _p, _p, _p]),
     "cm_readout_backward": (_i32, [_p, _p, _p, _f64, _i64, _i32, _p, _p, _p]),
+    "cm_node_glue_supported": (_i32, [_i32]),
+    "cm_node_glue_forward": (_i32, [_p] * 6 + [_i64, _i32, _i32, _f32, _p, _p, _p, _p]),
+    "cm_node_glue_backward": (_i32, [_p] * 6 + [_f64, _p, _p, _p, _i64, _i32, _i32, _f32, _p, _p]),
     "cm_neighbour_list_workspace": (_sz, [_i64, _i64]),
     "cm_neighbour_list_count": (_i32, [_p, _p, _i32, _i32, _i32, _f64, _i64, _i64, _p, _sz, _p, _p, _p]),
     "cm_neighbour_list_fill": (_i32, [_p, _f64, _i64, _i64, _p, _p, _i64, _p, _p, _p, _p, _p]),
     "cm_max_displacement": (_i32, [_p, _p, _i64, _p, _p]),
     # the whole step: (weights struct *, graph struct *, positions, shifts, workspace, bytes, 4 outputs, stream)
     "cm_mace_step_timing": (_i32, [ctypes.c_uint]),
+    "cm_probe_fma": (_i32, [_p, _i32, _i32, _p]),
     "cm_mace_step_timing_read": (_i32, [_p, _p, _i32]),
     "cm_mace_step_workspace": (_sz, [_i64, _i64, _i32]),
     "cm_mace_step": (_i32, [_p, _p, _p, _p, _p, _sz, _p, _p, _p, _p, _p, _p]),
@@ -450,6 +454,43 @@ def linear(X, W_T, node_perm=None, group_offsets=None, scale=None, zero_last_gro
         )
     )
     return OUT
+
+
+def node_glue_forward(B1, prod_WT, skip_WT, up_WT, node_perm, group_offsets, skip_scale: float):
+    """(h1, sc, X2) = (B1 . prod_W, skip_scale * h1 . skip_W[element], h1 . up_W) in one launch; weights transposed
+    ([C out, C in], skip_WT [nelements, C, C]); the grouping has nelements + 1 groups, the last for nodes without an
+    element (sc = 0 there)."""
+    N, C = B1.shape
+    ne = skip_WT.shape[0]
+    if tuple(prod_WT.shape) != (C, C) or tuple(up_WT.shape) != (C, C) or tuple(skip_WT.shape) != (ne, C, C):
+        raise CudaMaceError("node_glue_forward: weights must be [C, C], [nelements, C, C], [C, C]")
+    if group_offsets.numel() != ne + 2 or node_perm.numel() != N:
+        raise CudaMaceError("node_glue_forward: the grouping must list N nodes in nelements + 1 groups")
+    h1, sc, X2 = (torch.empty(N, C, dtype=F32, device=B1.device) for _ in range(3))
+    _check(lib.cm_node_glue_forward(_dev(B1, F32, "B1"), _dev(prod_WT, F32, "prod_WT"), _dev(skip_WT, F32, "skip_WT"),
+                                    _dev(up_WT, F32, "up_WT"), _dev(node_perm, I32, "node_perm"),
+                                    _dev(group_offsets, I32, "group_offsets"), N, ne + 1, C, float(skip_scale),
+                                    _dev(h1, F32, "h1"), _dev(sc, F32, "sc"), _dev(X2, F32, "X2"), _stream()))
+    return h1, sc, X2
+
+
+def node_glue_backward(gX2, d_h2, up_W, skip_W, prod_W, w1, scale: float, node_weights, node_perm, group_offsets,
+                       skip_scale: float):
+    """gB1 = (gX2 . up_W^T + g1 - skip_scale * d_h2 . skip_W[element]^T) . prod_W^T with g1[n, c] = -node_weights[n] *
+    scale * w1[c] (node_weights None = 1); weights plain ([C in, C out] passed as the transposes of the forward's)."""
+    N, C = gX2.shape
+    ne = skip_W.shape[0]
+    if tuple(d_h2.shape) != (N, C) or tuple(up_W.shape) != (C, C) or tuple(prod_W.shape) != (C, C) or tuple(skip_W.shape) != (ne, C, C):
+        raise CudaMaceError("node_glue_backward: operands must be [N, C] and weights [C, C], [nelements, C, C], [C, C]")
+    if group_offsets.numel() != ne + 2 or node_perm.numel() != N or w1.numel() != C:
+        raise CudaMaceError("node_glue_backward: the grouping must list N nodes in nelements + 1 groups, w1 holds C values")
+    gB1 = torch.empty(N, C, dtype=F32, device=gX2.device)
+    _check(lib.cm_node_glue_backward(_dev(gX2, F32, "gX2"), _dev(d_h2, F32, "d_h2"), _dev(up_W, F32, "up_W"),
+                                     _dev(skip_W, F32, "skip_W"), _dev(prod_W, F32, "prod_W"), _dev(w1, F64, "w1"), float(scale),
+                                     _dev(node_weights, F64, "node_weights"), _dev(node_perm, I32, "node_perm"),
+                                     _dev(group_offsets, I32, "group_offsets"), N, ne + 1, C, float(skip_scale),
+                                     _dev(gB1, F32, "gB1"), _stream()))
+    return gB1
 
 
 # ---- symmetric contraction -----------------------------------------------------------------------------

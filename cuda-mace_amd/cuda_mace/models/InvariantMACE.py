@@ -23,7 +23,7 @@ from cuda_mace.ops.spherical_harmonics import SphericalHarmonics
 from cuda_mace.ops.symmetric_contraction import SymmetricContraction as CUDAContraction
 from cuda_mace import _cabi as cabi
 from cuda_mace.ops._autograd import (EdgeGeometryAutograd, LinearContractionAutograd, ReadoutEnergyAutograd, ScalarLinearAutograd,
-                                     _cached, _cached_for, groups_of, groups_of_one_hot, monomials_from_packed)
+                                     _cached, _cached_for, _cached_per, groups_of, groups_of_one_hot, monomials_from_packed)
 from cuda_mace.utils.irreps import Instruction
 
 
@@ -605,12 +605,14 @@ class OptimizedInvariantMACE(torch.nn.Module):
 
         if native is not None:
             rows32 = None if node_rows is None else node_rows[0]
-            handle = _cached_for(edge_index, "_cm_native_graph_%d" % id(self._weights_token), node_attrs,
+            # one entry per model on the list's tensor, keyed on this model's weights token itself (the handle holds
+            # X1, which depends on this model's weights)
+            handle = _cached_per(edge_index, "_cm_native_graphs", self._weights_token, node_attrs,
                                  lambda: native.graph(edge_index, receiver, sender, node_attrs32, atom_types, data["ptr"],
                                                       node_feats_up, rows32))
             if node_weights is not None:
                 plain = handle
-                handle = _cached_for(data["node_weights"], "_cm_native_graph_weighted_%d" % id(self._weights_token), plain,
+                handle = _cached_per(data["node_weights"], "_cm_native_graphs_weighted", self._weights_token, plain,
                                      lambda: plain.with_node_weights(node_weights))
             want_virials = compute_virials or compute_stress
             res = native(handle, positions, shifts, want_virials=want_virials)

@@ -12,6 +12,7 @@ instead of once per call.
 from __future__ import annotations
 
 import functools
+import weakref
 
 import numpy as np
 import torch
@@ -72,6 +73,36 @@ def _cached_for(owner: torch.Tensor, slot: str, other, build):
         return hit[2]
     val = build()
     owner.__dict__[slot] = (other, tag, val)
+    return val
+
+
+class _PerToken(weakref.WeakKeyDictionary):
+    """Cache entries per weights token; a copy or a pickle of the tensor that carries it starts empty (the entries
+    hold device addresses and belong to live model objects)."""
+
+    def __reduce__(self):
+        return (_PerToken, ())
+
+    def __deepcopy__(self, memo):
+        return _PerToken()
+
+    def __copy__(self):
+        return _PerToken()
+
+
+def _cached_per(owner: torch.Tensor, slot: str, token, other, build):
+    """As `_cached_for`, with one entry per `token` (an object that stands for one model's weights) kept on `owner`.
+    Tokens are held weakly: an entry disappears with its model, so the id of a dead token can never be taken for a
+    live one's, and several models evaluated on the same tensors do not evict each other."""
+    table = owner.__dict__.get(slot)
+    if table is None:
+        table = owner.__dict__[slot] = _PerToken()
+    tag = (owner._version, owner.data_ptr(), getattr(other, "_version", 0))
+    hit = table.get(token)
+    if hit is not None and hit[0] is other and hit[1] == tag:
+        return hit[2]
+    val = build()
+    table[token] = (other, tag, val)
     return val
 
 

@@ -131,9 +131,15 @@ class NativeStep:
         if pos64.shape != (N, 3) or sh64.shape != (E, 3):
             raise cabi.CudaMaceError("native step: positions must be [%d, 3] and shifts [%d, 3]" % (N, E))
         need = cabi.lib.cm_mace_step_workspace(N, E, C)
-        ws = self._workspace
-        if ws is None or ws.numel() < need or ws.device != dev:
-            ws = self._workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+        if torch.cuda.is_current_stream_capturing():
+            # A captured step keeps the address it was recorded with for as long as its graph lives: its workspace comes
+            # from the capture's own memory pool (which the graph owns), never from the buffer eager calls share, which a
+            # later, larger evaluation replaces.
+            ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        else:
+            ws = self._workspace
+            if ws is None or ws.numel() < need or ws.device != dev:
+                ws = self._workspace = torch.empty(need, dtype=torch.uint8, device=dev)
         energy = torch.empty(int(g.ngraphs), dtype=F64, device=dev)
         node_energy = torch.empty(N, dtype=F64, device=dev)
         forces = torch.empty(N, 3, dtype=F64, device=dev)

@@ -92,6 +92,9 @@ int cm_stable_key_sort(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *p
  * allocates nothing.  It returns CM_ENOSPC when cm_stable_key_sort_workspace(n, nkeys) = 4 * (n + 2 * nkeys) bytes
  * (rounded up to 256) exceeds that capacity.  All calls on one GPU share that GPU's buffer: calls that may overlap
  * on one GPU (different streams, different threads) race and must be serialised by the caller.
+ * The first use on a GPU looks the buffer's address up (a runtime query, not to be made while a stream is capturing):
+ * before a capture, call cm_stable_key_sort_static_capacity() with that GPU current (it performs the lookup) or make
+ * one sort call; after that a call enqueues kernels only and can be recorded into a HIP graph.
  */
 size_t cm_stable_key_sort_static_capacity(void);
 int cm_stable_key_sort_static(const int32_t *keys, int64_t n, int64_t nkeys, int32_t *perm,
@@ -413,6 +416,29 @@ int cm_readout_backward(const double *grad_node_energies, const double *w1, cons
                         int64_t nnodes, int channels, float *grad_h1, float *grad_h2, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * The three [nnodes, C] x [C, C] linears between the two interaction layers as one launch per direction: the product's
+ * linear and linear_up (the reference's linear_matmul, models/InvariantMACE.py:41-53) and the per-element skip
+ * connection between them (element_linear_to_cuda, :56-74; called at :145-150 and :330).  A workgroup takes 128 nodes
+ * of one element through the chain with the intermediate rows in LDS; same arithmetic, rounding points and results as
+ * the three cm_linear calls it stands for.  channels = 32, 64, 96 or 128 (cm_node_glue_supported).
+ *   node_perm / group_offsets: nodes grouped by element, ngroups = nelements + 1 with the last group holding the nodes
+ *   without an element (their skip connection is zero), as cm_linear takes them with zero_last_group.
+ * Forward:  h1 = B1 . prod_W;  sc = skip_scale * h1 . skip_W[element];  X2 = h1 . up_W       (all fp32 [nnodes, C];
+ *   weights passed transposed, [C out, C in], skip_WT [nelements, C, C]).
+ * Backward: gB1 = (gX2 . up_W^T + g1 - skip_scale * d_h2 . skip_W[element]^T) . prod_W^T with
+ *   g1[n, c] = -node_weights[n] * scale * w1[c] (node_weights may be NULL = 1): the gradient of minus the weighted sum of
+ *   node energies (cm_readout_forward's d_h2, scale, w1) through the chain; weights passed plain, [C in, C out].
+ */
+int cm_node_glue_supported(int channels);
+int cm_node_glue_forward(const float *B1, const float *prod_WT, const float *skip_WT, const float *up_WT,
+                         const int32_t *node_perm, const int32_t *group_offsets, int64_t nnodes, int ngroups, int channels,
+                         float skip_scale, float *h1, float *sc, float *X2, cm_stream_t stream);
+int cm_node_glue_backward(const float *gX2, const float *d_h2, const float *up_W, const float *skip_W, const float *prod_W,
+                          const double *w1, double scale, const double *node_weights, const int32_t *node_perm,
+                          const int32_t *group_offsets, int64_t nnodes, int ngroups, int channels, float skip_scale,
+                          float *gB1, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * One energy + forces evaluation of the two-layer invariant model as a single call: every kernel of the step, forward
  * and backward, enqueued back to back by the library itself.  It replaces, for inference, what the reference runs as a
  * Python forward over its TorchScript classes followed by an autograd backward (models/InvariantMACE.py:246-379:
@@ -484,13 +510,18 @@ typedef struct cm_mace_graph {
 /* Per-stage timing of cm_mace_step (off by default): with bit s of stage_mask set, stage s of every later step is
  * bracketed by two events recorded on the launch stream; cm_mace_step_timing_read waits for the outstanding events and
  * returns, per stage, the accumulated milliseconds and the number of timed launches since the mask was set (arrays of
- * at least 24 entries; the return value is the number of stages).  Setting a mask resets the accumulators.  Leave it
- * off while a step is being captured into a graph.  Stages: 0 edge geometry; 1 / 7 message passing forward of layer
- * 0 / 1; 2 / 8 channel mixing; 3 / 9 contraction; 4 / 10 linear after it; 5 skip connection; 6 linear_up; 11 readouts;
- * 13 readout backward; 14 / 19 linear after the contraction, backward; 15 / 20 channel mixing backward (contraction
+ * at least 25 entries; the return value is the number of stages).  Setting a mask resets the accumulators.  A step
+ * enqueued while its stream is capturing is not timed (events recorded into a capture cannot be read back).  Stages: 0 edge geometry and live edge ranges; 1 / 7 message passing forward of layer
+ * 0 / 1; 2 / 8 channel mixing; 3 / 9 contraction; 4 / 10 linear after it; 5 skip connection; 6 linear_up; 11 readouts; 12 energy sums per graph;
+ * 13 seeds of the backward chain; 14 / 19 linear after the contraction, backward; 15 / 20 channel mixing backward (contraction
  * backward folded in); 16 message passing backward of layer 1 (edge pass + sender pass); 21 of layer 0 (edge pass
- * only); 17 linear_up backward; 18 skip backward; 23 edge geometry backward (forces). */
+ * only); 17 linear_up backward; 18 skip backward; 22 sum of the two layers' per-edge gradients; 23 edge geometry backward
+ * (forces); 24 virials. */
 int cm_mace_step_timing(unsigned stage_mask);
+/* A control launch for benchmarks (no counterpart in the reference): `workgroups` workgroups of 256 lanes, each lane
+ * 8 * iters independent fp32 multiply-adds and nothing else (2 * 8 * iters * 256 * workgroups flop); out: one float the
+ * kernel never writes.  Timed by the caller, it tells what the vector ALUs of this box deliver. */
+int cm_probe_fma(float *out, int workgroups, int iters, cm_stream_t stream);
 int cm_mace_step_timing_read(double *total_ms, int64_t *launches, int capacity);
 size_t cm_mace_step_workspace(int64_t nnodes, int64_t nedges, int channels);
 int cm_mace_step(const cm_mace_weights *weights, const cm_mace_graph *graph, const double *positions, const double *shifts,

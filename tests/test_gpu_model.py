@@ -408,3 +408,58 @@ def test_native_step_on_a_list_with_a_skin(cabi, relabel):
     torch.testing.assert_close(a["forces"], b["forces"].detach(), rtol=0, atol=5e-7 * fscale)
     torch.testing.assert_close(a["energy"], c["energy"], rtol=1e-6, atol=1e-6)
     torch.testing.assert_close(a["forces"], c["forces"], rtol=0, atol=2e-6 * fscale)
+
+
+def test_a_second_model_on_the_same_tensors_gets_its_own_graph_handle(cabi):
+    """Model A evaluated on a batch and deleted, model B (other weights) built and evaluated on the very same tensors,
+    several times over so that B's cache token can land on A's freed address: B's one-call step must use B's own first-layer
+    features, i.e. agree with B's autograd path, and differ from A's result."""
+    import gc
+
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+
+    data = make_system(120, 4, seed=8, density=0.1)
+    dev = to_device(data, "cuda")
+    avg = data["edge_index"].shape[1] / 120
+    last = None
+    for seed in range(6):
+        up = SyntheticInvariantMACE(channels=32, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=avg, seed=seed)
+        model = OptimizedInvariantMACE(up, device="cuda", native_step=True)
+        out = model(dict(dev))
+        assert model._native not in (None, False)
+        check = OptimizedInvariantMACE(up, device="cuda", native_step=False)(dict(dev))
+        assert torch.equal(out["node_energy"], check["node_energy"].detach()), "seed %d ran on another model's handle" % seed
+        if last is not None:
+            assert not torch.equal(out["node_energy"], last)
+        last = out["node_energy"].clone()
+        del model, out, check, up
+        gc.collect()
+
+
+def test_captured_step_survives_a_larger_eager_evaluation(cabi):
+    """A step captured as a HIP graph keeps its own workspace: evaluating the same model eagerly on a larger structure
+    afterwards (which replaces the buffer eager calls share) must not disturb the replays."""
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.utils.graph import GraphedStep
+
+    small, large = make_system(130, 4, seed=3, density=0.1), make_system(700, 4, seed=4, density=0.1)
+    up = SyntheticInvariantMACE(channels=64, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=50.0, seed=2)
+    model = OptimizedInvariantMACE(up, device="cuda")
+    dev_small, dev_large = to_device(small, "cuda"), to_device(large, "cuda")
+    step = GraphedStep(model, dev_small)
+    first = {k: v.clone() for k, v in step().items() if k in ("energy", "forces", "node_energy")}
+    big = model(dict(dev_large))
+    torch.cuda.synchronize()
+    big2 = model(dict(dev_large))
+    # the eager buffer was replaced and is in use by other work; the replay still reads and writes its own
+    for _ in range(3):
+        again = step()
+        torch.cuda.synchronize()
+        for k, v in first.items():
+            assert torch.equal(again[k], v), k
+        junk = torch.randn(1 << 22, device="cuda")  # allocator traffic between replays
+        del junk
+    fresh = model(dict(dev_small))
+    for k, v in first.items():
+        assert torch.equal(fresh[k].detach(), v), k
+    assert torch.equal(big["forces"], big2["forces"])

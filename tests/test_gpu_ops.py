@@ -335,6 +335,53 @@ def test_scalar_elemental_linear_and_zero_group(cabi, N, K, Nout, ne, seed):
     close(out16, ref16, 1e-5, 2e-6)
 
 
+@pytest.mark.parametrize("N,C,ne,seed", [(1, 32, 1, 0), (21, 64, 4, 1), (700, 128, 10, 2), (5000, 96, 10, 3), (25000, 128, 10, 4)])
+def test_node_glue_chains(cabi, N, C, ne, seed):
+    """The three [N, C] linears between the layers as one launch per direction: against the fp64 definition, and bit for
+    bit against the three separate launches of the linear kernel they stand for (rows without an element included)."""
+    _say("node_glue", N, C, ne, seed)
+    g = torch.Generator().manual_seed(seed)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float64)  # noqa: E731
+    B1, gX2, d_h2 = rnd(N, C), rnd(N, C), rnd(N, C)
+    Wp, Wu, Ws = rnd(C, C) / math.sqrt(C), rnd(C, C) / math.sqrt(C), rnd(ne, C, C)
+    w1, nw = rnd(C), torch.rand(N, generator=g, dtype=torch.float64)
+    scale, skip_scale = 0.8, 1.0 / math.sqrt(C * ne)
+    elem = torch.randint(0, ne + 1, (N,), generator=g)  # value ne = "no element"
+    Ws0 = torch.cat([Ws, torch.zeros(1, C, C, dtype=torch.float64)])[elem]  # [N, C, C]
+    h1_ref = B1 @ Wp
+    sc_ref = skip_scale * torch.einsum("nk,nkj->nj", h1_ref, Ws0)
+    X2_ref = h1_ref @ Wu
+    f32 = lambda t: t.float().to(DEV).contiguous()  # noqa: E731
+    T = lambda t: t.transpose(-1, -2).contiguous()  # noqa: E731
+    perm, off = cabi.stable_key_sort(elem.int().to(DEV), ne + 1)
+    h1, sc, X2 = cabi.node_glue_forward(f32(B1), f32(T(Wp)), f32(T(Ws)), f32(T(Wu)), perm, off, skip_scale)
+    close(h1, h1_ref, 1e-5, 2e-6)
+    close(sc, sc_ref, 1e-5, 2e-6)
+    close(X2, X2_ref, 1e-5, 2e-6)
+    assert float(sc[(elem == ne).to(DEV)].abs().sum()) == 0.0
+    h1_s = cabi.linear(f32(B1), f32(T(Wp)), scale=1.0)
+    sc_s = cabi.linear(h1_s, f32(T(Ws)), perm, off, scale=skip_scale, zero_last_group=True)
+    X2_s = cabi.linear(h1_s, f32(T(Wu)), scale=1.0)
+    assert torch.equal(h1, h1_s) and torch.equal(sc, sc_s) and torch.equal(X2, X2_s)
+    for weights in (None, nw):
+        wn = torch.ones(N, dtype=torch.float64) if weights is None else weights
+        g1_ref = (-1.0 * scale * w1)[None, :] * wn[:, None]  # the kernel's order of the fp64 products
+        gh1_ref = gX2 @ Wu.t() + g1_ref - skip_scale * torch.einsum("nj,nkj->nk", d_h2, Ws0)
+        gB_ref = gh1_ref @ Wp.t()
+        gB = cabi.node_glue_backward(f32(gX2), f32(d_h2), f32(Wu), f32(Ws), f32(Wp), w1.to(DEV), scale,
+                                     None if weights is None else weights.to(DEV), perm, off, skip_scale)
+        close(gB, gB_ref, 1e-5, 2e-6)
+        g1 = f32(g1_ref)  # rounded once from the fp64 product, as the kernel forms it
+        a = cabi.linear(f32(gX2), f32(Wu), scale=1.0, residual=g1)
+        b = cabi.linear(f32(d_h2), f32(Ws), perm, off, scale=-skip_scale, zero_last_group=True, residual=a)
+        c = cabi.linear(b, f32(Wp), scale=1.0)
+        assert torch.equal(gB, c)
+    with pytest.raises(cabi.CudaMaceError, match="32, 64, 96 or 128"):
+        cabi.node_glue_forward(torch.zeros(4, 160, device=DEV), torch.zeros(160, 160, device=DEV), torch.zeros(1, 160, 160, device=DEV),
+                               torch.zeros(160, 160, device=DEV), torch.zeros(4, dtype=torch.int32, device=DEV),
+                               torch.zeros(3, dtype=torch.int32, device=DEV), 1.0)
+
+
 @pytest.mark.parametrize("N,C,ne,seed", [(2048, 128, 1, 0), (2500, 128, 10, 1), (4099, 96, 5, 2), (3000, 64, 3, 3), (6000, 128, 130, 4)])
 def test_linear_many_rows(cabi, N, C, ne, seed):
     """16-component features with at least 2048 nodes and 64 / 96 / 128 square weights run on the kernel that keeps the

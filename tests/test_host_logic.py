@@ -194,3 +194,49 @@ def test_coupling_tensor_checks():
     del con.U_matrix_2
     with pytest.raises(ValueError, match="orders"):
         SymmetricContraction(up, device="cpu")
+
+
+def test_per_model_cache_survives_a_recycled_token_id():
+    """Entries kept on a tensor per model are keyed on the model's token object, weakly: when a model dies its entry
+    goes with it, so a new model whose token lands on the same address (same id) never sees the old value; two live
+    models keep one entry each; a pickle or a copy of the tensor starts without entries."""
+    import copy
+    import gc
+    import io
+
+    from cuda_mace.models.InvariantMACE import _WeightsToken
+    from cuda_mace.ops._autograd import _cached_per
+
+    owner, other = torch.arange(5), torch.zeros(3)
+    builds = []
+
+    def build_for(name):
+        def build():
+            builds.append(name)
+            return name
+        return build
+
+    seen_ids, recycled = set(), False
+    for round_ in range(200):  # CPython hands a freed object's address to the next object of that size
+        tok = _WeightsToken()
+        recycled |= id(tok) in seen_ids
+        seen_ids.add(id(tok))
+        name = "model %d" % round_
+        assert _cached_per(owner, "_slot", tok, other, build_for(name)) == name
+        assert _cached_per(owner, "_slot", tok, other, build_for("never built")) == name  # a hit while the model lives
+        del tok
+        gc.collect()
+        assert len(owner.__dict__["_slot"]) == 0
+    assert recycled and len(builds) == 200
+    a, b = _WeightsToken(), _WeightsToken()
+    assert _cached_per(owner, "_slot", a, other, build_for("A")) == "A"
+    assert _cached_per(owner, "_slot", b, other, build_for("B")) == "B"
+    assert _cached_per(owner, "_slot", a, other, build_for("A2")) == "A"  # B did not evict A
+    other.add_(1)  # the tensor the value was derived from changed in place
+    assert _cached_per(owner, "_slot", a, other, build_for("A3")) == "A3"
+    buf = io.BytesIO()
+    torch.save(owner, buf)
+    buf.seek(0)
+    loaded = torch.load(buf, weights_only=False)
+    assert torch.equal(loaded, owner) and len(loaded.__dict__.get("_slot", {})) == 0
+    assert len(copy.deepcopy(owner).__dict__["_slot"]) == 0

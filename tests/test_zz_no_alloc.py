@@ -53,3 +53,28 @@ def test_static_sort_rejects_sizes_beyond_its_buffer():
     offsets = torch.empty(2, dtype=torch.int32, device=dev)
     with pytest.raises(_cabi.CudaMaceError, match="built-in"):
         _cabi.stable_key_sort_static(keys, 1, perm, offsets)
+
+
+def test_static_sort_inside_a_captured_graph():
+    """After the set-up call the entry point only enqueues kernels: recorded into a HIP graph, every replay sorts the
+    keys that are in the input buffer at that time."""
+    from cuda_mace import _cabi
+
+    dev = torch.device("cuda:0")
+    assert _cabi.lib.cm_stable_key_sort_static_capacity() == 32 << 20  # looks the buffer up for this device
+    n, nkeys = 20_000, 700
+    keys = _pair(n, nkeys, 11, dev)
+    perm = torch.empty(n, dtype=torch.int32, device=dev)
+    offsets = torch.empty(nkeys + 1, dtype=torch.int32, device=dev)
+    _cabi.stable_key_sort_static(keys, nkeys, perm, offsets)  # warm call outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _cabi.stable_key_sort_static(keys, nkeys, perm, offsets)
+    for seed in (12, 13, 14):
+        keys.copy_(_pair(n, nkeys, seed, dev))
+        perm.fill_(-1), offsets.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        want_perm, want_off = _cabi.stable_key_sort(keys, nkeys)
+        assert torch.equal(perm, want_perm) and torch.equal(offsets, want_off), seed
