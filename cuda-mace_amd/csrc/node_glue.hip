@@ -14,11 +14,21 @@
 // v_mfma_f32_32x32x16_bf16, K in chunks of 32), and every intermediate is rounded to fp32 where the separate launches
 // store it, so the chain returns the bits of the separate launches.
 //
+// A third kernel does the same at the end of the forward, where the second layer's product linear, both readouts and
+// the transpose of that linear follow each other on the same rows (reference: models/InvariantMACE.py:330-343 and its
+// backward):
+//
+//   h2 = B2 . Wprod2 + sc      E_n, dE/dh2, feats = readouts(h1, h2)      gB2 = -dE/dh2 . Wprod2^T
+//
+// h2 only ever exists as the LDS tile (the model returns it inside the fp64 feature concatenation).
+//
 // g1 and g2 are the gradients of minus the (weighted) sum of node energies with respect to the two layers' features:
 // g1[n, c] = -weight[n] scale w1[c] is formed here from the linear readout's weights; g2 = -dE/dh2 arrives as dE/dh2 and
 // its sign goes into the scale of the skip product.
 #include "common.hpp"
 #include "mfma_split.hpp"
+#include "node_glue.hpp"
+#include "readout_device.hpp"  // before the pragma below: the readouts' fp64 arithmetic compiles as in readout.hip
 
 // Products and the additions that follow them stay separate roundings, as they are where separate launches store the
 // product before the next one adds to it.
@@ -212,16 +222,43 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_forward_kernel(
   });
 }
 
+// Energies per graph, riding in the backward launch (its tiles do not depend on them): out[g] = sum over the graph's nodes
+// of weight[n] * node_es[n], strided partial sums of the workgroup's 256 threads and a tree over them: a fixed order.
+struct EnergySums {
+  const double *node_es, *node_weights;
+  const int32_t *graph_ptr;
+  double *out;
+  int ngraphs;
+};
+__device__ __forceinline__ void graph_energy(const EnergySums &q, int graph, double *part) {
+  const int tid = threadIdx.x;
+  const int lo = q.graph_ptr[graph], hi = q.graph_ptr[graph + 1];
+  double sum = 0.0;
+  for (int i = lo + tid; i < hi; i += kGlWaves * kWave) sum += q.node_weights ? q.node_weights[i] * q.node_es[i] : q.node_es[i];
+  part[tid] = sum;
+  __syncthreads();
+  for (int d = kGlWaves * kWave / 2; d > 0; d >>= 1) {
+    if (tid < d) part[tid] += part[tid + d];
+    __syncthreads();
+  }
+  if (tid == 0) q.out[graph] = part[0];
+}
+
 // ---- backward: gh1 = gX2 . Wup^T + g1 - skip_scale dE/dh2 . Wskip[element]^T, gB1 = gh1 . Wprod^T ------------------
 template <int NT>
 __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_backward_kernel(
     const float *__restrict__ gX2, const float *__restrict__ d_h2, const float *__restrict__ up_W, const float *__restrict__ skip_W,
     const float *__restrict__ prod_W, const double *__restrict__ w1, double scale, const double *__restrict__ node_weights,
     const int32_t *__restrict__ node_perm, const int32_t *__restrict__ group_offsets, int nnodes, int ngroups, float skip_scale,
-    float *__restrict__ gB1) {
+    float *__restrict__ gB1, EnergySums sums, int tiles) {
   constexpr int C = 32 * NT;
   using S = GlueShared<NT>;
   __shared__ __attribute__((aligned(16))) S s;
+  if (static_cast<int>(blockIdx.x) >= tiles) {
+    // workgroups behind the tiles: the energy of one graph each, from node energies an earlier launch wrote
+    graph_energy(sums, blockIdx.x - tiles, reinterpret_cast<double *>(s.tile));
+    return;
+  }
   int g, pos0, gend;
   if (!locate_tile(group_offsets, ngroups, nnodes, blockIdx.x, g, pos0, gend)) return;
   stage_nodes<NT>(s, node_perm, pos0, gend, nnodes);
@@ -257,6 +294,93 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_backward_kernel(
   });
 }
 
+
+// ---- end of the forward: h2 = B2 . Wprod2 + sc, readouts, gB2 = -(weight) dE/dh2 . Wprod2^T -------------------------
+struct ReadoutArgs {
+  const double *w1, *W2a, *w2b;
+  double act_cst, scale, shift;
+  int hidden;
+  const double *node_weights;  // optional: rows of dE/dh2 are multiplied by the node's weight
+  const int32_t *feats_rows;   // optional row map of the feature concatenation
+  double *node_es;             // [nnodes]
+  float *d_h2;                 // [nnodes, C]
+  double *feats64;             // [nnodes, 2 C] or NULL
+};
+
+template <int NT>
+__global__ __launch_bounds__(kGlWaves *kWave) void node_glue_readout_kernel(const float *__restrict__ B2, const float *__restrict__ sc,
+                                                                           const float *__restrict__ h1,
+                                                                           const float *__restrict__ prod_WT,
+                                                                           const float *__restrict__ prod_W, ReadoutArgs ro,
+                                                                           int nnodes, float *__restrict__ gB2) {
+  constexpr int C = 32 * NT;
+  using S = GlueShared<NT>;
+  constexpr int kLdW = C + 2;  // doubles per row of the transposed hidden-layer weights
+  constexpr int kLd1 = C + 4;  // floats per staged row of h1
+  __shared__ __attribute__((aligned(16))) S s;
+  __shared__ __attribute__((aligned(16))) double sW[readout::kHidden * kLdW];
+  __shared__ double sw1[C];
+  __shared__ double sD[readout::kNodes * readout::kHidden];
+  static_assert(readout::kNodes * kLd1 * sizeof(float) <= sizeof(s.a), "the staged h1 rows live in the idle operand planes");
+  float *s1 = reinterpret_cast<float *>(s.a);
+  const int tid = threadIdx.x;
+  int g, pos0, gend;
+  if (!locate_tile(nullptr, 1, nnodes, blockIdx.x, g, pos0, gend)) return;
+  stage_nodes<NT>(s, nullptr, pos0, gend, nnodes);
+  readout::stage_weights(sW, sw1, ro.W2a, ro.w1, C, ro.hidden, tid, kGlWaves * kWave, kLdW);
+  const int nrows = min(kGlTile, nnodes - pos0);
+
+  v16f acc[NT];
+  product<NT>(s, [&](int row, int col) { return row < nrows ? ld4(B2 + static_cast<int64_t>(pos0 + row) * C + col) : zero4(); },
+              prod_WT, acc);
+  for_each_output<NT>(acc, [&](int row, int col, float v) {
+    const float part = v * 1.0f;
+    s.tile[row * S::kLdT + col] = row < nrows ? part + sc[static_cast<int64_t>(pos0 + row) * C + col] : part;
+  });
+  __syncthreads();  // the tile holds h2; the operand planes are idle until the last product
+
+  for (int sub = 0; sub * readout::kNodes < nrows; ++sub) {
+    const int node0 = pos0 + sub * readout::kNodes;
+    const int rows = min(readout::kNodes, nrows - sub * readout::kNodes);
+    const float *tile0 = s.tile + sub * readout::kNodes * S::kLdT;
+    for (int q = tid; q < rows * C / 4; q += kGlWaves * kWave) {
+      const int r = 4 * q / C, c = 4 * q % C;
+      const f4 a = ld4(h1 + static_cast<int64_t>(node0 + r) * C + c);
+      *reinterpret_cast<f4 *>(s1 + r * kLd1 + c) = a;
+      if (ro.feats64) {
+        const f4 b = *reinterpret_cast<const f4 *>(tile0 + r * S::kLdT + c);
+        const int row = ro.feats_rows ? ro.feats_rows[node0 + r] : node0 + r;
+        if (static_cast<unsigned>(row) < static_cast<unsigned>(nnodes)) {
+          double *f = ro.feats64 + static_cast<int64_t>(row) * (2 * C) + c;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            f[k] = a[k];
+            f[C + k] = b[k];
+          }
+        }
+      }
+    }
+    __syncthreads();
+    const int r = tid / readout::kHidden, j = tid % readout::kHidden;
+    const bool live = r < rows;
+    const double e = readout::node_energy(tid, live, C, ro.hidden, true, s1 + r * kLd1, tile0 + r * S::kLdT, sW, sw1, ro.w2b,
+                                          ro.act_cst, ro.scale, ro.shift, sD, kLdW);
+    if (live && j == 0) ro.node_es[node0 + r] = e;
+    __syncthreads();
+    // dE/dh2 of these rows takes the place of their h2 in the tile: the X operand of the last product
+    readout::energy_gradient(tid, rows, C, sW, sD, ro.scale, [&](int rr, int c, float v) {
+      if (ro.node_weights) v = static_cast<float>(static_cast<double>(v) * ro.node_weights[node0 + rr]);
+      ro.d_h2[static_cast<int64_t>(node0 + rr) * C + c] = v;
+      s.tile[(sub * readout::kNodes + rr) * S::kLdT + c] = v;
+    }, kLdW);
+    __syncthreads();  // s1 and sD are free for the next rows
+  }
+  product<NT>(s, [&](int row, int col) { return *reinterpret_cast<const f4 *>(s.tile + row * S::kLdT + col); }, prod_W, acc);
+  for_each_output<NT>(acc, [&](int row, int col, float v) {
+    if (row < nrows) gB2[static_cast<int64_t>(pos0 + row) * C + col] = v * -1.0f;
+  });
+}
+
 template <int NT>
 void launch_forward(const float *B1, const float *prod_WT, const float *skip_WT, const float *up_WT, const int32_t *perm,
                     const int32_t *offs, int64_t nnodes, int ngroups, float skip_scale, float *h1, float *sc, float *X2,
@@ -269,10 +393,19 @@ void launch_forward(const float *B1, const float *prod_WT, const float *skip_WT,
 template <int NT>
 void launch_backward(const float *gX2, const float *d_h2, const float *up_W, const float *skip_W, const float *prod_W,
                      const double *w1, double scale, const double *node_weights, const int32_t *perm, const int32_t *offs,
-                     int64_t nnodes, int ngroups, float skip_scale, float *gB1, hipStream_t st) {
-  const unsigned tiles = static_cast<unsigned>(ceil_div(nnodes, kGlTile) + ngroups);
-  hipLaunchKernelGGL(node_glue_backward_kernel<NT>, dim3(tiles), dim3(kGlWaves * kWave), 0, st, gX2, d_h2, up_W, skip_W, prod_W,
-                     w1, scale, node_weights, perm, offs, static_cast<int>(nnodes), ngroups, skip_scale, gB1);
+                     int64_t nnodes, int ngroups, float skip_scale, float *gB1, const EnergySums &sums, hipStream_t st) {
+  const int tiles = static_cast<int>(ceil_div(nnodes, kGlTile) + ngroups);
+  const unsigned extra = sums.out ? static_cast<unsigned>(sums.ngraphs) : 0u;
+  hipLaunchKernelGGL(node_glue_backward_kernel<NT>, dim3(static_cast<unsigned>(tiles) + extra), dim3(kGlWaves * kWave), 0, st, gX2, d_h2,
+                     up_W, skip_W, prod_W, w1, scale, node_weights, perm, offs, static_cast<int>(nnodes), ngroups, skip_scale, gB1, sums,
+                     tiles);
+}
+
+template <int NT>
+void launch_readout(const float *B2, const float *sc, const float *h1, const float *prod_WT, const float *prod_W, const ReadoutArgs &ro,
+                    int64_t nnodes, float *gB2, hipStream_t st) {
+  hipLaunchKernelGGL(node_glue_readout_kernel<NT>, dim3(static_cast<unsigned>(ceil_div(nnodes, kGlTile))), dim3(kGlWaves * kWave), 0,
+                     st, B2, sc, h1, prod_WT, prod_W, ro, static_cast<int>(nnodes), gB2);
 }
 
 }  // namespace
@@ -298,6 +431,49 @@ extern "C" int cm_node_glue_forward(const float *B1, const float *prod_WT, const
   return cm::check_launch("cm_node_glue_forward");
 }
 
+namespace cm {
+
+// cm_node_glue_backward whose launch also sums the node energies per graph (operands checked by the caller, cm_mace_step)
+int node_glue_backward_with_energy_sums(const float *gX2, const float *d_h2, const float *up_W, const float *skip_W, const float *prod_W,
+                                        const double *w1, double scale, const double *node_weights, const int32_t *node_perm,
+                                        const int32_t *group_offsets, int64_t nnodes, int ngroups, int channels, float skip_scale,
+                                        float *gB1, const double *node_es, const int32_t *graph_ptr, int ngraphs, double *energies,
+                                        hipStream_t st) {
+  const EnergySums sums{node_es, node_weights, graph_ptr, energies, ngraphs};
+  switch (channels / 32) {
+    case 1: launch_backward<1>(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets, nnodes, ngroups, skip_scale, gB1, sums, st); break;
+    case 2: launch_backward<2>(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets, nnodes, ngroups, skip_scale, gB1, sums, st); break;
+    case 3: launch_backward<3>(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets, nnodes, ngroups, skip_scale, gB1, sums, st); break;
+    case 4: launch_backward<4>(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets, nnodes, ngroups, skip_scale, gB1, sums, st); break;
+    default: set_error("node glue: channels=%d not supported", channels); return CM_EINVAL;
+  }
+  return check_launch("cm_node_glue_backward");
+}
+
+}  // namespace cm
+
+extern "C" int cm_node_glue_readout(const float *B2, const float *sc, const float *h1, const float *prod_WT, const float *prod_W,
+                                    const double *w1, const double *W2a, const double *w2b, double act_cst, double scale,
+                                    double shift, const double *node_weights, int64_t nnodes, int channels, int hidden,
+                                    double *node_energies, float *d_h2, double *node_feats64, const int32_t *feats_rows, float *gB2,
+                                    cm_stream_t stream) {
+  CM_REQUIRE(cm_node_glue_supported(channels), "cm_node_glue_readout: channels=%d must be 32, 64, 96 or 128", channels);
+  CM_REQUIRE(hidden >= 1 && hidden <= cm::readout::kHidden, "cm_node_glue_readout: hidden=%d must be in [1, %d]", hidden,
+             cm::readout::kHidden);
+  CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 256, "cm_node_glue_readout: nnodes out of range");
+  if (nnodes == 0) return CM_OK;
+  CM_REQUIRE(B2 && sc && h1 && prod_WT && prod_W && w1 && W2a && w2b && node_energies && d_h2 && gB2, "cm_node_glue_readout: NULL pointer");
+  const cm::ReadoutArgs ro{w1, W2a, w2b, act_cst, scale, shift, hidden, node_weights, feats_rows, node_energies, d_h2, node_feats64};
+  hipStream_t st = cm::as_stream(stream);
+  switch (channels / 32) {
+    case 1: cm::launch_readout<1>(B2, sc, h1, prod_WT, prod_W, ro, nnodes, gB2, st); break;
+    case 2: cm::launch_readout<2>(B2, sc, h1, prod_WT, prod_W, ro, nnodes, gB2, st); break;
+    case 3: cm::launch_readout<3>(B2, sc, h1, prod_WT, prod_W, ro, nnodes, gB2, st); break;
+    case 4: cm::launch_readout<4>(B2, sc, h1, prod_WT, prod_W, ro, nnodes, gB2, st); break;
+  }
+  return cm::check_launch("cm_node_glue_readout");
+}
+
 extern "C" int cm_node_glue_backward(const float *gX2, const float *d_h2, const float *up_W, const float *skip_W,
                                      const float *prod_W, const double *w1, double scale, const double *node_weights,
                                      const int32_t *node_perm, const int32_t *group_offsets, int64_t nnodes, int ngroups,
@@ -307,12 +483,7 @@ extern "C" int cm_node_glue_backward(const float *gX2, const float *d_h2, const 
   CM_REQUIRE(ngroups >= 2, "cm_node_glue_backward: ngroups counts the elements plus the group of nodes without one");
   if (nnodes == 0) return CM_OK;
   CM_REQUIRE(gX2 && d_h2 && up_W && skip_W && prod_W && w1 && node_perm && group_offsets && gB1, "cm_node_glue_backward: NULL pointer");
-  hipStream_t st = cm::as_stream(stream);
-  switch (channels / 32) {
-    case 1: cm::launch_backward<1>(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets, nnodes, ngroups, skip_scale, gB1, st); break;
-    case 2: cm::launch_backward<2>(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets, nnodes, ngroups, skip_scale, gB1, st); break;
-    case 3: cm::launch_backward<3>(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets, nnodes, ngroups, skip_scale, gB1, st); break;
-    case 4: cm::launch_backward<4>(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets, nnodes, ngroups, skip_scale, gB1, st); break;
-  }
-  return cm::check_launch("cm_node_glue_backward");
+  return cm::node_glue_backward_with_energy_sums(gX2, d_h2, up_W, skip_W, prod_W, w1, scale, node_weights, node_perm, group_offsets,
+                                                 nnodes, ngroups, channels, skip_scale, gB1, nullptr, nullptr, 0, nullptr,
+                                                 cm::as_stream(stream));
 }

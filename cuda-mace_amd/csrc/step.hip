@@ -25,6 +25,7 @@
 
 #include "common.hpp"
 #include "mp_common.hpp"
+#include "node_glue.hpp"
 
 namespace cm {
 namespace {
@@ -381,12 +382,18 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
     if (t == 0 && glue)
       CM_STAGE(4, cm_node_glue_forward(L.B1, w->prod_WT[0], w->skip_WT, w->up_WT, oh_perm, oh_off, N, ne + 1, C, w->skip_scale, L.h1, L.sc,
                                        L.X2, stream));
+    else if (glue)
+      // the product linear, both readouts and the transpose of that linear (the start of the backward chain: seed -1 on
+      // every node energy, times the node's weight) on the same rows in one launch
+      CM_STAGE(10, cm_node_glue_readout(L.B2, L.sc, L.h1, w->prod_WT[1], w->prod_W[1], w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift,
+                                        g->node_weights, N, C, w->hidden, node_energy, L.d_h2, node_feats, g->node_rows, L.gB, stream));
     else
       CM_STAGE(t == 0 ? 4 : 10, cm_linear(B[t], w->prod_WT[t], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, t == 1 ? L.sc : none, h[t], stream));
   }
-  CM_STAGE(11, cm_readout_forward(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden, node_energy,
+  if (!glue)
+    CM_STAGE(11, cm_readout_forward(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden, node_energy,
                              L.d_h2, node_feats, g->node_rows, stream));
-  {
+  if (!glue) {  // with the chained kernels the sums ride in the backward chain's launch
     cm::StageTimer timer_(st, 12, timing_mask);
     hipLaunchKernelGGL(cm::segment_sum_f64_kernel, dim3(g->ngraphs), dim3(cm::kSumThreads), 0, st, node_energy, g->node_weights,
                        g->graph_ptr, interaction_energy);
@@ -397,24 +404,25 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   // own: the gradient with respect to the second layer's features is -d_h2 (the sign goes into the scale of the two
   // linears that consume it, which is exact; node weights scale its rows first), the one with respect to the first
   // layer's is a constant row (times the node's weight).
-  if (!glue || g->node_weights) {
+  if (!glue) {  // the chained kernels form the constant rows and weight the rows of dE/dh2 themselves
     cm::StageTimer timer_(st, 13, timing_mask);
     const dim3 grid(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(N * C, 256), 2048)));
-    if (!glue)  // the glue kernel forms the constant rows itself
-      hipLaunchKernelGGL(cm::seed_linear_readout_kernel, grid, dim3(256), 0, st, L.g1, w->w1, w->scale, g->node_weights,
-                         static_cast<int64_t>(N) * C, C);
+    hipLaunchKernelGGL(cm::seed_linear_readout_kernel, grid, dim3(256), 0, st, L.g1, w->w1, w->scale, g->node_weights,
+                       static_cast<int64_t>(N) * C, C);
     if (g->node_weights)
       hipLaunchKernelGGL(cm::weight_rows_kernel, grid, dim3(256), 0, st, L.d_h2, g->node_weights, static_cast<int64_t>(N) * C, C);
   }
   // layer 1 (second interaction)
-  CM_STAGE(14, cm_linear(L.d_h2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, -1.0f, none, none, L.gB, stream));
+  if (!glue)
+    CM_STAGE(14, cm_linear(L.d_h2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, -1.0f, none, none, L.gB, stream));
   CM_STAGE(15, cm_linear(L.bufM2, w->mix_W[1], nullptr, nullptr, N, 1, 0, 16, C, C, w->mix_scale[1], L.gB, none, L.bufA, stream));
   CM_STAGE(16, cm_mp_edge_backward(L.X2, L.vec, w->r_knots, w->spline[1], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
                               g->first_occ, g->sender_perm, g->sender_offsets, N, E, C, L.gX2, L.gv2, L.edge_scratch, stream));
   // layer 0 (first interaction): its input features depend on the species alone, so no gradient with respect to them
   if (glue) {
-    CM_STAGE(17, cm_node_glue_backward(L.gX2, L.d_h2, w->up_W, w->skip_W, w->prod_W[0], w->w1, w->scale, g->node_weights, oh_perm, oh_off, N,
-                                       ne + 1, C, w->skip_scale, L.gB, stream));
+    CM_STAGE(17, cm::node_glue_backward_with_energy_sums(L.gX2, L.d_h2, w->up_W, w->skip_W, w->prod_W[0], w->w1, w->scale, g->node_weights,
+                                                         oh_perm, oh_off, N, ne + 1, C, w->skip_scale, L.gB, node_energy, g->graph_ptr,
+                                                         g->ngraphs, interaction_energy, st));
   } else {
     CM_STAGE(17, cm_linear(L.gX2, w->up_W, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, L.g1, L.gh1a, stream));
     CM_STAGE(18, cm_linear(L.d_h2, w->skip_W, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, -w->skip_scale, none, L.gh1a, L.gh1, stream));
