@@ -32,7 +32,7 @@ KERNEL_SOURCES = os.path.join(ROOT, "cuda-mace_amd", "csrc")
 STAGE_NAMES = {
     0: "00 edge geometry + live ranges", 1: "01 mp forward L0", 2: "02 channel mixing L0 [N,16,C]", 3: "03 contraction L0",
     4: "04 product linear L0 (+ skip, linear_up when chained)", 5: "05 skip connection", 6: "06 linear_up",
-    7: "07 mp forward L1", 8: "08 channel mixing L1 [N,16,C]", 9: "09 contraction L1", 10: "10 product linear L1 + skip (+ readouts, product linear L1 backward when chained)",
+    7: "07 mp forward L1", 8: "08 channel mixing L1 [N,16,C]", 9: "09 contraction L1", 10: "10 product linear L1 + skip",
     11: "11 readouts", 12: "12 energy sums", 13: "13 backward seeds", 14: "14 product linear L1 backward",
     15: "15 channel mixing L1 backward (+ contraction backward)", 16: "16 mp backward L1 (edge pass + sender pass)",
     17: "17 linear_up backward (+ skip, product linear L0 backward, energy sums when chained)", 18: "18 skip backward",

@@ -114,6 +114,19 @@ __device__ __forceinline__ int stage_edges(const float *__restrict__ Y, const in
   return nlive;
 }
 
+// LDS of one wave's staged chunk: Y [kChunk][16], sender, knot interval, offset in it, position (floats / ints)
+constexpr int kStageBytes = kChunk * 64 + 4 * kChunk * 4;
+
+// Parts a node's edge range is cut into where one wave per node would leave most of the device idle (a 216-atom cell is
+// 216 waves for 1 024 SIMDs, each walking its ~90 edges one after the other): as many as fill about 2 048 wave slots
+// and leave a part a dozen edges on average, at most 8.
+inline int parts_for(int64_t nnodes, int64_t nedges) {
+  if (nnodes <= 0) return 1;
+  const int64_t by_slots = 2048 / nnodes, by_edges = nedges / (12 * nnodes);
+  const int64_t parts = by_slots < by_edges ? by_slots : by_edges;
+  return parts < 1 ? 1 : (parts > 8 ? 8 : static_cast<int>(parts));
+}
+
 template <int L>
 struct MRange {
   static constexpr int lo = L * L;
@@ -123,38 +136,51 @@ struct MRange {
 // -----------------------------------------------------------------------------------------------
 // forward
 // -----------------------------------------------------------------------------------------------
-template <int C, bool FROM_VEC>
-__global__ __launch_bounds__(kWave, (Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVES)) void mp_spline_forward_kernel(const float *__restrict__ X,
+// MULTI: a workgroup of up to eight waves per node, each on a part of the node's edge range (launched for few nodes)
+template <int C, bool FROM_VEC, bool MULTI>
+__global__ __launch_bounds__(MULTI ? 8 * kWave : kWave, (Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVES)) void mp_spline_forward_kernel(const float *__restrict__ X,
                                                                  const float *__restrict__ Y, Spline sp,
                                                                  const int32_t *__restrict__ sender,
                                                                  const int32_t *__restrict__ first_occ, int nnodes,
                                                                  int64_t nedges, float *__restrict__ out) {
   using K = Cfg<C, true>;
   using vec = typename K::vec;
-  __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
-  __shared__ int sS[kChunk];
-  __shared__ int sIdx[kChunk];
-  __shared__ float sXr[kChunk];
-  __shared__ int sOrig[kChunk];
+  // A workgroup is one wave per part of the node's edge range (MULTI; otherwise one wave and one part: see parts_for).
+  // Every wave stages its own edges in its own piece of LDS; the waves meet once, at the end.
+  extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
+  const int wave = MULTI ? threadIdx.x / kWave : 0;
+  const int parts = MULTI ? blockDim.x / kWave : 1;
+  unsigned char *mine = dyn_lds + wave * kStageBytes;
+  float *sY = reinterpret_cast<float *>(mine);
+  int *sS = reinterpret_cast<int *>(mine + kChunk * 64);
+  int *sIdx = sS + kChunk;
+  float *sXr = reinterpret_cast<float *>(sIdx + kChunk);
+  int *sOrig = reinterpret_cast<int *>(sXr + kChunk);
 
   const int node = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x % kWave;
   const int slot = lane / K::SW;
   const int cl = lane % K::SW;
   const bool active = cl < K::LPE;
   int e0 = first_occ[node];
   int e1 = first_occ[nnodes + node];
   clamp_edge_range(e0, e1, nedges);
+  if (parts > 1) {
+    const int64_t len = e1 - e0;
+    const int lo = e0 + static_cast<int>(len * wave / parts);
+    e1 = e0 + static_cast<int>(len * (wave + 1) / parts);
+    e0 = lo;
+  }
 
   vec acc[16];
 #pragma unroll
   for (int m = 0; m < 16; ++m) acc[m] = zerov<vec>();
 
   for (int base = e0; base < e1;) {
-    __syncthreads();
+    wave_lds_fence();  // the staged edges belong to this wave alone
     const int nlive = stage_edges<FROM_VEC>(Y, sender, sp, nnodes, nedges, base, e1, lane, sY, sS, sIdx, sXr, sOrig,
                                             [](int, int, unsigned long long, bool) {});
-    __syncthreads();
+    wave_lds_fence();
     if (active) {
       for (int j = slot; j < nlive; j += K::EPW) {
         const int s = sS[j];
@@ -196,6 +222,24 @@ __global__ __launch_bounds__(kWave, (Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVE
 #pragma unroll
     for (int m = 0; m < 16; ++m) acc[m] += shfl_downv(acc[m], off);
   }
+  if (parts > 1) {
+    // sums of the parts, added up by the first wave in the order of the parts (the same on every run)
+    float *comb = reinterpret_cast<float *>(dyn_lds + parts * kStageBytes);
+    if (wave > 0 && slot == 0 && active) {
+      float *cp = comb + (wave - 1) * (16 * C) + K::off(cl);
+#pragma unroll
+      for (int m = 0; m < 16; ++m) K::st(cp + m * C, acc[m]);
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    if (slot == 0 && active) {
+      for (int w = 1; w < parts; ++w) {
+        const float *cp = comb + (w - 1) * (16 * C) + K::off(cl);
+#pragma unroll
+        for (int m = 0; m < 16; ++m) acc[m] += K::ld(cp + m * C);
+      }
+    }
+  }
   if (slot == 0 && active) {
     float *op = out + static_cast<int64_t>(node) * (16 * C) + K::off(cl);
 #pragma unroll
@@ -210,7 +254,7 @@ template <int C, bool FROM_VEC, bool WANT_GY, bool WANT_GR, bool WANT_GX>
 __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_edge_kernel(
     const float *__restrict__ X, const float *__restrict__ Y, Spline sp, const float *__restrict__ G,
     const int32_t *__restrict__ sender, const int32_t *__restrict__ first_occ, int nnodes, int64_t nedges,
-    float *__restrict__ gY, float *__restrict__ g_r, float *__restrict__ gXe) {
+    float *__restrict__ gY, float *__restrict__ g_r, float *__restrict__ gXe, int parts) {
   using K = Cfg<C>;
   using vec = typename K::vec;
   __shared__ __attribute__((aligned(16))) float sY[kChunk * 16];
@@ -221,7 +265,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   __shared__ float sGY[16 * kChunk];  // [m][edge]
   __shared__ float sGr[kChunk];
 
-  const int node = blockIdx.x;
+  // one wave per node, or (few nodes: parts_for) per part of a node's edge range: every output of this pass belongs to
+  // one edge, so the parts share nothing but the node's gradient rows, which each of them reads
+  const int node = parts == 1 ? blockIdx.x : blockIdx.x / parts;
   const int lane = threadIdx.x;
   const int slot = lane / K::SW;
   const int cl = lane % K::SW;
@@ -230,6 +276,13 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   int e0 = first_occ[node];
   int e1 = first_occ[nnodes + node];
   clamp_edge_range(e0, e1, nedges);
+  if (parts > 1) {
+    const int part = blockIdx.x % parts;
+    const int64_t len = e1 - e0;
+    const int lo = e0 + static_cast<int>(len * part / parts);
+    e1 = e0 + static_cast<int>(len * (part + 1) / parts);
+    e0 = lo;
+  }
   if (e0 >= e1) return;
 
   vec g[16];
@@ -396,8 +449,14 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
 template <int C, bool FROM_VEC>
 int launch_forward(const float *X, const float *Y, const Spline &sp, const int32_t *sender, const int32_t *first_occ,
                    int64_t nnodes, int64_t nedges, float *out, hipStream_t st) {
-  hipLaunchKernelGGL((mp_spline_forward_kernel<C, FROM_VEC>), dim3(static_cast<unsigned>(nnodes)), dim3(kWave), 0, st, X, Y, sp,
-                     sender, first_occ, static_cast<int>(nnodes), nedges, out);
+  const int parts = parts_for(nnodes, nedges);
+  const size_t lds = static_cast<size_t>(parts) * kStageBytes + static_cast<size_t>(parts - 1) * 16 * C * sizeof(float);
+  if (parts > 1)
+    hipLaunchKernelGGL((mp_spline_forward_kernel<C, FROM_VEC, true>), dim3(static_cast<unsigned>(nnodes)), dim3(kWave * parts), lds, st,
+                       X, Y, sp, sender, first_occ, static_cast<int>(nnodes), nedges, out);
+  else
+    hipLaunchKernelGGL((mp_spline_forward_kernel<C, FROM_VEC, false>), dim3(static_cast<unsigned>(nnodes)), dim3(kWave), lds, st, X, Y,
+                       sp, sender, first_occ, static_cast<int>(nnodes), nedges, out);
   return check_launch(FROM_VEC ? "cm_mp_edge_forward" : "cm_mp_spline_forward");
 }
 
@@ -405,8 +464,9 @@ template <int C, bool FROM_VEC, bool GY, bool GR, bool GX>
 void launch_edge(const float *X, const float *Y, const Spline &sp, const float *G, const int32_t *sender,
                  const int32_t *first_occ, int64_t nnodes, int64_t nedges, float *gY, float *g_r, float *gXe,
                  hipStream_t st) {
-  hipLaunchKernelGGL((mp_spline_backward_edge_kernel<C, FROM_VEC, GY, GR, GX>), dim3(static_cast<unsigned>(nnodes)),
-                     dim3(kWave), 0, st, X, Y, sp, G, sender, first_occ, static_cast<int>(nnodes), nedges, gY, g_r, gXe);
+  const int parts = parts_for(nnodes, nedges);
+  hipLaunchKernelGGL((mp_spline_backward_edge_kernel<C, FROM_VEC, GY, GR, GX>), dim3(static_cast<unsigned>(nnodes * parts)),
+                     dim3(kWave), 0, st, X, Y, sp, G, sender, first_occ, static_cast<int>(nnodes), nedges, gY, g_r, gXe, parts);
 }
 
 // gY / g_r: outputs of the Y-and-r variant; in the FROM_VEC variant gY is the [E, 3] vector gradient and g_r, when given,

@@ -14,21 +14,12 @@
 // v_mfma_f32_32x32x16_bf16, K in chunks of 32), and every intermediate is rounded to fp32 where the separate launches
 // store it, so the chain returns the bits of the separate launches.
 //
-// A third kernel does the same at the end of the forward, where the second layer's product linear, both readouts and
-// the transpose of that linear follow each other on the same rows (reference: models/InvariantMACE.py:330-343 and its
-// backward):
-//
-//   h2 = B2 . Wprod2 + sc      E_n, dE/dh2, feats = readouts(h1, h2)      gB2 = -dE/dh2 . Wprod2^T
-//
-// h2 only ever exists as the LDS tile (the model returns it inside the fp64 feature concatenation).
-//
 // g1 and g2 are the gradients of minus the (weighted) sum of node energies with respect to the two layers' features:
 // g1[n, c] = -weight[n] scale w1[c] is formed here from the linear readout's weights; g2 = -dE/dh2 arrives as dE/dh2 and
 // its sign goes into the scale of the skip product.
 #include "common.hpp"
 #include "mfma_split.hpp"
 #include "node_glue.hpp"
-#include "readout_device.hpp"  // before the pragma below: the readouts' fp64 arithmetic compiles as in readout.hip
 
 // Products and the additions that follow them stay separate roundings, as they are where separate launches store the
 // product before the next one adds to it.
@@ -73,53 +64,86 @@ __device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ group_of
   return pos0 < nnodes;
 }
 
-// acc = X . W over K = C, X rows given by `xrow(row, col)` (four consecutive columns of a tile row), W as its transpose
-// Wg [C, C] (row = output column).  All threads of the workgroup take part; ends with every wave past its last LDS read
-// of the planes only after the caller's next barrier.
-template <int NT, class XRow>
-__device__ __forceinline__ void product(GlueShared<NT> &s, XRow xrow, const float *__restrict__ Wg, v16f (&acc)[NT]) {
+// Operands of a product on their way from memory: a thread's 16-byte pieces of every K chunk, requested all at once
+// and long before the product that consumes them (a chain of three products otherwise pays a memory latency per chunk).
+// Staging map: eight threads cover the 32 columns of a chunk of one row, 32 rows per pass.
+constexpr int kGlTPR = kGlKC / 4;                  // threads per staged row
+constexpr int kGlRPP = kGlWaves * kWave / kGlTPR;  // rows per pass
+constexpr int kGlAPasses = kGlTile / kGlRPP;
+template <int NT>
+struct WeightPieces {
+  f4 v[NT][NT];  // [chunk][pass]: row 32 pass + tid / 8 of the transposed block, columns 32 chunk + 4 (tid % 8) ..
+};
+template <int NT>
+struct RowPieces {
+  f4 v[NT][kGlAPasses];
+};
+
+template <int NT>
+__device__ __forceinline__ void fetch_weights(const float *__restrict__ Wg, WeightPieces<NT> &w) {
   constexpr int C = 32 * NT;
+  const int srow = threadIdx.x / kGlTPR, scol = (threadIdx.x % kGlTPR) * 4;
+#pragma unroll
+  for (int k = 0; k < NT; ++k)
+#pragma unroll
+    for (int i = 0; i < NT; ++i) w.v[k][i] = ld4(Wg + static_cast<int64_t>(kGlRPP * i + srow) * C + kGlKC * k + scol);
+}
+
+// rows of X [*, C] named by the tile's node list (zeros for rows beyond the tile)
+template <int NT>
+__device__ __forceinline__ void fetch_rows(const GlueShared<NT> &s, const float *__restrict__ X, RowPieces<NT> &a) {
+  constexpr int C = 32 * NT;
+  const int srow = threadIdx.x / kGlTPR, scol = (threadIdx.x % kGlTPR) * 4;
+#pragma unroll
+  for (int i = 0; i < kGlAPasses; ++i) {
+    const int node = s.node[kGlRPP * i + srow];
+#pragma unroll
+    for (int k = 0; k < NT; ++k) a.v[k][i] = node >= 0 ? ld4(X + static_cast<int64_t>(node) * C + kGlKC * k + scol) : zero4();
+  }
+}
+
+// acc = X . W over K = C.  X: the pieces fetched by fetch_rows, or (FROM_TILE) the fp32 tile in LDS; W: the pieces fetched
+// by fetch_weights from the transposed block [C out, C in].  All threads of the workgroup take part; on return the
+// operand planes may still be read by slower waves: whatever overwrites them next sits behind a barrier.
+template <int NT, bool FROM_TILE>
+__device__ __forceinline__ void product(GlueShared<NT> &s, const RowPieces<NT> *rows, const WeightPieces<NT> &w, v16f (&acc)[NT]) {
+  constexpr int C = 32 * NT;
+  using S = GlueShared<NT>;
   const int tid = threadIdx.x;
   const int lane = tid % kWave, wave = tid / kWave;
-  constexpr int kTPR = kGlKC / 4;                 // threads per staged row
-  constexpr int kRPP = kGlWaves * kWave / kTPR;   // rows per pass
-  constexpr int A_PASSES = kGlTile / kRPP, B_PASSES = C / kRPP;
-  const int srow = tid / kTPR, scol = (tid % kTPR) * 4;
+  const int srow = tid / kGlTPR, scol = (tid % kGlTPR) * 4;
   const int mrow = lane % 32, half = lane / 32;
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
-  f4 pa[A_PASSES], pb[B_PASSES];
-  auto prefetch = [&](int kc) {
 #pragma unroll
-    for (int i = 0; i < A_PASSES; ++i) pa[i] = xrow(kRPP * i + srow, kc + scol);
+  for (int k = 0; k < NT; ++k) {
+    __syncthreads();  // previous chunk fully consumed (and, before the first, the tile complete)
 #pragma unroll
-    for (int i = 0; i < B_PASSES; ++i) pb[i] = ld4(Wg + static_cast<int64_t>(kRPP * i + srow) * C + kc + scol);
-  };
-  prefetch(0);
-  for (int kc = 0; kc < C; kc += kGlKC) {
-    __syncthreads();  // previous chunk fully consumed
-#pragma unroll
-    for (int i = 0; i < A_PASSES; ++i) {
+    for (int i = 0; i < kGlAPasses; ++i) {
+      f4 x;
+      if constexpr (FROM_TILE)
+        x = *reinterpret_cast<const f4 *>(s.tile + (kGlRPP * i + srow) * S::kLdT + kGlKC * k + scol);
+      else
+        x = rows->v[k][i];
       bf16x4 h, md, lw;
-      split3(pa[i], h, md, lw);
-      const int at = (kRPP * i + srow) * kGlLdH + scol;
+      split3(x, h, md, lw);
+      const int at = (kGlRPP * i + srow) * kGlLdH + scol;
       *reinterpret_cast<bf16x4 *>(s.a + at) = h;
       *reinterpret_cast<bf16x4 *>(s.a + kGlTile * kGlLdH + at) = md;
       *reinterpret_cast<bf16x4 *>(s.a + 2 * kGlTile * kGlLdH + at) = lw;
     }
 #pragma unroll
-    for (int i = 0; i < B_PASSES; ++i) {
+    for (int i = 0; i < NT; ++i) {
       bf16x4 h, md, lw;
-      split3(pb[i], h, md, lw);
-      const int at = (kRPP * i + srow) * kGlLdH + scol;
+      split3(w.v[k][i], h, md, lw);
+      const int at = (kGlRPP * i + srow) * kGlLdH + scol;
       *reinterpret_cast<bf16x4 *>(s.b + at) = h;
       *reinterpret_cast<bf16x4 *>(s.b + C * kGlLdH + at) = md;
       *reinterpret_cast<bf16x4 *>(s.b + 2 * C * kGlLdH + at) = lw;
     }
     __syncthreads();
-    if (kc + kGlKC < C) prefetch(kc + kGlKC);
 #pragma unroll
     for (int ks = 0; ks < kGlKC; ks += 16) {
       const int aoff = (32 * wave + mrow) * kGlLdH + ks + 8 * half;
@@ -188,34 +212,36 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_forward_kernel(
   if (!locate_tile(group_offsets, ngroups, nnodes, blockIdx.x, g, pos0, gend)) return;
   stage_nodes<NT>(s, node_perm, pos0, gend, nnodes);
 
+  const bool no_element = g == ngroups - 1;  // nodes of no element: the skip connection is defined as zero there
+  WeightPieces<NT> wa, wb;
+  RowPieces<NT> a0;
+  fetch_weights<NT>(prod_WT, wa);
+  fetch_rows<NT>(s, B1, a0);
+  if (!no_element) fetch_weights<NT>(skip_WT + static_cast<int64_t>(g) * C * C, wb);  // in flight during the first product
+
   v16f acc[NT];
-  product<NT>(s, [&](int row, int col) {
-    const int node = s.node[row];
-    return node >= 0 ? ld4(B1 + static_cast<int64_t>(node) * C + col) : zero4();
-  }, prod_WT, acc);
+  product<NT, false>(s, &a0, wa, acc);
+  fetch_weights<NT>(up_WT, wa);
   for_each_output<NT>(acc, [&](int row, int col, float v) {
     const float out = v * 1.0f;
     s.tile[row * S::kLdT + col] = out;
     const int node = s.node[row];
     if (node >= 0) h1[static_cast<int64_t>(node) * C + col] = out;
   });
-  __syncthreads();  // the tile is complete before any wave stages from it
-  auto tile_row = [&](int row, int col) { return *reinterpret_cast<const f4 *>(s.tile + row * S::kLdT + col); };
-
-  if (g == ngroups - 1) {
-    // nodes of no element: the skip connection is defined as zero there
+  // (the tile is complete behind the barrier at the top of the next product)
+  if (no_element) {
     for_each_output<NT>(acc, [&](int row, int col, float) {
       const int node = s.node[row];
       if (node >= 0) sc[static_cast<int64_t>(node) * C + col] = 0.f;
     });
   } else {
-    product<NT>(s, tile_row, skip_WT + static_cast<int64_t>(g) * C * C, acc);
+    product<NT, true>(s, nullptr, wb, acc);
     for_each_output<NT>(acc, [&](int row, int col, float v) {
       const int node = s.node[row];
       if (node >= 0) sc[static_cast<int64_t>(node) * C + col] = v * skip_scale;
     });
   }
-  product<NT>(s, tile_row, up_WT, acc);
+  product<NT, true>(s, nullptr, wa, acc);
   for_each_output<NT>(acc, [&](int row, int col, float v) {
     const int node = s.node[row];
     if (node >= 0) X2[static_cast<int64_t>(node) * C + col] = v * 1.0f;
@@ -250,27 +276,32 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_backward_kernel(
     const float *__restrict__ gX2, const float *__restrict__ d_h2, const float *__restrict__ up_W, const float *__restrict__ skip_W,
     const float *__restrict__ prod_W, const double *__restrict__ w1, double scale, const double *__restrict__ node_weights,
     const int32_t *__restrict__ node_perm, const int32_t *__restrict__ group_offsets, int nnodes, int ngroups, float skip_scale,
-    float *__restrict__ gB1, EnergySums sums, int tiles) {
+    float *__restrict__ gB1, EnergySums sums, int first_tile) {
   constexpr int C = 32 * NT;
   using S = GlueShared<NT>;
   __shared__ __attribute__((aligned(16))) S s;
-  if (static_cast<int>(blockIdx.x) >= tiles) {
-    // workgroups behind the tiles: the energy of one graph each, from node energies an earlier launch wrote
-    graph_energy(sums, blockIdx.x - tiles, reinterpret_cast<double *>(s.tile));
+  if (static_cast<int>(blockIdx.x) < first_tile) {
+    // workgroups ahead of the tiles: the energy of one graph each, from node energies an earlier launch wrote
+    graph_energy(sums, blockIdx.x, reinterpret_cast<double *>(s.tile));
     return;
   }
   int g, pos0, gend;
-  if (!locate_tile(group_offsets, ngroups, nnodes, blockIdx.x, g, pos0, gend)) return;
+  if (!locate_tile(group_offsets, ngroups, nnodes, blockIdx.x - first_tile, g, pos0, gend)) return;
   stage_nodes<NT>(s, node_perm, pos0, gend, nnodes);
 
+  const bool no_element = g == ngroups - 1;
+  WeightPieces<NT> wa, wb;
+  RowPieces<NT> a0, a1;
+  fetch_weights<NT>(up_W, wa);
+  fetch_rows<NT>(s, gX2, a0);
+  if (!no_element) {  // in flight during the first product
+    fetch_weights<NT>(skip_W + static_cast<int64_t>(g) * C * C, wb);
+    fetch_rows<NT>(s, d_h2, a1);
+  }
+
   v16f acc[NT];
-  auto rows_of = [&](const float *X) {
-    return [X](int row, int col) {
-      const int node = s.node[row];
-      return node >= 0 ? ld4(X + static_cast<int64_t>(node) * C + col) : zero4();
-    };
-  };
-  product<NT>(s, rows_of(gX2), up_W, acc);
+  product<NT, false>(s, &a0, wa, acc);
+  fetch_weights<NT>(prod_W, wa);
   for_each_output<NT>(acc, [&](int row, int col, float v) {
     const int node = s.node[row];
     const double nw = (node_weights && node >= 0) ? node_weights[node] : 1.0;
@@ -278,106 +309,18 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_backward_kernel(
     const float part = v * 1.0f;
     s.tile[row * S::kLdT + col] = part + g1;
   });
-  if (g != ngroups - 1) {
-    product<NT>(s, rows_of(d_h2), skip_W + static_cast<int64_t>(g) * C * C, acc);
+  if (!no_element) {
+    product<NT, false>(s, &a1, wb, acc);
     // each element of the tile is read and written by the lane that wrote it above
     for_each_output<NT>(acc, [&](int row, int col, float v) {
       const float part = v * -skip_scale;
       s.tile[row * S::kLdT + col] += part;
     });
   }
-  __syncthreads();  // the tile is complete before any wave stages from it
-  product<NT>(s, [&](int row, int col) { return *reinterpret_cast<const f4 *>(s.tile + row * S::kLdT + col); }, prod_W, acc);
+  product<NT, true>(s, nullptr, wa, acc);
   for_each_output<NT>(acc, [&](int row, int col, float v) {
     const int node = s.node[row];
     if (node >= 0) gB1[static_cast<int64_t>(node) * C + col] = v * 1.0f;
-  });
-}
-
-
-// ---- end of the forward: h2 = B2 . Wprod2 + sc, readouts, gB2 = -(weight) dE/dh2 . Wprod2^T -------------------------
-struct ReadoutArgs {
-  const double *w1, *W2a, *w2b;
-  double act_cst, scale, shift;
-  int hidden;
-  const double *node_weights;  // optional: rows of dE/dh2 are multiplied by the node's weight
-  const int32_t *feats_rows;   // optional row map of the feature concatenation
-  double *node_es;             // [nnodes]
-  float *d_h2;                 // [nnodes, C]
-  double *feats64;             // [nnodes, 2 C] or NULL
-};
-
-template <int NT>
-__global__ __launch_bounds__(kGlWaves *kWave) void node_glue_readout_kernel(const float *__restrict__ B2, const float *__restrict__ sc,
-                                                                           const float *__restrict__ h1,
-                                                                           const float *__restrict__ prod_WT,
-                                                                           const float *__restrict__ prod_W, ReadoutArgs ro,
-                                                                           int nnodes, float *__restrict__ gB2) {
-  constexpr int C = 32 * NT;
-  using S = GlueShared<NT>;
-  constexpr int kLdW = C + 2;  // doubles per row of the transposed hidden-layer weights
-  constexpr int kLd1 = C + 4;  // floats per staged row of h1
-  __shared__ __attribute__((aligned(16))) S s;
-  __shared__ __attribute__((aligned(16))) double sW[readout::kHidden * kLdW];
-  __shared__ double sw1[C];
-  __shared__ double sD[readout::kNodes * readout::kHidden];
-  static_assert(readout::kNodes * kLd1 * sizeof(float) <= sizeof(s.a), "the staged h1 rows live in the idle operand planes");
-  float *s1 = reinterpret_cast<float *>(s.a);
-  const int tid = threadIdx.x;
-  int g, pos0, gend;
-  if (!locate_tile(nullptr, 1, nnodes, blockIdx.x, g, pos0, gend)) return;
-  stage_nodes<NT>(s, nullptr, pos0, gend, nnodes);
-  readout::stage_weights(sW, sw1, ro.W2a, ro.w1, C, ro.hidden, tid, kGlWaves * kWave, kLdW);
-  const int nrows = min(kGlTile, nnodes - pos0);
-
-  v16f acc[NT];
-  product<NT>(s, [&](int row, int col) { return row < nrows ? ld4(B2 + static_cast<int64_t>(pos0 + row) * C + col) : zero4(); },
-              prod_WT, acc);
-  for_each_output<NT>(acc, [&](int row, int col, float v) {
-    const float part = v * 1.0f;
-    s.tile[row * S::kLdT + col] = row < nrows ? part + sc[static_cast<int64_t>(pos0 + row) * C + col] : part;
-  });
-  __syncthreads();  // the tile holds h2; the operand planes are idle until the last product
-
-  for (int sub = 0; sub * readout::kNodes < nrows; ++sub) {
-    const int node0 = pos0 + sub * readout::kNodes;
-    const int rows = min(readout::kNodes, nrows - sub * readout::kNodes);
-    const float *tile0 = s.tile + sub * readout::kNodes * S::kLdT;
-    for (int q = tid; q < rows * C / 4; q += kGlWaves * kWave) {
-      const int r = 4 * q / C, c = 4 * q % C;
-      const f4 a = ld4(h1 + static_cast<int64_t>(node0 + r) * C + c);
-      *reinterpret_cast<f4 *>(s1 + r * kLd1 + c) = a;
-      if (ro.feats64) {
-        const f4 b = *reinterpret_cast<const f4 *>(tile0 + r * S::kLdT + c);
-        const int row = ro.feats_rows ? ro.feats_rows[node0 + r] : node0 + r;
-        if (static_cast<unsigned>(row) < static_cast<unsigned>(nnodes)) {
-          double *f = ro.feats64 + static_cast<int64_t>(row) * (2 * C) + c;
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            f[k] = a[k];
-            f[C + k] = b[k];
-          }
-        }
-      }
-    }
-    __syncthreads();
-    const int r = tid / readout::kHidden, j = tid % readout::kHidden;
-    const bool live = r < rows;
-    const double e = readout::node_energy(tid, live, C, ro.hidden, true, s1 + r * kLd1, tile0 + r * S::kLdT, sW, sw1, ro.w2b,
-                                          ro.act_cst, ro.scale, ro.shift, sD, kLdW);
-    if (live && j == 0) ro.node_es[node0 + r] = e;
-    __syncthreads();
-    // dE/dh2 of these rows takes the place of their h2 in the tile: the X operand of the last product
-    readout::energy_gradient(tid, rows, C, sW, sD, ro.scale, [&](int rr, int c, float v) {
-      if (ro.node_weights) v = static_cast<float>(static_cast<double>(v) * ro.node_weights[node0 + rr]);
-      ro.d_h2[static_cast<int64_t>(node0 + rr) * C + c] = v;
-      s.tile[(sub * readout::kNodes + rr) * S::kLdT + c] = v;
-    }, kLdW);
-    __syncthreads();  // s1 and sD are free for the next rows
-  }
-  product<NT>(s, [&](int row, int col) { return *reinterpret_cast<const f4 *>(s.tile + row * S::kLdT + col); }, prod_W, acc);
-  for_each_output<NT>(acc, [&](int row, int col, float v) {
-    if (row < nrows) gB2[static_cast<int64_t>(pos0 + row) * C + col] = v * -1.0f;
   });
 }
 
@@ -398,14 +341,7 @@ void launch_backward(const float *gX2, const float *d_h2, const float *up_W, con
   const unsigned extra = sums.out ? static_cast<unsigned>(sums.ngraphs) : 0u;
   hipLaunchKernelGGL(node_glue_backward_kernel<NT>, dim3(static_cast<unsigned>(tiles) + extra), dim3(kGlWaves * kWave), 0, st, gX2, d_h2,
                      up_W, skip_W, prod_W, w1, scale, node_weights, perm, offs, static_cast<int>(nnodes), ngroups, skip_scale, gB1, sums,
-                     tiles);
-}
-
-template <int NT>
-void launch_readout(const float *B2, const float *sc, const float *h1, const float *prod_WT, const float *prod_W, const ReadoutArgs &ro,
-                    int64_t nnodes, float *gB2, hipStream_t st) {
-  hipLaunchKernelGGL(node_glue_readout_kernel<NT>, dim3(static_cast<unsigned>(ceil_div(nnodes, kGlTile))), dim3(kGlWaves * kWave), 0,
-                     st, B2, sc, h1, prod_WT, prod_W, ro, static_cast<int>(nnodes), gB2);
+                     static_cast<int>(extra));
 }
 
 }  // namespace
@@ -451,28 +387,6 @@ int node_glue_backward_with_energy_sums(const float *gX2, const float *d_h2, con
 }
 
 }  // namespace cm
-
-extern "C" int cm_node_glue_readout(const float *B2, const float *sc, const float *h1, const float *prod_WT, const float *prod_W,
-                                    const double *w1, const double *W2a, const double *w2b, double act_cst, double scale,
-                                    double shift, const double *node_weights, int64_t nnodes, int channels, int hidden,
-                                    double *node_energies, float *d_h2, double *node_feats64, const int32_t *feats_rows, float *gB2,
-                                    cm_stream_t stream) {
-  CM_REQUIRE(cm_node_glue_supported(channels), "cm_node_glue_readout: channels=%d must be 32, 64, 96 or 128", channels);
-  CM_REQUIRE(hidden >= 1 && hidden <= cm::readout::kHidden, "cm_node_glue_readout: hidden=%d must be in [1, %d]", hidden,
-             cm::readout::kHidden);
-  CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 256, "cm_node_glue_readout: nnodes out of range");
-  if (nnodes == 0) return CM_OK;
-  CM_REQUIRE(B2 && sc && h1 && prod_WT && prod_W && w1 && W2a && w2b && node_energies && d_h2 && gB2, "cm_node_glue_readout: NULL pointer");
-  const cm::ReadoutArgs ro{w1, W2a, w2b, act_cst, scale, shift, hidden, node_weights, feats_rows, node_energies, d_h2, node_feats64};
-  hipStream_t st = cm::as_stream(stream);
-  switch (channels / 32) {
-    case 1: cm::launch_readout<1>(B2, sc, h1, prod_WT, prod_W, ro, nnodes, gB2, st); break;
-    case 2: cm::launch_readout<2>(B2, sc, h1, prod_WT, prod_W, ro, nnodes, gB2, st); break;
-    case 3: cm::launch_readout<3>(B2, sc, h1, prod_WT, prod_W, ro, nnodes, gB2, st); break;
-    case 4: cm::launch_readout<4>(B2, sc, h1, prod_WT, prod_W, ro, nnodes, gB2, st); break;
-  }
-  return cm::check_launch("cm_node_glue_readout");
-}
 
 extern "C" int cm_node_glue_backward(const float *gX2, const float *d_h2, const float *up_W, const float *skip_W,
                                      const float *prod_W, const double *w1, double scale, const double *node_weights,

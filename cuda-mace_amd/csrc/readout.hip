@@ -19,17 +19,18 @@
 #include <cmath>
 
 #include "common.hpp"
-#include "readout_device.hpp"
 
 namespace cm {
 namespace {
 
-using readout::kHidden;
-using readout::kLdW;
-using readout::kMaxC;
-using readout::kNodes;
+constexpr int kNodes = 16;    // nodes per workgroup
+constexpr int kHidden = 16;   // threads per node = largest hidden width handled
+constexpr int kMaxC = 256;
+constexpr int kLdW = kMaxC + 2;   // row stride (doubles) of W2a transposed, [hidden][channel]: rows j and j + 1 start 4 banks apart,
+                                  // so the 16 hidden units of a node read their 16-byte pieces without conflicts
 constexpr int kMaxGroups = 512;   // workgroups of a forward launch
 constexpr int kLdS = kMaxC + 4;   // row stride (floats) of a feature tile: 16-byte aligned rows, the four nodes of a wave 4 banks apart
+typedef double d2v __attribute__((ext_vector_type(2)));
 
 __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     const float *__restrict__ h1, const float *__restrict__ h2, const double *__restrict__ w1, const double *__restrict__ W2a,
@@ -42,7 +43,11 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
   __shared__ __attribute__((aligned(16))) float s2[kNodes * kLdS];
   __shared__ double sD[kNodes * kHidden];  // w2b[j] * act'(z_j) per node
   const int t = threadIdx.x;
-  readout::stage_weights(sW, sw1, W2a, w1, C, H, t, blockDim.x);
+  for (int i = t; i < C * kHidden; i += blockDim.x) {
+    const int c = i / kHidden, j = i % kHidden;
+    sW[j * kLdW + c] = j < H ? W2a[c * H + j] : 0.0;
+  }
+  for (int c = t; c < C; c += blockDim.x) sw1[c] = w1[c];
   // a workgroup stages the weights once and then walks tiles of 16 nodes; the rows of its next tile are requested
   // before the current one is worked on (one element per trip, each waited for, would cost a memory latency per trip)
   const int ntiles = (nnodes + kNodes - 1) / kNodes;
@@ -108,11 +113,67 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     __syncthreads();
     const int r = t / kHidden, j = t % kHidden;
     const bool live = r < rows;
-    const double e = readout::node_energy(t, live, C, H, wide, s1 + r * kLdS, s2 + r * kLdS, sW, sw1, w2b, act_cst, scale, shift, sD);
-    if (live && j == 0) node_es[node0 + r] = e;
+    // first readout: each of the node's 16 threads takes every 16th channel
+    double e1 = 0.0, z = 0.0;
+    if (live) {
+      const float *row1 = s1 + r * kLdS;
+      for (int c = j; c < C; c += kHidden) e1 += static_cast<double>(row1[c]) * sw1[c];
+      // four independent partial sums (channels c = 0, 1, 2, 3 modulo 4): the fp64 multiply-add chain is otherwise as long
+      // as the channel count.  Four channels per trip: one 16-byte read of the node's row, two of the weight row.
+      double z0 = 0.0, z1 = 0.0, z2 = 0.0, z3 = 0.0;
+      const float *srow = s2 + r * kLdS;
+      const double *wrow = sW + j * kLdW;
+      int c = 0;
+      if (wide) {
+#pragma unroll 2
+        for (; c + 3 < C; c += 4) {
+          const f4 x = *reinterpret_cast<const f4 *>(srow + c);
+          const d2v w01 = *reinterpret_cast<const d2v *>(wrow + c), w23 = *reinterpret_cast<const d2v *>(wrow + c + 2);
+          z0 += static_cast<double>(x.x) * w01.x;
+          z1 += static_cast<double>(x.y) * w01.y;
+          z2 += static_cast<double>(x.z) * w23.x;
+          z3 += static_cast<double>(x.w) * w23.y;
+        }
+      } else {
+        for (; c + 3 < C; c += 4) {
+          z0 += static_cast<double>(srow[c]) * wrow[c];
+          z1 += static_cast<double>(srow[c + 1]) * wrow[c + 1];
+          z2 += static_cast<double>(srow[c + 2]) * wrow[c + 2];
+          z3 += static_cast<double>(srow[c + 3]) * wrow[c + 3];
+        }
+      }
+      for (; c < C; ++c) z0 += static_cast<double>(srow[c]) * wrow[c];
+      z = (z0 + z1) + (z2 + z3);
+    }
+    double e2 = 0.0, dj = 0.0;
+    if (live && j < H) {
+      const double sig = 1.0 / (1.0 + exp(-z));
+      e2 = w2b[j] * act_cst * z * sig;
+      dj = w2b[j] * act_cst * (sig + z * sig * (1.0 - sig));
+    }
+    sD[t] = dj;
+    double e = e1 + e2;
+#pragma unroll
+    for (int off = kHidden / 2; off > 0; off >>= 1) e += __shfl_xor(e, off);
+    if (live && j == 0) node_es[node0 + r] = scale * e + shift;
     __syncthreads();
-    readout::energy_gradient(t, rows, C, sW, sD, scale,
-                             [&](int rr, int c, float v) { d2[static_cast<int64_t>(node0 + rr) * C + c] = v; });
+    // d e / d h2: a thread keeps the 16 weights of its channel in registers and serves a share of the tile's rows
+    // (256 / C row groups; the rows' 16 factors are read by all lanes of a group at once)
+    const int groups = kNodes * kHidden / C;  // at least 1: C <= 256 = threads of the workgroup
+    const int per = (kNodes + groups - 1) / groups;
+    const int c = t % C, grp = t / C;
+    if (grp < groups) {
+      double wq[kHidden];
+#pragma unroll
+      for (int q = 0; q < kHidden; ++q) wq[q] = sW[q * kLdW + c];
+      const int r1 = min(rows, (grp + 1) * per);
+      for (int rr = grp * per; rr < r1; ++rr) {
+        double acc = 0.0;
+#pragma unroll
+        for (int q = 0; q < kHidden; ++q) acc += wq[q] * sD[rr * kHidden + q];
+        d2[static_cast<int64_t>(node0 + rr) * C + c] = static_cast<float>(scale * acc);
+      }
+    }
   }
 }
 

@@ -20,6 +20,7 @@
 //   E_n, dE/dh2, feats = readouts(h1, h2);  E_graph = sum over the graph's nodes
 // With node weights (cm_mace_graph.node_weights) E_graph = sum_n weight[n] E_n and the seed of node n is -weight[n]: g1's
 // rows and the rows of dE/dh2 are multiplied by the node's weight before the chain starts.
+#include <cstdlib>
 #include <mutex>
 #include <vector>
 
@@ -363,7 +364,8 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   float *B[2] = {L.B1, L.B2};
   float *h[2] = {L.h1, L.h2};
   // the three [N, C] products between the layers (and their three transposes in the backward) as one launch each
-  const bool glue = cm_node_glue_supported(C) != 0;
+  const char *glue_env = getenv("CM_STEP_GLUE");  // development switch: 0 keeps the separate launches
+  const bool glue = cm_node_glue_supported(C) != 0 && !(glue_env && atoi(glue_env) == 0);
   for (int t = 0; t < 2; ++t) {
     if (t == 1 && !glue) {
       // residual skip connection per element and linear_up, both of the first layer's output
@@ -382,16 +384,10 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
     if (t == 0 && glue)
       CM_STAGE(4, cm_node_glue_forward(L.B1, w->prod_WT[0], w->skip_WT, w->up_WT, oh_perm, oh_off, N, ne + 1, C, w->skip_scale, L.h1, L.sc,
                                        L.X2, stream));
-    else if (glue)
-      // the product linear, both readouts and the transpose of that linear (the start of the backward chain: seed -1 on
-      // every node energy, times the node's weight) on the same rows in one launch
-      CM_STAGE(10, cm_node_glue_readout(L.B2, L.sc, L.h1, w->prod_WT[1], w->prod_W[1], w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift,
-                                        g->node_weights, N, C, w->hidden, node_energy, L.d_h2, node_feats, g->node_rows, L.gB, stream));
     else
       CM_STAGE(t == 0 ? 4 : 10, cm_linear(B[t], w->prod_WT[t], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, t == 1 ? L.sc : none, h[t], stream));
   }
-  if (!glue)
-    CM_STAGE(11, cm_readout_forward(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden, node_energy,
+  CM_STAGE(11, cm_readout_forward(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden, node_energy,
                              L.d_h2, node_feats, g->node_rows, stream));
   if (!glue) {  // with the chained kernels the sums ride in the backward chain's launch
     cm::StageTimer timer_(st, 12, timing_mask);
@@ -404,17 +400,17 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   // own: the gradient with respect to the second layer's features is -d_h2 (the sign goes into the scale of the two
   // linears that consume it, which is exact; node weights scale its rows first), the one with respect to the first
   // layer's is a constant row (times the node's weight).
-  if (!glue) {  // the chained kernels form the constant rows and weight the rows of dE/dh2 themselves
+  if (!glue || g->node_weights) {  // the chained kernel forms the constant rows itself
     cm::StageTimer timer_(st, 13, timing_mask);
     const dim3 grid(static_cast<unsigned>(std::min<int64_t>(cm::ceil_div(N * C, 256), 2048)));
-    hipLaunchKernelGGL(cm::seed_linear_readout_kernel, grid, dim3(256), 0, st, L.g1, w->w1, w->scale, g->node_weights,
-                       static_cast<int64_t>(N) * C, C);
+    if (!glue)
+      hipLaunchKernelGGL(cm::seed_linear_readout_kernel, grid, dim3(256), 0, st, L.g1, w->w1, w->scale, g->node_weights,
+                         static_cast<int64_t>(N) * C, C);
     if (g->node_weights)
       hipLaunchKernelGGL(cm::weight_rows_kernel, grid, dim3(256), 0, st, L.d_h2, g->node_weights, static_cast<int64_t>(N) * C, C);
   }
   // layer 1 (second interaction)
-  if (!glue)
-    CM_STAGE(14, cm_linear(L.d_h2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, -1.0f, none, none, L.gB, stream));
+  CM_STAGE(14, cm_linear(L.d_h2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, -1.0f, none, none, L.gB, stream));
   CM_STAGE(15, cm_linear(L.bufM2, w->mix_W[1], nullptr, nullptr, N, 1, 0, 16, C, C, w->mix_scale[1], L.gB, none, L.bufA, stream));
   CM_STAGE(16, cm_mp_edge_backward(L.X2, L.vec, w->r_knots, w->spline[1], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
                               g->first_occ, g->sender_perm, g->sender_offsets, N, E, C, L.gX2, L.gv2, L.edge_scratch, stream));

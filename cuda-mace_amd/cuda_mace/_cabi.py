@@ -67,7 +67,6 @@ SIGNATURES = {
     "cm_node_glue_supported": (_i32, [_i32]),
     "cm_node_glue_forward": (_i32, [_p] * 6 + [_i64, _i32, _i32, _f32, _p, _p, _p, _p]),
     "cm_node_glue_backward": (_i32, [_p] * 6 + [_f64, _p, _p, _p, _i64, _i32, _i32, _f32, _p, _p]),
-    "cm_node_glue_readout": (_i32, [_p] * 8 + [_f64, _f64, _f64, _p, _i64, _i32, _i32] + [_p] * 6),
     "cm_neighbour_list_workspace": (_sz, [_i64, _i64]),
     "cm_neighbour_list_count": (_i32, [_p, _p, _i32, _i32, _i32, _f64, _i64, _i64, _p, _sz, _p, _p, _p]),
     "cm_neighbour_list_fill": (_i32, [_p, _f64, _i64, _i64, _p, _p, _i64, _p, _p, _p, _p, _p]),
@@ -492,24 +491,6 @@ def node_glue_backward(gX2, d_h2, up_W, skip_W, prod_W, w1, scale: float, node_w
                                      _dev(group_offsets, I32, "group_offsets"), N, ne + 1, C, float(skip_scale),
                                      _dev(gB1, F32, "gB1"), _stream()))
     return gB1
-
-
-def node_glue_readout(B2, sc, h1, prod_WT, prod_W, w1, W2a, w2b, act_cst: float, scale: float, shift: float, node_weights=None,
-                      want_feats: bool = True, feats_rows=None):
-    """(node_energies fp64 [N], d_h2 fp32 [N, C], feats fp64 [N, 2C] or None, gB2 fp32 [N, C]) of h2 = B2 . prod_W + sc, the
-    readouts of (h1, h2) and gB2 = -d_h2 . prod_W^T, in one launch."""
-    N, C = B2.shape
-    H = W2a.shape[1]
-    es = torch.empty(N, dtype=F64, device=B2.device)
-    d2 = torch.empty(N, C, dtype=F32, device=B2.device)
-    gB2 = torch.empty(N, C, dtype=F32, device=B2.device)
-    feats = torch.empty(N, 2 * C, dtype=F64, device=B2.device) if want_feats else None
-    _check(lib.cm_node_glue_readout(_dev(B2, F32, "B2"), _dev(sc, F32, "sc"), _dev(h1, F32, "h1"), _dev(prod_WT, F32, "prod_WT"),
-                                    _dev(prod_W, F32, "prod_W"), _dev(w1, F64, "w1"), _dev(W2a, F64, "W2a"), _dev(w2b, F64, "w2b"),
-                                    float(act_cst), float(scale), float(shift), _dev(node_weights, F64, "node_weights"), N, C, H,
-                                    _dev(es, F64, "node_energies"), _dev(d2, F32, "d_h2"), _dev(feats, F64, "node_feats64"),
-                                    _dev(feats_rows, I32, "feats_rows"), _dev(gB2, F32, "gB2"), _stream()))
-    return es, d2, feats, gB2
 
 
 # ---- symmetric contraction -----------------------------------------------------------------------------

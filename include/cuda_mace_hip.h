@@ -416,8 +416,7 @@ int cm_readout_backward(const double *grad_node_energies, const double *w1, cons
                         int64_t nnodes, int channels, float *grad_h1, float *grad_h2, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
- * The three [nnodes, C] x [C, C] linears between the two interaction layers as one launch per direction, and the
- * second layer's product linear with the readouts and its transpose as a third: the product's
+ * The three [nnodes, C] x [C, C] linears between the two interaction layers as one launch per direction: the product's
  * linear and linear_up (the reference's linear_matmul, models/InvariantMACE.py:41-53) and the per-element skip
  * connection between them (element_linear_to_cuda, :56-74; called at :145-150 and :330).  A workgroup takes 128 nodes
  * of one element through the chain with the intermediate rows in LDS; same arithmetic, rounding points and results as
@@ -429,16 +428,8 @@ int cm_readout_backward(const double *grad_node_energies, const double *w1, cons
  * Backward: gB1 = (gX2 . up_W^T + g1 - skip_scale * d_h2 . skip_W[element]^T) . prod_W^T with
  *   g1[n, c] = -node_weights[n] * scale * w1[c] (node_weights may be NULL = 1): the gradient of minus the weighted sum of
  *   node energies (cm_readout_forward's d_h2, scale, w1) through the chain; weights passed plain, [C in, C out].
- * End of the forward (cm_node_glue_readout): h2 = B2 . prod_W + sc; node energies, dE/dh2 and the fp64 feature
- *   concatenation exactly as cm_readout_forward(h1, h2, ...) returns them (h2 itself is not stored); with node_weights
- *   the rows of d_h2 come out multiplied by the node's weight; gB2 = -d_h2 . prod_W^T.  It stands for a cm_linear with a
- *   residual, cm_readout_forward and a cm_linear with scale -1, and returns their bits.
  */
 int cm_node_glue_supported(int channels);
-int cm_node_glue_readout(const float *B2, const float *sc, const float *h1, const float *prod_WT, const float *prod_W,
-                         const double *w1, const double *W2a, const double *w2b, double act_cst, double scale, double shift,
-                         const double *node_weights, int64_t nnodes, int channels, int hidden, double *node_energies,
-                         float *d_h2, double *node_feats64, const int32_t *feats_rows, float *gB2, cm_stream_t stream);
 int cm_node_glue_forward(const float *B1, const float *prod_WT, const float *skip_WT, const float *up_WT,
                          const int32_t *node_perm, const int32_t *group_offsets, int64_t nnodes, int ngroups, int channels,
                          float skip_scale, float *h1, float *sc, float *X2, cm_stream_t stream);

@@ -606,40 +606,6 @@ def test_readout_forward_backward(cabi, N, C, H, seed):
     assert only2[0] is None and torch.equal(only2[1], g2)
 
 
-@pytest.mark.parametrize("N,C,H,seed", [(1, 32, 16, 0), (21, 64, 16, 1), (300, 96, 7, 2), (4100, 128, 16, 3), (25000, 128, 16, 4)])
-def test_node_glue_readout_chain(cabi, N, C, H, seed):
-    """The second layer's product linear, the readouts and the transpose of that linear as one launch: bit for bit what
-    cm_linear (with residual), cm_readout_forward and cm_linear (scale -1) return one after the other, with and without
-    node weights and a row map of the feature output; energies and dE/dh2 also against the fp64 definition."""
-    _say("node_glue_readout", N, C, H, seed)
-    g = torch.Generator().manual_seed(seed)
-    rnd = lambda *shape: torch.randn(*shape, generator=g, dtype=torch.float64)  # noqa: E731
-    dev = lambda t: t.to(DEV).contiguous()  # noqa: E731
-    B2, sc, h1 = (dev(rnd(N, C).float()) for _ in range(3))
-    Wp = rnd(C, C) / math.sqrt(C)
-    WpT, Wpp = dev(Wp.t().float()), dev(Wp.float())
-    w1, W2a, w2b = dev(rnd(C) / C ** 0.5), dev(rnd(C, H) / C ** 0.5), dev(rnd(H) / H ** 0.5)
-    cst, scale, shift = 1.6791767923989418, 0.8, -0.3
-    nw = dev(torch.rand(N, generator=g, dtype=torch.float64))
-    rows = dev(torch.randperm(N, generator=g).int())
-    h2 = cabi.linear(B2, WpT, scale=1.0, residual=sc)
-    es_s, d2_s, feats_s = cabi.readout_forward(h1, h2, w1, W2a, w2b, cst, scale, shift, feats_rows=rows)
-    for weights in (None, nw):
-        es, d2, feats, gB2 = cabi.node_glue_readout(B2, sc, h1, WpT, Wpp, w1, W2a, w2b, cst, scale, shift, node_weights=weights,
-                                                    feats_rows=rows)
-        d2_w = d2_s if weights is None else (d2_s.double() * weights[:, None]).float()
-        assert torch.equal(es, es_s) and torch.equal(feats, feats_s) and torch.equal(d2, d2_w)
-        assert torch.equal(gB2, cabi.linear(d2_w, Wpp, scale=-1.0))
-    a2 = (B2.double().cpu() @ Wp.float().double() + sc.double().cpu()).requires_grad_(True)
-    ref = O.readout_energies(h1.double().cpu(), a2, w1.cpu(), W2a.cpu(), w2b.cpu(), cst, scale, shift)
-    ref.sum().backward()
-    es, d2, feats, gB2 = cabi.node_glue_readout(B2, sc, h1, WpT, Wpp, w1, W2a, w2b, cst, scale, shift, want_feats=False)
-    assert feats is None
-    close(es, ref.detach(), 2e-6, 2e-6)  # h2 is an fp32 product here
-    close(d2, a2.grad, 1e-4, 1e-5)
-    close(gB2, -(a2.grad @ Wp.float().double().t()), 1e-4, 1e-5)
-
-
 def test_linear_row_scale(cabi):
     """row_scale folds an element-wise factor shared by the 16 components into the operand load."""
     g = torch.Generator().manual_seed(3)
