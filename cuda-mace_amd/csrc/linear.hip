@@ -36,15 +36,19 @@ constexpr int kTileNodes = 32 * kWaves;  // rows per workgroup (MFMA M = 32 per 
 constexpr int kKC = 32;                  // K columns staged per step
 constexpr int kLdH = kKC + 8;            // padded LDS row stride of a bf16 plane (elements; 80 bytes: conflict-free b128 reads)
 
-// Nout = 32 * NT; SCALED: X is multiplied by row_scale on the way in
+// A workgroup computes 32 * NT output columns, starting at column blockIdx.y * 32 * NT of the nout_total columns of a row
+// (one workgroup per tile for all columns where there are many tiles; few tiles are spread over more workgroups, 32
+// columns each, which shortens the chain of staging and matrix instructions a tile waits for: every output element sums
+// the same products in the same order either way).  SCALED: X is multiplied by row_scale on the way in
 template <int NT, bool SCALED>
 __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__restrict__ X, const float *__restrict__ WT,
                                                                const int32_t *__restrict__ node_perm,
                                                                const int32_t *__restrict__ group_offsets, int nnodes,
                                                                int ngroups, int zero_last_group, int ncomp, int K,
                                                                float scale, const float *__restrict__ row_scale,
-                                                               const float *residual, float *OUT) {
+                                                               const float *residual, float *OUT, int nout_total) {
   constexpr int NOUT = 32 * NT;
+  const int col0 = blockIdx.y * NOUT;
   // three bf16 planes per operand: plane p of X at sAp + p * kTileNodes * kLdH, of the weights at sBp + p * NOUT * kLdH
   // (77 KB at Nout = 192, 92 KB at 256: beyond 64 KB, within the 160 KB of a gfx950 compute unit)
   __shared__ __attribute__((aligned(16))) __bf16 sAp[3 * kTileNodes * kLdH];
@@ -98,13 +102,13 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
     for (int i = tid; i < kTileNodes * NOUT; i += kWaves * kWave) {
       const int node = sNode[i / NOUT];
       if (node >= 0) {
-        const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + i % NOUT;
+        const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * nout_total + col0 + i % NOUT;
         OUT[at] = residual ? residual[at] : 0.f;
       }
     }
     return;
   }
-  const float *Wg = WT + (static_cast<int64_t>(g) * nblocks + l) * NOUT * K;  // [NOUT, K]
+  const float *Wg = WT + ((static_cast<int64_t>(g) * nblocks + l) * nout_total + col0) * K;  // [NOUT, K] of [nout_total, K]
 
   v16f acc[NT];
 #pragma unroll
@@ -200,12 +204,16 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
     const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
     const int node = sNode[row];
     if (node >= 0) {
-      const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
+      const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * nout_total + col0 + mrow;
       float *op = OUT + at;
       if (residual) {  // may be OUT itself: every element is read and written by the same lane
         const float *rp = residual + at;
 #pragma unroll
-        for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale + rp[32 * t];
+        for (int t = 0; t < NT; ++t) {
+#pragma clang fp contract(off)  // the product is rounded before the residual is added, as in the kernels that stage it in LDS
+          const float v = acc[t][r] * scale;
+          op[32 * t] = v + rp[32 * t];
+        }
       } else {
 #pragma unroll
         for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
@@ -489,7 +497,11 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
         if (residual) {  // may be OUT itself: every element is read and written by the same lane
           const float *rp = residual + at;
 #pragma unroll
-          for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale + rp[32 * t];
+          for (int t = 0; t < NT; ++t) {
+#pragma clang fp contract(off)
+            const float v = acc[t][r] * scale;
+            op[32 * t] = v + rp[32 * t];
+          }
         } else {
 #pragma unroll
           for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
@@ -853,6 +865,18 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
            hipStream_t st) {
   const int64_t tiles = ceil_div(nnodes, kTileNodes) + (offs ? ngroups : 0);
   const dim3 grid(static_cast<unsigned>(tiles * ncomp)), block(kWaves * kWave);
+  constexpr int NOUT = 32 * NT;
+  // few tiles (less than half a workgroup per compute unit): 32 columns per workgroup
+  if (NT > 1 && tiles * ncomp * 2 <= device_compute_units()) {
+    const dim3 split(grid.x, NT);
+    if (row_scale)
+      hipLaunchKernelGGL((linear_kernel<1, true>), split, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                         zero_last_group, ncomp, K, scale, row_scale, residual, OUT, NOUT);
+    else
+      hipLaunchKernelGGL((linear_kernel<1, false>), split, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
+                         zero_last_group, ncomp, K, scale, row_scale, residual, OUT, NOUT);
+    return check_launch("cm_linear");
+  }
   // The ring variant wherever it runs two workgroups per compute unit or the plain one does not either (Nout up to 128,
   // and 224 / 256), and K has more than one chunk to overlap; measured at 25 000 nodes: 108 vs 119-127 us at 128
   // columns, 76 vs 80-83 at 96, equal at 64, 224 and 256, slower at 32 (one chunk), 160 and 192 (one workgroup per CU).
@@ -877,10 +901,10 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
   }
   if (row_scale)
     hipLaunchKernelGGL((linear_kernel<NT, true>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
-                       zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
+                       zero_last_group, ncomp, K, scale, row_scale, residual, OUT, NOUT);
   else
     hipLaunchKernelGGL((linear_kernel<NT, false>), grid, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
-                       zero_last_group, ncomp, K, scale, row_scale, residual, OUT);
+                       zero_last_group, ncomp, K, scale, row_scale, residual, OUT, NOUT);
   return check_launch("cm_linear");
 }
 

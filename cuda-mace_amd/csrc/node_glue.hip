@@ -28,55 +28,79 @@
 namespace cm {
 namespace {
 
-constexpr int kGlWaves = 4;
-constexpr int kGlTile = 32 * kGlWaves;  // nodes per workgroup
-constexpr int kGlKC = 32;               // K columns staged per step
-constexpr int kGlLdH = kGlKC + 8;       // padded row stride of a bf16 plane (elements)
+constexpr int kGlTile = 128;       // nodes per workgroup
+constexpr int kGlKC = 32;          // K columns staged per step
+constexpr int kGlLdH = kGlKC + 8;  // padded row stride of a bf16 plane (elements)
+constexpr int kGlTPR = kGlKC / 4;  // threads that cover the 32 columns of a staged row, 16 bytes each
+constexpr int kGlSumThreads = 256; // threads that take part in a graph's energy sum
 
+// A workgroup has 4 * NT waves (C = 32 NT): wave w owns the 32 x 32 block of the tile's output at rows 32 (w % 4),
+// columns 32 (w / 4).  With one wave per block a product's matrix instructions, operand reads and staging are spread over
+// four waves per SIMD, which hide each other's latencies; with four waves and NT blocks each, a chain of three products
+// on one tile took twice as long (26 against 13 us at 128 channels).
 template <int NT>
 struct GlueShared {
   static constexpr int C = 32 * NT;
+  static constexpr int kThreads = 4 * NT * kWave;
   static constexpr int kLdT = C + 4;  // padded row stride of the fp32 tile (floats): rows 16 bytes apart in bank space
+  // pieces of 16 bytes per thread and K chunk: X (128 rows x 8 pieces over kThreads threads), weights (C rows x 8: one)
+  static constexpr int kAPieces = (kGlTile * kGlTPR + kThreads - 1) / kThreads;
   __bf16 a[3 * kGlTile * kGlLdH];
   __bf16 b[3 * C * kGlLdH];
   float tile[kGlTile * kLdT];
   int node[kGlTile];
 };
 
-// Tile of the grouped node order that a workgroup owns: false when the workgroup has none.
+// Tile of the grouped node order that a workgroup owns: false when the workgroup has none.  Up to 64 groups are
+// searched with one load per lane and a prefix sum over the lanes (a loop over the groups is a chain of dependent loads:
+// microseconds at the head of a kernel that runs for ten).
 __device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ group_offsets, int ngroups, int nnodes, int tile, int &g,
                                             int &pos0, int &gend) {
   g = 0, pos0 = 0, gend = nnodes;
-  if (group_offsets) {
-    for (g = 0; g < ngroups; ++g) {
-      const int lo = group_offsets[g], hi = group_offsets[g + 1];
-      const int tiles = (hi - lo + kGlTile - 1) / kGlTile;
-      if (tile < tiles) {
-        pos0 = lo + tile * kGlTile;
-        gend = hi;
-        return true;
-      }
-      tile -= tiles;
-    }
-    return false;
+  if (!group_offsets) {
+    pos0 = tile * kGlTile;
+    return pos0 < nnodes;
   }
-  pos0 = tile * kGlTile;
-  return pos0 < nnodes;
+  if (ngroups <= kWave) {
+    const int lane = threadIdx.x % kWave;
+    const int lo = lane < ngroups ? group_offsets[lane] : 0, hi = lane < ngroups ? group_offsets[lane + 1] : 0;
+    const int tiles = (hi - lo + kGlTile - 1) / kGlTile;
+    int upto = tiles;  // inclusive prefix sum over the lanes
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int v = __shfl_up(upto, d);
+      if (lane >= d) upto += v;
+    }
+    const unsigned long long owners = __ballot(tile < upto);
+    if (owners == 0) return false;
+    g = __ffsll(static_cast<long long>(owners)) - 1;
+    const int first = __shfl(upto - tiles, g);
+    pos0 = __shfl(lo, g) + (tile - first) * kGlTile;
+    gend = __shfl(hi, g);
+    return true;
+  }
+  for (g = 0; g < ngroups; ++g) {
+    const int lo = group_offsets[g], hi = group_offsets[g + 1];
+    const int tiles = (hi - lo + kGlTile - 1) / kGlTile;
+    if (tile < tiles) {
+      pos0 = lo + tile * kGlTile;
+      gend = hi;
+      return true;
+    }
+    tile -= tiles;
+  }
+  return false;
 }
 
 // Operands of a product on their way from memory: a thread's 16-byte pieces of every K chunk, requested all at once
-// and long before the product that consumes them (a chain of three products otherwise pays a memory latency per chunk).
-// Staging map: eight threads cover the 32 columns of a chunk of one row, 32 rows per pass.
-constexpr int kGlTPR = kGlKC / 4;                  // threads per staged row
-constexpr int kGlRPP = kGlWaves * kWave / kGlTPR;  // rows per pass
-constexpr int kGlAPasses = kGlTile / kGlRPP;
+// and long before the product that consumes them.
 template <int NT>
 struct WeightPieces {
-  f4 v[NT][NT];  // [chunk][pass]: row 32 pass + tid / 8 of the transposed block, columns 32 chunk + 4 (tid % 8) ..
+  f4 v[NT];  // [chunk]: row tid / 8 of the transposed block, columns 32 chunk + 4 (tid % 8) ..
 };
 template <int NT>
 struct RowPieces {
-  f4 v[NT][kGlAPasses];
+  f4 v[NT][GlueShared<NT>::kAPieces];
 };
 
 template <int NT>
@@ -84,61 +108,62 @@ __device__ __forceinline__ void fetch_weights(const float *__restrict__ Wg, Weig
   constexpr int C = 32 * NT;
   const int srow = threadIdx.x / kGlTPR, scol = (threadIdx.x % kGlTPR) * 4;
 #pragma unroll
-  for (int k = 0; k < NT; ++k)
-#pragma unroll
-    for (int i = 0; i < NT; ++i) w.v[k][i] = ld4(Wg + static_cast<int64_t>(kGlRPP * i + srow) * C + kGlKC * k + scol);
+  for (int k = 0; k < NT; ++k) w.v[k] = ld4(Wg + static_cast<int64_t>(srow) * C + kGlKC * k + scol);
 }
 
 // rows of X [*, C] named by the tile's node list (zeros for rows beyond the tile)
 template <int NT>
 __device__ __forceinline__ void fetch_rows(const GlueShared<NT> &s, const float *__restrict__ X, RowPieces<NT> &a) {
+  using S = GlueShared<NT>;
   constexpr int C = 32 * NT;
-  const int srow = threadIdx.x / kGlTPR, scol = (threadIdx.x % kGlTPR) * 4;
 #pragma unroll
-  for (int i = 0; i < kGlAPasses; ++i) {
-    const int node = s.node[kGlRPP * i + srow];
+  for (int i = 0; i < S::kAPieces; ++i) {
+    const int piece = threadIdx.x + i * S::kThreads;
+    const int row = piece / kGlTPR, scol = (piece % kGlTPR) * 4;
+    const int node = row < kGlTile ? s.node[row] : -1;
 #pragma unroll
     for (int k = 0; k < NT; ++k) a.v[k][i] = node >= 0 ? ld4(X + static_cast<int64_t>(node) * C + kGlKC * k + scol) : zero4();
   }
 }
 
-// acc = X . W over K = C.  X: the pieces fetched by fetch_rows, or (FROM_TILE) the fp32 tile in LDS; W: the pieces fetched
-// by fetch_weights from the transposed block [C out, C in].  All threads of the workgroup take part; on return the
-// operand planes may still be read by slower waves: whatever overwrites them next sits behind a barrier.
+// acc = the wave's 32 x 32 block of X . W over K = C.  X: the pieces fetched by fetch_rows, or (FROM_TILE) the fp32 tile in
+// LDS; W: the pieces fetched by fetch_weights from the transposed block [C out, C in].  All threads of the workgroup
+// take part; on return the operand planes may still be read by slower waves: whatever overwrites them next sits behind
+// a barrier.
 template <int NT, bool FROM_TILE>
-__device__ __forceinline__ void product(GlueShared<NT> &s, const RowPieces<NT> *rows, const WeightPieces<NT> &w, v16f (&acc)[NT]) {
+__device__ __forceinline__ void product(GlueShared<NT> &s, const RowPieces<NT> *rows, const WeightPieces<NT> &w, v16f &acc) {
   constexpr int C = 32 * NT;
   using S = GlueShared<NT>;
   const int tid = threadIdx.x;
   const int lane = tid % kWave, wave = tid / kWave;
-  const int srow = tid / kGlTPR, scol = (tid % kGlTPR) * 4;
+  const int wr = wave % 4, wc = wave / 4;
   const int mrow = lane % 32, half = lane / 32;
 #pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
 #pragma unroll
   for (int k = 0; k < NT; ++k) {
     __syncthreads();  // previous chunk fully consumed (and, before the first, the tile complete)
 #pragma unroll
-    for (int i = 0; i < kGlAPasses; ++i) {
+    for (int i = 0; i < S::kAPieces; ++i) {
+      const int piece = tid + i * S::kThreads;
+      const int row = piece / kGlTPR, scol = (piece % kGlTPR) * 4;
+      if (S::kAPieces * S::kThreads != kGlTile * kGlTPR && row >= kGlTile) continue;
       f4 x;
       if constexpr (FROM_TILE)
-        x = *reinterpret_cast<const f4 *>(s.tile + (kGlRPP * i + srow) * S::kLdT + kGlKC * k + scol);
+        x = *reinterpret_cast<const f4 *>(s.tile + row * S::kLdT + kGlKC * k + scol);
       else
         x = rows->v[k][i];
       bf16x4 h, md, lw;
       split3(x, h, md, lw);
-      const int at = (kGlRPP * i + srow) * kGlLdH + scol;
+      const int at = row * kGlLdH + scol;
       *reinterpret_cast<bf16x4 *>(s.a + at) = h;
       *reinterpret_cast<bf16x4 *>(s.a + kGlTile * kGlLdH + at) = md;
       *reinterpret_cast<bf16x4 *>(s.a + 2 * kGlTile * kGlLdH + at) = lw;
     }
-#pragma unroll
-    for (int i = 0; i < NT; ++i) {
+    {
       bf16x4 h, md, lw;
-      split3(w.v[k][i], h, md, lw);
-      const int at = (kGlRPP * i + srow) * kGlLdH + scol;
+      split3(w.v[k], h, md, lw);
+      const int at = (tid / kGlTPR) * kGlLdH + (tid % kGlTPR) * 4;
       *reinterpret_cast<bf16x4 *>(s.b + at) = h;
       *reinterpret_cast<bf16x4 *>(s.b + C * kGlLdH + at) = md;
       *reinterpret_cast<bf16x4 *>(s.b + 2 * C * kGlLdH + at) = lw;
@@ -146,43 +171,30 @@ __device__ __forceinline__ void product(GlueShared<NT> &s, const RowPieces<NT> *
     __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < kGlKC; ks += 16) {
-      const int aoff = (32 * wave + mrow) * kGlLdH + ks + 8 * half;
-      bf16x8 a[3], b[NT][3];
+      bf16x8 a[3], b[3];
 #pragma unroll
-      for (int p = 0; p < 3; ++p) a[p] = *reinterpret_cast<const bf16x8 *>(s.a + p * kGlTile * kGlLdH + aoff);
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int p = 0; p < 3; ++p)
-          b[t][p] = *reinterpret_cast<const bf16x8 *>(s.b + p * C * kGlLdH + (32 * t + mrow) * kGlLdH + ks + 8 * half);
+      for (int p = 0; p < 3; ++p) {
+        a[p] = *reinterpret_cast<const bf16x8 *>(s.a + p * kGlTile * kGlLdH + (32 * wr + mrow) * kGlLdH + ks + 8 * half);
+        b[p] = *reinterpret_cast<const bf16x8 *>(s.b + p * C * kGlLdH + (32 * wc + mrow) * kGlLdH + ks + 8 * half);
+      }
       // piece products from small to large, as in the linear kernels
-#pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], b[t][0], acc[t], 0, 0, 0);
-#pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][2], acc[t], 0, 0, 0);
-#pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[t][1], acc[t], 0, 0, 0);
-#pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[t][0], acc[t], 0, 0, 0);
-#pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][1], acc[t], 0, 0, 0);
-#pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][0], acc[t], 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], b[0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[2], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[1], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[1], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[0], acc, 0, 0, 0);
     }
   }
 }
 
-// Accumulator r of a lane is row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32 + 32 t of the wave's block.
-template <int NT, class F>
-__device__ __forceinline__ void for_each_output(const v16f (&acc)[NT], F f) {
+// Accumulator r of a lane is row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32 of the wave's block.
+template <class F>
+__device__ __forceinline__ void for_each_output(const v16f &acc, F f) {
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   const int mrow = lane % 32, half = lane / 32;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
-#pragma unroll
-    for (int t = 0; t < NT; ++t) f(row, 32 * t + mrow, acc[t][r]);
-  }
+  for (int r = 0; r < 16; ++r) f(32 * (wave % 4) + 8 * (r / 4) + 4 * half + (r % 4), 32 * (wave / 4) + mrow, acc[r]);
 }
 
 template <int NT>
@@ -201,7 +213,7 @@ __device__ __forceinline__ void stage_nodes(GlueShared<NT> &s, const int32_t *__
 
 // ---- forward: h1 = B1 . Wprod, sc = skip_scale h1 . Wskip[element], X2 = h1 . Wup ---------------------------------
 template <int NT>
-__global__ __launch_bounds__(kGlWaves *kWave) void node_glue_forward_kernel(
+__global__ __launch_bounds__(4 * NT *kWave) void node_glue_forward_kernel(
     const float *__restrict__ B1, const float *__restrict__ prod_WT, const float *__restrict__ skip_WT,
     const float *__restrict__ up_WT, const int32_t *__restrict__ node_perm, const int32_t *__restrict__ group_offsets, int nnodes,
     int ngroups, float skip_scale, float *__restrict__ h1, float *__restrict__ sc, float *__restrict__ X2) {
@@ -219,10 +231,10 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_forward_kernel(
   fetch_rows<NT>(s, B1, a0);
   if (!no_element) fetch_weights<NT>(skip_WT + static_cast<int64_t>(g) * C * C, wb);  // in flight during the first product
 
-  v16f acc[NT];
+  v16f acc;
   product<NT, false>(s, &a0, wa, acc);
   fetch_weights<NT>(up_WT, wa);
-  for_each_output<NT>(acc, [&](int row, int col, float v) {
+  for_each_output(acc, [&](int row, int col, float v) {
     const float out = v * 1.0f;
     s.tile[row * S::kLdT + col] = out;
     const int node = s.node[row];
@@ -230,26 +242,26 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_forward_kernel(
   });
   // (the tile is complete behind the barrier at the top of the next product)
   if (no_element) {
-    for_each_output<NT>(acc, [&](int row, int col, float) {
+    for_each_output(acc, [&](int row, int col, float) {
       const int node = s.node[row];
       if (node >= 0) sc[static_cast<int64_t>(node) * C + col] = 0.f;
     });
   } else {
     product<NT, true>(s, nullptr, wb, acc);
-    for_each_output<NT>(acc, [&](int row, int col, float v) {
+    for_each_output(acc, [&](int row, int col, float v) {
       const int node = s.node[row];
       if (node >= 0) sc[static_cast<int64_t>(node) * C + col] = v * skip_scale;
     });
   }
   product<NT, true>(s, nullptr, wa, acc);
-  for_each_output<NT>(acc, [&](int row, int col, float v) {
+  for_each_output(acc, [&](int row, int col, float v) {
     const int node = s.node[row];
     if (node >= 0) X2[static_cast<int64_t>(node) * C + col] = v * 1.0f;
   });
 }
 
 // Energies per graph, riding in the backward launch (its tiles do not depend on them): out[g] = sum over the graph's nodes
-// of weight[n] * node_es[n], strided partial sums of the workgroup's 256 threads and a tree over them: a fixed order.
+// of weight[n] * node_es[n], strided partial sums of 256 threads and a tree over them: a fixed order.
 struct EnergySums {
   const double *node_es, *node_weights;
   const int32_t *graph_ptr;
@@ -258,12 +270,14 @@ struct EnergySums {
 };
 __device__ __forceinline__ void graph_energy(const EnergySums &q, int graph, double *part) {
   const int tid = threadIdx.x;
-  const int lo = q.graph_ptr[graph], hi = q.graph_ptr[graph + 1];
-  double sum = 0.0;
-  for (int i = lo + tid; i < hi; i += kGlWaves * kWave) sum += q.node_weights ? q.node_weights[i] * q.node_es[i] : q.node_es[i];
-  part[tid] = sum;
+  if (tid < kGlSumThreads) {
+    const int lo = q.graph_ptr[graph], hi = q.graph_ptr[graph + 1];
+    double sum = 0.0;
+    for (int i = lo + tid; i < hi; i += kGlSumThreads) sum += q.node_weights ? q.node_weights[i] * q.node_es[i] : q.node_es[i];
+    part[tid] = sum;
+  }
   __syncthreads();
-  for (int d = kGlWaves * kWave / 2; d > 0; d >>= 1) {
+  for (int d = kGlSumThreads / 2; d > 0; d >>= 1) {
     if (tid < d) part[tid] += part[tid + d];
     __syncthreads();
   }
@@ -272,7 +286,7 @@ __device__ __forceinline__ void graph_energy(const EnergySums &q, int graph, dou
 
 // ---- backward: gh1 = gX2 . Wup^T + g1 - skip_scale dE/dh2 . Wskip[element]^T, gB1 = gh1 . Wprod^T ------------------
 template <int NT>
-__global__ __launch_bounds__(kGlWaves *kWave) void node_glue_backward_kernel(
+__global__ __launch_bounds__(4 * NT *kWave) void node_glue_backward_kernel(
     const float *__restrict__ gX2, const float *__restrict__ d_h2, const float *__restrict__ up_W, const float *__restrict__ skip_W,
     const float *__restrict__ prod_W, const double *__restrict__ w1, double scale, const double *__restrict__ node_weights,
     const int32_t *__restrict__ node_perm, const int32_t *__restrict__ group_offsets, int nnodes, int ngroups, float skip_scale,
@@ -299,10 +313,10 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_backward_kernel(
     fetch_rows<NT>(s, d_h2, a1);
   }
 
-  v16f acc[NT];
+  v16f acc;
   product<NT, false>(s, &a0, wa, acc);
   fetch_weights<NT>(prod_W, wa);
-  for_each_output<NT>(acc, [&](int row, int col, float v) {
+  for_each_output(acc, [&](int row, int col, float v) {
     const int node = s.node[row];
     const double nw = (node_weights && node >= 0) ? node_weights[node] : 1.0;
     const float g1 = static_cast<float>(-1.0 * scale * w1[col] * nw);
@@ -312,13 +326,13 @@ __global__ __launch_bounds__(kGlWaves *kWave) void node_glue_backward_kernel(
   if (!no_element) {
     product<NT, false>(s, &a1, wb, acc);
     // each element of the tile is read and written by the lane that wrote it above
-    for_each_output<NT>(acc, [&](int row, int col, float v) {
+    for_each_output(acc, [&](int row, int col, float v) {
       const float part = v * -skip_scale;
       s.tile[row * S::kLdT + col] += part;
     });
   }
   product<NT, true>(s, nullptr, wa, acc);
-  for_each_output<NT>(acc, [&](int row, int col, float v) {
+  for_each_output(acc, [&](int row, int col, float v) {
     const int node = s.node[row];
     if (node >= 0) gB1[static_cast<int64_t>(node) * C + col] = v * 1.0f;
   });
@@ -329,7 +343,7 @@ void launch_forward(const float *B1, const float *prod_WT, const float *skip_WT,
                     const int32_t *offs, int64_t nnodes, int ngroups, float skip_scale, float *h1, float *sc, float *X2,
                     hipStream_t st) {
   const unsigned tiles = static_cast<unsigned>(ceil_div(nnodes, kGlTile) + ngroups);
-  hipLaunchKernelGGL(node_glue_forward_kernel<NT>, dim3(tiles), dim3(kGlWaves * kWave), 0, st, B1, prod_WT, skip_WT, up_WT, perm,
+  hipLaunchKernelGGL(node_glue_forward_kernel<NT>, dim3(tiles), dim3(4 * NT * kWave), 0, st, B1, prod_WT, skip_WT, up_WT, perm,
                      offs, static_cast<int>(nnodes), ngroups, skip_scale, h1, sc, X2);
 }
 
@@ -339,7 +353,7 @@ void launch_backward(const float *gX2, const float *d_h2, const float *up_W, con
                      int64_t nnodes, int ngroups, float skip_scale, float *gB1, const EnergySums &sums, hipStream_t st) {
   const int tiles = static_cast<int>(ceil_div(nnodes, kGlTile) + ngroups);
   const unsigned extra = sums.out ? static_cast<unsigned>(sums.ngraphs) : 0u;
-  hipLaunchKernelGGL(node_glue_backward_kernel<NT>, dim3(static_cast<unsigned>(tiles) + extra), dim3(kGlWaves * kWave), 0, st, gX2, d_h2,
+  hipLaunchKernelGGL(node_glue_backward_kernel<NT>, dim3(static_cast<unsigned>(tiles) + extra), dim3(4 * NT * kWave), 0, st, gX2, d_h2,
                      up_W, skip_W, prod_W, w1, scale, node_weights, perm, offs, static_cast<int>(nnodes), ngroups, skip_scale, gB1, sums,
                      static_cast<int>(extra));
 }

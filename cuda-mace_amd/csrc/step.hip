@@ -364,8 +364,9 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   float *B[2] = {L.B1, L.B2};
   float *h[2] = {L.h1, L.h2};
   // the three [N, C] products between the layers (and their three transposes in the backward) as one launch each
-  const char *glue_env = getenv("CM_STEP_GLUE");  // development switch: 0 keeps the separate launches
-  const bool glue = cm_node_glue_supported(C) != 0 && !(glue_env && atoi(glue_env) == 0);
+  const char *glue_env = getenv("CM_STEP_GLUE");  // development switch: smallest node count that takes the chained kernels; -1: none
+  const int glue_min = glue_env ? atoi(glue_env) : 0;
+  const bool glue = cm_node_glue_supported(C) != 0 && glue_min >= 0 && N >= glue_min;
   for (int t = 0; t < 2; ++t) {
     if (t == 1 && !glue) {
       // residual skip connection per element and linear_up, both of the first layer's output
