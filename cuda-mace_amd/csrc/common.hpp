@@ -65,6 +65,49 @@ __host__ __device__ __forceinline__ void clamp_edge_range(int &e0, int &e1, int6
   e1 = e1 < e0 ? e0 : (e1 > ne ? ne : e1);
 }
 
+// Tile `tile` of `tile_rows` consecutive positions of the grouped node order (tiles do not straddle groups; without
+// groups, of the plain node order): its group g, first position pos0 and the end of its group; false when there is no
+// such tile.  Called by all threads of a workgroup with the same arguments (whole waves).  Up to 64 groups are
+// searched with one load per lane and a prefix sum over the lanes (a loop over the groups is a chain of dependent loads:
+// microseconds at the head of a kernel that runs for ten).
+__device__ __forceinline__ bool locate_group_tile(const int32_t *__restrict__ group_offsets, int ngroups, int nnodes, int tile,
+                                                  int tile_rows, int &g, int &pos0, int &gend) {
+  g = 0, pos0 = 0, gend = nnodes;
+  if (!group_offsets) {
+    pos0 = tile * tile_rows;
+    return pos0 < nnodes;
+  }
+  if (ngroups <= kWave) {
+    const int lane = threadIdx.x % kWave;
+    const int lo = lane < ngroups ? group_offsets[lane] : 0, hi = lane < ngroups ? group_offsets[lane + 1] : 0;
+    const int tiles = (hi - lo + tile_rows - 1) / tile_rows;
+    int upto = tiles;  // inclusive prefix sum over the lanes
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int v = __shfl_up(upto, d);
+      if (lane >= d) upto += v;
+    }
+    const unsigned long long owners = __ballot(tile < upto);
+    if (owners == 0) return false;
+    g = __ffsll(static_cast<long long>(owners)) - 1;
+    const int first = __shfl(upto - tiles, g);
+    pos0 = __shfl(lo, g) + (tile - first) * tile_rows;
+    gend = __shfl(hi, g);
+    return true;
+  }
+  for (g = 0; g < ngroups; ++g) {
+    const int lo = group_offsets[g], hi = group_offsets[g + 1];
+    const int tiles = (hi - lo + tile_rows - 1) / tile_rows;
+    if (tile < tiles) {
+      pos0 = lo + tile * tile_rows;
+      gend = hi;
+      return true;
+    }
+    tile -= tiles;
+  }
+  return false;
+}
+
 // Orders LDS traffic of one wavefront: stores issued before are visible to loads issued after.
 __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -65,26 +65,8 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
   const int nblocks = ncomp == 1 ? 1 : 4;  // weight blocks per group
 
   // locate (group, first position in the grouped node order) of this tile
-  int tile = blockIdx.x / ncomp;
-  int g = 0, pos0 = 0, gend = nnodes;
-  if (group_offsets) {
-    bool found = false;
-    for (g = 0; g < ngroups; ++g) {
-      const int lo = group_offsets[g], hi = group_offsets[g + 1];
-      const int tiles = (hi - lo + kTileNodes - 1) / kTileNodes;
-      if (tile < tiles) {
-        pos0 = lo + tile * kTileNodes;
-        gend = hi;
-        found = true;
-        break;
-      }
-      tile -= tiles;
-    }
-    if (!found) return;
-  } else {
-    pos0 = tile * kTileNodes;
-    if (pos0 >= nnodes) return;
-  }
+  int g, pos0, gend;
+  if (!locate_group_tile(group_offsets, ngroups, nnodes, blockIdx.x / ncomp, kTileNodes, g, pos0, gend)) return;
   const int nrows = min(kTileNodes, gend - pos0);
 
   if (tid < kTileNodes) {
@@ -282,26 +264,8 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
   const int l = ncomp == 1 ? 0 : l_of_m(m);
   const int nblocks = ncomp == 1 ? 1 : 4;
 
-  int tile = blockIdx.x / ncomp;
-  int g = 0, pos0 = 0, gend = nnodes;
-  if (group_offsets) {
-    bool found = false;
-    for (g = 0; g < ngroups; ++g) {
-      const int lo = group_offsets[g], hi = group_offsets[g + 1];
-      const int tiles = (hi - lo + kTileNodes - 1) / kTileNodes;
-      if (tile < tiles) {
-        pos0 = lo + tile * kTileNodes;
-        gend = hi;
-        found = true;
-        break;
-      }
-      tile -= tiles;
-    }
-    if (!found) return;
-  } else {
-    pos0 = tile * kTileNodes;
-    if (pos0 >= nnodes) return;
-  }
+  int g, pos0, gend;
+  if (!locate_group_tile(group_offsets, ngroups, nnodes, blockIdx.x / ncomp, kTileNodes, g, pos0, gend)) return;
   const int nrows = min(kTileNodes, gend - pos0);
 
   if (tid < kTileNodes) {

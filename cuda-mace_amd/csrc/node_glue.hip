@@ -51,47 +51,6 @@ struct GlueShared {
   int node[kGlTile];
 };
 
-// Tile of the grouped node order that a workgroup owns: false when the workgroup has none.  Up to 64 groups are
-// searched with one load per lane and a prefix sum over the lanes (a loop over the groups is a chain of dependent loads:
-// microseconds at the head of a kernel that runs for ten).
-__device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ group_offsets, int ngroups, int nnodes, int tile, int &g,
-                                            int &pos0, int &gend) {
-  g = 0, pos0 = 0, gend = nnodes;
-  if (!group_offsets) {
-    pos0 = tile * kGlTile;
-    return pos0 < nnodes;
-  }
-  if (ngroups <= kWave) {
-    const int lane = threadIdx.x % kWave;
-    const int lo = lane < ngroups ? group_offsets[lane] : 0, hi = lane < ngroups ? group_offsets[lane + 1] : 0;
-    const int tiles = (hi - lo + kGlTile - 1) / kGlTile;
-    int upto = tiles;  // inclusive prefix sum over the lanes
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const int v = __shfl_up(upto, d);
-      if (lane >= d) upto += v;
-    }
-    const unsigned long long owners = __ballot(tile < upto);
-    if (owners == 0) return false;
-    g = __ffsll(static_cast<long long>(owners)) - 1;
-    const int first = __shfl(upto - tiles, g);
-    pos0 = __shfl(lo, g) + (tile - first) * kGlTile;
-    gend = __shfl(hi, g);
-    return true;
-  }
-  for (g = 0; g < ngroups; ++g) {
-    const int lo = group_offsets[g], hi = group_offsets[g + 1];
-    const int tiles = (hi - lo + kGlTile - 1) / kGlTile;
-    if (tile < tiles) {
-      pos0 = lo + tile * kGlTile;
-      gend = hi;
-      return true;
-    }
-    tile -= tiles;
-  }
-  return false;
-}
-
 // Operands of a product on their way from memory: a thread's 16-byte pieces of every K chunk, requested all at once
 // and long before the product that consumes them.
 template <int NT>
@@ -221,7 +180,7 @@ __global__ __launch_bounds__(4 * NT *kWave) void node_glue_forward_kernel(
   using S = GlueShared<NT>;
   __shared__ __attribute__((aligned(16))) S s;
   int g, pos0, gend;
-  if (!locate_tile(group_offsets, ngroups, nnodes, blockIdx.x, g, pos0, gend)) return;
+  if (!locate_group_tile(group_offsets, ngroups, nnodes, blockIdx.x, kGlTile, g, pos0, gend)) return;
   stage_nodes<NT>(s, node_perm, pos0, gend, nnodes);
 
   const bool no_element = g == ngroups - 1;  // nodes of no element: the skip connection is defined as zero there
@@ -300,7 +259,7 @@ __global__ __launch_bounds__(4 * NT *kWave) void node_glue_backward_kernel(
     return;
   }
   int g, pos0, gend;
-  if (!locate_tile(group_offsets, ngroups, nnodes, blockIdx.x - first_tile, g, pos0, gend)) return;
+  if (!locate_group_tile(group_offsets, ngroups, nnodes, blockIdx.x - first_tile, kGlTile, g, pos0, gend)) return;
   stage_nodes<NT>(s, node_perm, pos0, gend, nnodes);
 
   const bool no_element = g == ngroups - 1;

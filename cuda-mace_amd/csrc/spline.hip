@@ -220,7 +220,7 @@ __global__ __launch_bounds__(kSpThreads) void spline_backward_sliced_kernel(
           part += __shfl_xor(part, 1);
           part += __shfl_xor(part, 2);
           part += __shfl_xor(part, 4);
-          if (q == 0 && base + src < n) atomicAdd(&sSum[base + src], part);  // this lane group alone adds to the cell in this slice
+          if (q == 0 && base + src < n) sSum[base + src] += part;  // this lane alone adds to the cell in this slice; slices are barriers apart
         }
       }
     }

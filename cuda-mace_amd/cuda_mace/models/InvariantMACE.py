@@ -52,14 +52,14 @@ def get_edge_vectors_and_lengths(positions, edge_index, shifts) -> Tuple[torch.T
 
 
 class _RowsOfSortedIndex(torch.autograd.Function):
-    """src[index] for a non-decreasing index whose segment boundaries are `offsets` (offsets[g] = first position with
-    index g).  The backward is one reduction per segment (a slice each); the plain gather's backward adds every row into
+    """src[index] for a non-decreasing index whose segment boundaries are `bounds` (a list of ints: bounds[g] = first
+    position with index g).  The backward is one reduction per segment (a slice each); the plain gather's backward adds every row into
     the few rows of src with atomics, which serialises when thousands of rows share one, and torch.segment_reduce gives a
     segment to a single thread."""
 
     @staticmethod
-    def forward(ctx, src, index, offsets):
-        ctx.bounds = [int(v) for v in offsets.tolist()]
+    def forward(ctx, src, index, bounds):
+        ctx.bounds = bounds  # python ints, read from the device once per index tensor by the caller
         return src.index_select(0, index)
 
     @staticmethod
@@ -86,12 +86,23 @@ def get_symmetric_displacement(positions, unit_shifts, cell, edge_index, num_gra
         positions = positions + (positions.unsqueeze(-1) * symmetric[0].unsqueeze(0)).sum(dim=1)
         shifts = (unit_shifts.to(cell.dtype).unsqueeze(-1) * cell[0].unsqueeze(0)).sum(dim=1)
     else:
-        graphs = torch.arange(num_graphs + 1, device=batch.device, dtype=batch.dtype)
-        edge_graph = batch[sender]
-        sorted_lists = bool((batch[1:] >= batch[:-1]).all()) and bool((edge_graph[1:] >= edge_graph[:-1]).all())
+        # what depends on the lists alone (the graph of every edge, whether atoms and edges come graph by graph, and where
+        # the graphs' segments begin) is read from the device once per pair of tensors, not per step: a steady-state
+        # evaluation then has no host synchronisation here
+        def segments():
+            graphs = torch.arange(num_graphs + 1, device=batch.device, dtype=batch.dtype)
+            edge_graph = batch[sender]
+            sorted_lists = bool((batch[1:] >= batch[:-1]).all()) and bool((edge_graph[1:] >= edge_graph[:-1]).all())
+            if not sorted_lists:
+                return edge_graph, False, None, None
+            return (edge_graph, True, [int(v) for v in torch.searchsorted(batch, graphs).tolist()],
+                    [int(v) for v in torch.searchsorted(edge_graph, graphs).tolist()])
+
+        edge_graph, sorted_lists, atom_bounds, edge_bounds = _cached_for(edge_index, "_cm_strain_segments_%d" % num_graphs, batch,
+                                                                          segments)
         if sorted_lists:  # atoms and edges graph by graph, as every collated batch has them
-            per_atom = _RowsOfSortedIndex.apply(symmetric, batch, torch.searchsorted(batch, graphs))
-            per_edge = _RowsOfSortedIndex.apply(cell, edge_graph, torch.searchsorted(edge_graph, graphs))
+            per_atom = _RowsOfSortedIndex.apply(symmetric, batch, atom_bounds)
+            per_edge = _RowsOfSortedIndex.apply(cell, edge_graph, edge_bounds)
         else:
             per_atom, per_edge = symmetric[batch], cell[edge_graph]
         positions = positions + torch.einsum("be,bec->bc", positions, per_atom)
