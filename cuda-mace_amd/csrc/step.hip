@@ -104,12 +104,12 @@ __global__ void weight_rows_kernel(float *__restrict__ x, const double *__restri
 
 // Edge range of every receiver node cut back to its last edge inside the cutoff: live[n] = first_occ[n],
 // live[nnodes + n] = one past the last edge e of the node with |vec[e]| <= r_max (the node's first edge if there is
-// none).  The forward message passing skips the edges behind it, which contribute exact zeros (the backward keeps the
-// full range: it writes the zero gradients of those edges).  A Verlet list holds a third more pairs than the cutoff
+// none).  The message-passing kernels, forward and backward, skip the edges behind it: they contribute exact zeros to the
+// forward, and their vector gradients, exact zeros as well, are written by this kernel.  A Verlet list holds a third more pairs than the cutoff
 // takes in; the model orders each node's pairs with those of the skin shell last, nearest first, so that most of them
 // fall behind this mark.  The length is the one the message-passing kernels compute from the same fp32 vector.
 __global__ void live_range_kernel(const int32_t *__restrict__ first_occ, const float *__restrict__ vec, float r_max, int nnodes,
-                                  int64_t nedges, int32_t *__restrict__ live) {
+                                  int64_t nedges, int32_t *__restrict__ live, float *__restrict__ gv1, float *__restrict__ gv2) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= nnodes) return;
   int e0 = first_occ[n], e1 = first_occ[nnodes + n];
@@ -118,6 +118,9 @@ __global__ void live_range_kernel(const int32_t *__restrict__ first_occ, const f
   while (e > e0) {
     const int64_t q = e - 1;
     if (mp::edge_length(vec[3 * q + 0], vec[3 * q + 1], vec[3 * q + 2]) <= r_max) break;
+    // an edge behind the mark: the backward edge passes skip it as well, so its vector gradients are cleared here
+    gv1[3 * q + 0] = gv1[3 * q + 1] = gv1[3 * q + 2] = 0.f;
+    gv2[3 * q + 0] = gv2[3 * q + 1] = gv2[3 * q + 2] = 0.f;
     --e;
   }
   live[n] = e0;
@@ -356,9 +359,9 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
     if (rc_ != CM_OK) return rc_;
     if (E > 0)
       hipLaunchKernelGGL(cm::live_range_kernel, dim3(static_cast<unsigned>(cm::ceil_div(N, 256))), dim3(256), 0, st, g->first_occ,
-                         L.vec, w->r_max, static_cast<int>(N), E, L.live);
+                         L.vec, w->r_max, static_cast<int>(N), E, L.live, L.gv1, L.gv2);
   }
-  const int32_t *fo_forward = E > 0 ? L.live : g->first_occ;
+  const int32_t *fo_live = E > 0 ? L.live : g->first_occ;
   const float *X[2] = {g->X1, L.X2};
   float *bufM[2] = {L.bufM1, L.bufM2};
   float *B[2] = {L.B1, L.B2};
@@ -373,7 +376,7 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
       CM_STAGE(5, cm_linear(L.h1, w->skip_WT, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, w->skip_scale, none, none, L.sc, stream));
       CM_STAGE(6, cm_linear(L.h1, w->up_WT, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, none, L.X2, stream));
     }
-    CM_STAGE(t == 0 ? 1 : 7, cm_mp_edge_forward(X[t], L.vec, w->r_knots, w->spline[t], w->nknots, w->r_width, w->r_max, g->sender, fo_forward, N,
+    CM_STAGE(t == 0 ? 1 : 7, cm_mp_edge_forward(X[t], L.vec, w->r_knots, w->spline[t], w->nknots, w->r_width, w->r_max, g->sender, fo_live, N,
                                E, C, bufM[t], stream));
     if (t == 0)
       CM_STAGE(2, cm_linear(bufM[t], w->mix_WT[t], oh_perm, oh_off, N, ne + 1, 1, 16, C, C, w->mix_scale[t], none, none, L.bufA, stream));
@@ -414,7 +417,7 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   CM_STAGE(14, cm_linear(L.d_h2, w->prod_W[1], nullptr, nullptr, N, 1, 0, 1, C, C, -1.0f, none, none, L.gB, stream));
   CM_STAGE(15, cm_linear(L.bufM2, w->mix_W[1], nullptr, nullptr, N, 1, 0, 16, C, C, w->mix_scale[1], L.gB, none, L.bufA, stream));
   CM_STAGE(16, cm_mp_edge_backward(L.X2, L.vec, w->r_knots, w->spline[1], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
-                              g->first_occ, g->sender_perm, g->sender_offsets, N, E, C, L.gX2, L.gv2, L.edge_scratch, stream));
+                              fo_live, g->sender_perm, g->sender_offsets, N, E, C, L.gX2, L.gv2, L.edge_scratch, stream));
   // layer 0 (first interaction): its input features depend on the species alone, so no gradient with respect to them
   if (glue) {
     CM_STAGE(17, cm::node_glue_backward_with_energy_sums(L.gX2, L.d_h2, w->up_W, w->skip_W, w->prod_W[0], w->w1, w->scale, g->node_weights,
@@ -428,7 +431,7 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   CM_STAGE(20, cm_linear(L.bufM1, w->mix_W[0], oh_perm, oh_off, N, ne + 1, 1, 16, C, C, w->mix_scale[0], L.gB, none, L.bufA, stream));
   // its vector gradient is written onto the second layer's: gv1 = (this layer's) + gv2
   CM_STAGE(21, cm::mp::edge_backward_onto(g->X1, L.vec, w->r_knots, w->spline[0], w->nknots, w->r_width, w->r_max, L.bufA, g->sender,
-                                         g->first_occ, N, E, C, L.gv1, L.gv2, st));
+                                         fo_live, N, E, C, L.gv1, L.gv2, st));
   CM_STAGE(23, cm_edge_geometry_backward(positions, g->receiver, g->sender, shifts, g->node_rows, g->first_occ, g->sender_perm,
                                     g->sender_offsets, L.gv1, nullptr, N, E, forces, nullptr, stream));
   if (virials) {

@@ -64,6 +64,8 @@ SIGNATURES = {
     "cm_symcon_backward": (_i32, [_p, _p, _i64, _i32, _p, _p]),
     "cm_readout_forward": (_i32, [_p] * 5 + [_f64, _f64, _f64, _i64, _i32, _i32, _p, _p, _p, _p, _p]),
     "cm_readout_backward": (_i32, [_p, _p, _p, _f64, _i64, _i32, _p, _p, _p]),
+    "cm_graph_prepare_workspace": (_sz, [_i64, _i64, _i32, _i32]),
+    "cm_graph_prepare": (_i32, [_p] * 5 + [_i64, _i64, _i32, _f64, _i32] + [_p] * 10 + [_sz, _p]),
     "cm_node_glue_supported": (_i32, [_i32]),
     "cm_node_glue_forward": (_i32, [_p] * 6 + [_i64, _i32, _i32, _f32, _p, _p, _p, _p]),
     "cm_node_glue_backward": (_i32, [_p] * 6 + [_f64, _p, _p, _p, _i64, _i32, _i32, _f32, _p, _p]),
@@ -192,6 +194,30 @@ def stable_key_sort_static(keys: torch.Tensor, nkeys: int, perm: torch.Tensor, o
             _dev(keys, I32, "keys"), n, nkeys, _dev(perm, I32, "perm"), _dev(offsets, I32, "offsets"), _stream()
         )
     )
+
+
+def graph_prepare(positions: torch.Tensor, row_i: torch.Tensor, row_j: torch.Tensor, shifts: torch.Tensor,
+                  graph_of_node: Optional[torch.Tensor], ngraphs: int, r_max: float, bins: int) -> dict:
+    """cm_graph_prepare: the spatially ordered, shell-last copy of a neighbour list with its CSR offsets and its view sorted
+    by sender, in one call without a host synchronisation.  Returns a dict of int32 tensors (node_perm, node_inverse,
+    receiver, sender, edge_perm, first_occ, sender_perm, sender_offsets) and shifts (fp64 [E, 3], reordered)."""
+    N, E = positions.shape[0], row_i.numel()
+    dev = positions.device
+    i32 = lambda n: torch.empty(n, dtype=I32, device=dev)  # noqa: E731
+    out = {"node_perm": i32(N), "node_inverse": i32(N), "receiver": i32(E), "sender": i32(E), "edge_perm": i32(E),
+           "shifts": torch.empty(E, 3, dtype=F64, device=dev), "first_occ": i32(2 * N), "sender_perm": i32(E),
+           "sender_offsets": i32(N + 1)}
+    need = lib.cm_graph_prepare_workspace(N, E, int(ngraphs), int(bins))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+    _check(lib.cm_graph_prepare(
+        _dev(positions, F64, "positions"), _dev(row_i, I32, "row_i"), _dev(row_j, I32, "row_j"), _dev(shifts, F64, "shifts"),
+        _dev(graph_of_node, I32, "graph_of_node"), N, E, int(ngraphs), float(r_max), int(bins),
+        _dev(out["node_perm"], I32, "node_perm"), _dev(out["node_inverse"], I32, "node_inverse"),
+        _dev(out["receiver"], I32, "receiver"), _dev(out["sender"], I32, "sender"), _dev(out["edge_perm"], I32, "edge_perm"),
+        _dev(out["shifts"], F64, "shifts_out"), _dev(out["first_occ"], I32, "first_occ"),
+        _dev(out["sender_perm"], I32, "sender_perm"), _dev(out["sender_offsets"], I32, "sender_offsets"),
+        ws.data_ptr(), ws.numel(), _stream()))
+    return out
 
 
 # ---- message passing --------------------------------------------------------------------------

@@ -84,7 +84,7 @@ class DeviceCalculator:
         if self._graph is not None:
             return self._graph(positions)
         data = dict(self._data)
-        data["positions"] = positions.clone()
+        data["positions"] = positions.detach()  # an alias: the model marks its own handle as differentiable, not the caller's
         out = self.model(data, compute_virials=self.compute_stress, compute_stress=self.compute_stress)
         return {k: v.detach() for k, v in out.items() if isinstance(v, torch.Tensor)}
 

@@ -473,47 +473,38 @@ class OptimizedInvariantMACE(torch.nn.Module):
         return g("mono3"), g("mono2"), g("T3"), g("T2"), g("T1"), self._contraction_builtin[i]
 
     def _spatial_order(self, data: Dict[str, torch.Tensor]):
-        """Relabelling of one neighbour list: atoms sorted by (graph, 3-D bin of half the cutoff, lexicographic), edges
-        re-sorted by the new row-0 label and, inside a row-0 segment, by the row-1 label with the pairs beyond the cutoff
-        last.  Returns (perm new -> old [N], inverse [N], edge_perm new -> old [E],
-        relabelled edge_index [2, E], relabelled batch [N]).  Any permutation is valid; this one is cheap and keeps
+        """Relabelling of one neighbour list: atoms sorted by (graph, cell of a 3-D grid of at least half the cutoff,
+        original index), edges re-sorted by the new row-0 label and, inside a row-0 segment, by the row-1 label with the
+        pairs beyond the cutoff (the skin shell of a Verlet list) last, nearest first: the native step cuts every segment
+        back to its last pair inside the cutoff, and with this order the pairs that drift inside between two list builds
+        are the first of the shell, so the cut stays close to the pairs that count.  One library call on the device
+        (cm_graph_prepare), no host synchronisation; it also delivers the CSR offsets and the sender-sorted view of the new
+        list, which are left where the ops look for them.  Returns (perm new -> old [N], inverse [N], edge_perm new -> old
+        [E], relabelled edge_index [2, E], relabelled batch [N]).  Any permutation is valid; this one is cheap and keeps
         neighbours within a few hundred indices of each other."""
-        pos = data["positions"].detach()
+        pos = data["positions"].detach().double().contiguous()
         batch, edge_index = data["batch"], data["edge_index"]
-        n = pos.shape[0]
-        bins = torch.floor((pos - pos.min(dim=0).values) / (0.5 * float(self.r_max))).long()
-        bins.clamp_(max=(1 << 16) - 1)  # 48 bits for the bin, the rest for the graph index: the key cannot overflow
-        nb = int(bins.max()) + 1
-        key = ((batch * nb + bins[:, 0]) * nb + bins[:, 1]) * nb + bins[:, 2]
-        perm = torch.argsort(key, stable=True)
-        inverse = torch.empty_like(perm)
-        inverse[perm] = torch.arange(n, device=perm.device)
-        row0, row1 = inverse[edge_index[0]], inverse[edge_index[1]]
-        # Inside a row-0 segment: the pairs within the cutoff by their row-1 label, then those beyond it (the skin shell
-        # of a Verlet list), nearest first.  The native step cuts every segment back to its last pair inside the cutoff
-        # before the forward message passing; with this order the pairs that drift inside between two list builds are
-        # the first of the shell, so the cut stays close to the pairs that count.  Three stable sorts, least significant
-        # key first: by length among the shell pairs, by row-1 label among the others, by segment; the two with node
-        # labels as keys are counting sorts of the library (on the device, where the model runs).
-        def by_label(keys, nkeys):
-            if keys.is_cuda and nkeys < 2**31 - 1:
-                return cabi.stable_key_sort(keys.int().contiguous(), nkeys)[0].long()
-            return torch.argsort(keys, stable=True)
-
-        if "shifts" in data:
-            length = (pos[edge_index[1]] - pos[edge_index[0]] + data["shifts"].detach().to(pos.dtype)).norm(dim=1)
-            shell = length > float(self.r_max)
-            by_length = torch.argsort(torch.where(shell, length, torch.zeros_like(length)).float(), stable=True)  # the rest stays put
-            # by_length holds the pairs within the cutoff first, in the list's order: only those are sorted by label
-            # (as one key the shell would be a single bucket of a quarter of all pairs, which a counting sort ranks serially)
-            n_within = edge_index.shape[1] - int(shell.sum())
-            within, beyond = by_length[:n_within], by_length[n_within:]
-            by_inner = torch.cat((within[by_label(row1[within], n)], beyond))
-            edge_perm = by_inner[by_label(row0[by_inner], n)]
-        else:
-            edge_perm = torch.argsort(row0 * n + row1, stable=True)
-        new_edges = torch.stack((row0[edge_perm], row1[edge_perm])).contiguous()
-        return perm, inverse, edge_perm, new_edges, batch[perm].contiguous()
+        n, ngraphs = pos.shape[0], int(data["ptr"].numel()) - 1
+        row0, row1 = _cached(edge_index, "_cm_int32_rows", None,
+                             lambda: (edge_index[0].int().contiguous(), edge_index[1].int().contiguous()))
+        shifts = data["shifts"].detach().double().contiguous()
+        # cells per axis from the size alone (a host constant): enough for cells of half a cutoff at 0.05 atoms / A^3
+        bins = int(min(64, max(1, np.ceil((n / max(ngraphs, 1) / 0.05) ** (1.0 / 3.0) / (0.5 * float(self.r_max))))))
+        while ngraphs * bins ** 3 >= 2 ** 24:
+            bins -= 1
+        g = cabi.graph_prepare(pos, row0, row1, shifts, None if ngraphs == 1 else batch.int().contiguous(), ngraphs,
+                               float(self.r_max), bins)
+        perm, inverse, edge_perm = g["node_perm"].long(), g["node_inverse"].long(), g["edge_perm"].long()
+        receiver, sender = g["receiver"], g["sender"]
+        new_edges = torch.stack((receiver, sender)).long()
+        # what the ops derive from a list is already there: leave it where they look it up
+        new_edges.__dict__["_cm_int32_rows"] = ((new_edges._version, new_edges.data_ptr(), None), (receiver, sender))
+        receiver.__dict__["_cm_csr"] = ((receiver._version, receiver.data_ptr(), n), g["first_occ"])
+        sender.__dict__["_cm_sender_view"] = ((sender._version, sender.data_ptr(), n), (g["sender_perm"], g["sender_offsets"]))
+        if data["shifts"].dtype == torch.float64:
+            t = data["shifts"]
+            edge_index.__dict__["_cm_spatial_shifts"] = (t, (edge_index._version, edge_index.data_ptr(), t._version), g["shifts"])
+        return perm, inverse, edge_perm, new_edges, batch.index_select(0, perm)
 
     def forward(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
                 compute_virials: bool = False, compute_stress: bool = False,

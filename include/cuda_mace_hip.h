@@ -416,6 +416,31 @@ int cm_readout_backward(const double *grad_node_energies, const double *w1, cons
                         int64_t nnodes, int channels, float *grad_h1, float *grad_h2, cm_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Index structures of one neighbour list in one call, without a host synchronisation (no counterpart in the reference,
+ * which takes the list as upstream's host-side search returns it, tests/test_utils.py:62-105, and builds its N x N
+ * reverse-edge table inside every forward call, jit_wrappers/src/invariant_message_passing_wrapper.cpp:91-93).
+ *   in:  positions fp64 [nnodes, 3]; the list row_i (non-decreasing, in [0, nnodes)), row_j int32 [nedges] with
+ *        shifts fp64 [nedges, 3] (vector of a pair = positions[row_j] - positions[row_i] + shift);
+ *        graph_of_node int32 [nnodes] (non-decreasing) or NULL for one graph; r_max: the model's cutoff;
+ *        bins: cells per axis of the grid the atoms are ordered by (1 .. 64; ngraphs * bins^3 < 2^24; cells are at
+ *        least r_max / 2 wide and cover the bounding box of the positions)
+ *   out: node_perm [nnodes]: atom a of the new order is atom node_perm[a] of the caller (atoms sorted by graph, grid
+ *        cell, original index); node_inverse [nnodes] its inverse;
+ *        receiver / sender int32 [nedges]: the list in the new labels, sorted by receiver (= new label of row_i); inside a
+ *        receiver's segment the pairs within r_max by sender label, then the others by length; ties keep the list's order;
+ *        edge_perm [nedges]: pair e of the new list is pair edge_perm[e] of the caller's; shifts_out fp64 [nedges, 3];
+ *        first_occ [2 nnodes] = cm_first_occurences(receiver);
+ *        sender_perm [nedges], sender_offsets [nnodes + 1] = cm_stable_key_sort(sender, nedges, nnodes).
+ *   workspace: cm_graph_prepare_workspace(nnodes, nedges, ngraphs, bins) bytes, 256-byte aligned.
+ * Every output is a function of the inputs alone (fixed orders throughout): the same list gives the same bits. */
+size_t cm_graph_prepare_workspace(int64_t nnodes, int64_t nedges, int ngraphs, int bins);
+int cm_graph_prepare(const double *positions, const int32_t *row_i, const int32_t *row_j, const double *shifts,
+                     const int32_t *graph_of_node, int64_t nnodes, int64_t nedges, int ngraphs, double r_max, int bins,
+                     int32_t *node_perm, int32_t *node_inverse, int32_t *receiver, int32_t *sender, int32_t *edge_perm,
+                     double *shifts_out, int32_t *first_occ, int32_t *sender_perm, int32_t *sender_offsets, void *workspace,
+                     size_t workspace_bytes, cm_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * The three [nnodes, C] x [C, C] linears between the two interaction layers as one launch per direction: the product's
  * linear and linear_up (the reference's linear_matmul, models/InvariantMACE.py:41-53) and the per-element skip
  * connection between them (element_linear_to_cuda, :56-74; called at :145-150 and :330).  A workgroup takes 128 nodes

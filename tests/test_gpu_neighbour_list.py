@@ -127,3 +127,54 @@ def test_max_displacement(cabi, n):
     if n:
         pos[n // 2, 1] = float("nan")
         assert float(cabi.max_displacement(pos, ref, out=got)[0]) == float("inf")
+
+
+@pytest.mark.parametrize("case", ["periodic_skin", "batch", "exact_list", "cluster", "no_edges", "headline"])
+def test_graph_prepare_matches_the_host_restatement(cabi, case):
+    """cm_graph_prepare (relabelled atoms, re-sorted pairs with the skin shell last, CSR offsets, sender-sorted view) entry
+    for entry against a numpy restatement with library sorts, and its derived structures against the index oracles."""
+    from cuda_mace.utils.synthetic import collate, make_system
+    from oracle import ops as O
+    from tests.util import spatial_order_reference
+
+    r_max = 5.0
+    if case == "periodic_skin":
+        data = make_system(400, 4, seed=5, density=0.1, cutoff=5.6)
+    elif case == "batch":
+        data = collate([make_system(n, 4, seed=20 + k, density=0.1, cutoff=5.2) for k, n in enumerate((150, 230, 120))])
+    elif case == "exact_list":
+        data = make_system(300, 4, seed=6, density=0.1)
+    elif case == "cluster":
+        data = make_system(21, 4, seed=0, density=None, cluster_box=8.0)
+    elif case == "no_edges":
+        data = make_system(12, 4, seed=2, density=None, cluster_box=60.0, min_dist=8.0)
+        assert data["edge_index"].shape[1] == 0
+    else:
+        data = make_system(25000, 10, seed=0, density=0.1, cutoff=5.5)
+    N, E = data["positions"].shape[0], data["edge_index"].shape[1]
+    ngraphs = int(data["ptr"].numel()) - 1
+    print("graph_prepare", case, N, E, ngraphs, flush=True)
+    dev = lambda t: t.to("cuda").contiguous()  # noqa: E731
+    bins = 64 if ngraphs == 1 else 16
+    got = cabi.graph_prepare(dev(data["positions"].double()), dev(data["edge_index"][0].int()), dev(data["edge_index"][1].int()),
+                             dev(data["shifts"].double()), None if ngraphs == 1 else dev(data["batch"].int()), ngraphs, r_max, bins)
+    perm, inverse, rcv, snd, order = spatial_order_reference(data["positions"], data["batch"], data["edge_index"], data["shifts"],
+                                                             r_max, bins)
+    eq = lambda name, want: np.testing.assert_array_equal(got[name].cpu().numpy(), want, err_msg=name)  # noqa: E731
+    eq("node_perm", perm)
+    eq("node_inverse", inverse)
+    eq("receiver", rcv)
+    eq("sender", snd)
+    eq("edge_perm", order)
+    assert torch.equal(got["shifts"].cpu(), data["shifts"].double()[torch.from_numpy(order)])
+    assert torch.equal(got["first_occ"].cpu(), O.first_occurences(torch.from_numpy(rcv).int(), N))
+    sperm, soff = O.stable_key_sort(torch.from_numpy(snd).int(), N)
+    assert torch.equal(got["sender_perm"].cpu(), sperm) and torch.equal(got["sender_offsets"].cpu(), soff)
+    if E:
+        # every receiver's pairs beyond the cutoff come last
+        v = data["positions"][data["edge_index"][1]] - data["positions"][data["edge_index"][0]] + data["shifts"]
+        beyond = (v.norm(dim=1) > r_max)[torch.from_numpy(order)]
+        fo = got["first_occ"].cpu()
+        for n in (0, N // 2, N - 1):
+            seg = beyond[fo[n]:fo[N + n]]
+            assert bool((seg[1:] >= seg[:-1]).all())

@@ -110,3 +110,30 @@ try:
         forward = _oracle_forward
 except ImportError:  # the package needs its built library; tests that use this class fail loudly on their own
     OracleBackedMACE = None
+
+
+def spatial_order_reference(positions, batch, edge_index, shifts, r_max, bins=64):
+    """Host restatement (numpy, library sorts) of the relabelling that cm_graph_prepare performs on the device:
+    (perm new -> old, inverse, receiver, sender, edge_perm new -> old) with atoms sorted by (graph, grid cell, index) and
+    every receiver's pairs ordered by (beyond the cutoff?, sender label | length, position in the list)."""
+    import numpy as np
+
+    pos = positions.double().cpu().numpy()
+    ei = edge_index.cpu().numpy()
+    sh = shifts.double().cpu().numpy()
+    n = pos.shape[0]
+    lo = pos.min(axis=0) if n else np.zeros(3)
+    extent = float((pos.max(axis=0) - lo).max()) if n else 0.0
+    width = max(extent / bins * (1.0 + 1e-12), 0.5 * r_max)
+    b = np.clip(np.floor((pos - lo) / width), 0, bins - 1).astype(np.int64)
+    key = ((batch.cpu().numpy().astype(np.int64) * bins + b[:, 0]) * bins + b[:, 1]) * bins + b[:, 2]
+    perm = np.argsort(key, kind="stable")
+    inverse = np.empty(n, dtype=np.int64)
+    inverse[perm] = np.arange(n)
+    v = (pos[ei[1]] - pos[ei[0]]) + sh
+    length = np.sqrt((v[:, 0] * v[:, 0] + v[:, 1] * v[:, 1]) + v[:, 2] * v[:, 2])
+    shell = length > r_max
+    row0, row1 = inverse[ei[0]], inverse[ei[1]]
+    second = np.where(shell, length, row1.astype(np.float64))  # labels are exact in fp64
+    order = np.lexsort((np.arange(ei.shape[1]), second, shell, row0))  # last key is the most significant
+    return perm, inverse, row0[order], row1[order], order
