@@ -36,6 +36,47 @@ constexpr int kTileNodes = 32 * kWaves;  // rows per workgroup (MFMA M = 32 per 
 constexpr int kKC = 32;                  // K columns staged per step
 constexpr int kLdH = kKC + 8;            // padded LDS row stride of a bf16 plane (elements; 80 bytes: conflict-free b128 reads)
 
+// A wave's 32 x (32 NT) block of accumulators to memory, four bytes per lane and store (a store instruction covers two
+// rows of 128 bytes): OUT = acc * scale (+ residual).  The residual may be OUT itself, so the compiler cannot move a
+// load of it across a store: all of a lane's residual values are read before its first store (every element is read
+// and written by the same lane), instead of one dependent load per store.  The product is rounded before the residual is
+// added, as in the kernels that stage it in LDS.
+template <int NT>
+__device__ __forceinline__ void store_block(const v16f (&acc)[NT], const int *sNode, int wave, int half, int mrow, int ncomp, int m,
+                                            int row_stride, int col0, float scale, const float *residual, float *OUT) {
+  if (residual) {
+    float res[16][NT];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int node = sNode[32 * wave + 8 * (r / 4) + 4 * half + (r % 4)];
+      const float *rp = residual + (static_cast<int64_t>(node >= 0 ? node : 0) * ncomp + m) * row_stride + col0 + mrow;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) res[r][t] = node >= 0 ? rp[32 * t] : 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int node = sNode[32 * wave + 8 * (r / 4) + 4 * half + (r % 4)];
+      if (node < 0) continue;
+      float *op = OUT + (static_cast<int64_t>(node) * ncomp + m) * row_stride + col0 + mrow;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma clang fp contract(off)
+        const float v = acc[t][r] * scale;
+        op[32 * t] = v + res[r][t];
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int node = sNode[32 * wave + 8 * (r / 4) + 4 * half + (r % 4)];
+    if (node < 0) continue;
+    float *op = OUT + (static_cast<int64_t>(node) * ncomp + m) * row_stride + col0 + mrow;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
+  }
+}
+
 // A workgroup computes 32 * NT output columns, starting at column blockIdx.y * 32 * NT of the nout_total columns of a row
 // (one workgroup per tile for all columns where there are many tiles; few tiles are spread over more workgroups, 32
 // columns each, which shortens the chain of staging and matrix instructions a tile waits for: every output element sums
@@ -181,27 +222,7 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
   }
 
   // accumulator r of a lane is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of the wave's 32x32 block
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
-    const int node = sNode[row];
-    if (node >= 0) {
-      const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * nout_total + col0 + mrow;
-      float *op = OUT + at;
-      if (residual) {  // may be OUT itself: every element is read and written by the same lane
-        const float *rp = residual + at;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-#pragma clang fp contract(off)  // the product is rounded before the residual is added, as in the kernels that stage it in LDS
-          const float v = acc[t][r] * scale;
-          op[32 * t] = v + rp[32 * t];
-        }
-      } else {
-#pragma unroll
-        for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
-      }
-    }
-  }
+  store_block<NT>(acc, sNode, wave, half, mrow, ncomp, m, nout_total, col0, scale, residual, OUT);
 }
 
 // -----------------------------------------------------------------------------------------------
@@ -451,27 +472,7 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
       }
     }
   } else {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = 32 * wave + 8 * (r / 4) + 4 * half + (r % 4);
-      const int node = sNode[row];
-      if (node >= 0) {
-        const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * NOUT + mrow;
-        float *op = OUT + at;
-        if (residual) {  // may be OUT itself: every element is read and written by the same lane
-          const float *rp = residual + at;
-#pragma unroll
-          for (int t = 0; t < NT; ++t) {
-#pragma clang fp contract(off)
-            const float v = acc[t][r] * scale;
-            op[32 * t] = v + rp[32 * t];
-          }
-        } else {
-#pragma unroll
-          for (int t = 0; t < NT; ++t) op[32 * t] = acc[t][r] * scale;
-        }
-      }
-    }
+    store_block<NT>(acc, sNode, wave, half, mrow, ncomp, m, NOUT, 0, scale, residual, OUT);
   }
 }
 
