@@ -56,6 +56,21 @@ inline int check_launch(const char *what) {
 // l(m) = floor(sqrt(m)) for m in 0..15 without a sqrt.
 __device__ __forceinline__ constexpr int l_of_m(int m) { return m == 0 ? 0 : (m < 4 ? 1 : (m < 9 ? 2 : 3)); }
 
+// The vector of edge e in fp64: pos[b[e]] - pos[a[e]] + shift[e], atom n being row rows[n] of pos when a row map is given;
+// zero when either index lies outside the node range.  The one definition every kernel that forms an edge vector uses,
+// so that all of them arrive at the same bits.
+__device__ __forceinline__ void edge_vector_f64(const double *__restrict__ pos, const int32_t *__restrict__ a,
+                                                const int32_t *__restrict__ b, const double *__restrict__ shifts,
+                                                const int32_t *__restrict__ rows, int64_t e, int nnodes, double (&v)[3]) {
+  const int ia = a[e], ib = b[e];
+  v[0] = v[1] = v[2] = 0.0;
+  if (static_cast<unsigned>(ia) < static_cast<unsigned>(nnodes) && static_cast<unsigned>(ib) < static_cast<unsigned>(nnodes)) {
+    const int ra = rows ? rows[ia] : ia, rb = rows ? rows[ib] : ib;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) v[k] = pos[3 * rb + k] - pos[3 * ra + k] + shifts[3 * e + k];
+  }
+}
+
 // Edge range [e0, e1) of a node as read from caller-provided CSR offsets, forced into [0, nedges] with e0 <= e1: offsets
 // derived from an unsorted or out-of-range receiver list then name a wrong but addressable range instead of memory
 // outside the edge arrays.

@@ -23,13 +23,8 @@ __global__ void edge_geometry_forward_kernel(const double *__restrict__ pos, con
                                              float *__restrict__ vec, float *__restrict__ len) {
   const int64_t e = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
   if (e >= nedges) return;
-  const int ia = a[e], ib = b[e];
-  double v[3] = {0.0, 0.0, 0.0};
-  if (static_cast<unsigned>(ia) < static_cast<unsigned>(nnodes) && static_cast<unsigned>(ib) < static_cast<unsigned>(nnodes)) {
-    const int ra = row_of(rows, ia), rb = row_of(rows, ib);
-#pragma unroll
-    for (int k = 0; k < 3; ++k) v[k] = pos[3 * rb + k] - pos[3 * ra + k] + shifts[3 * e + k];
-  }
+  double v[3];
+  edge_vector_f64(pos, a, b, shifts, rows, e, nnodes, v);
   vec[3 * e + 0] = static_cast<float>(v[0]);
   vec[3 * e + 1] = static_cast<float>(v[1]);
   vec[3 * e + 2] = static_cast<float>(v[2]);

@@ -263,7 +263,10 @@ __device__ __forceinline__ void dma16(const float *src, unsigned lds_byte_addres
 __device__ __forceinline__ void ldg16(f4 &dst, const float *src) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(src) : "memory");
 }
-__device__ __forceinline__ void after_wait(f4 &v) { asm volatile("" : "+v"(v)); }
+// Marks the point from which a register that a hand-issued load lands in holds the loaded value (the wait that covers the
+// load precedes it): no use can move above it, and the build's scan of the generated code, which refuses any instruction
+// that touches such a register between the load's issue and this mark, reads the comment it leaves in the assembly.
+__device__ __forceinline__ void after_wait(f4 &v) { asm volatile("; landed %0" : "+v"(v)); }
 
 // two workgroups per compute unit (two waves per SIMD) wherever LDS allows it: 256 registers per lane
 template <int NT, bool SCALED>
@@ -364,27 +367,36 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
     }
   };
 
-  const int nch = K / kKC;
-  issue_w(0, std::integral_constant<int, 0>{});
-  issue_x(0, 0);
-  if (nch > 1) issue_x(kKC, 1);
-
-  auto iteration = [&](int c, int stage, auto par) {
+  // What the next iteration consumes has landed when an iteration (or the prologue) ends: the wait sits at the end of
+  // the code that issued the loads, so that every register a load was issued into passes through after_wait before
+  // the loop's back edge (a copy the compiler makes there then copies the loaded value).
+  auto landed = [&](auto par) {
     constexpr int P = decltype(par)::value;
-    const int kc = c * kKC;
-    // every wave has finished multiplying chunk c - 1: the weight planes and ring stage (c + 2) % 3 are free
-    asm volatile("s_barrier" ::: "memory");
-    // weights (and scales) of chunk c and X chunk c have landed; the four loads of X chunk c + 1 may still be out
-    if (c + 1 < nch)
-      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
     for (int i = 0; i < NT; ++i) after_wait(pb[i]);
     if constexpr (SCALED) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) after_wait(sc[P][q]);
     }
+  };
+  const int nch = K / kKC;
+  issue_w(0, std::integral_constant<int, 0>{});
+  issue_x(0, 0);
+  if (nch > 1) {
+    issue_x(kKC, 1);
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");  // all but the four loads of X chunk 1
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+  landed(std::integral_constant<int, 0>{});
+
+  auto iteration = [&](int c, int stage, auto par) {
+    constexpr int P = decltype(par)::value;
+    const int kc = c * kKC;
+    // every wave has finished multiplying chunk c - 1: the weight planes and ring stage (c + 2) % 3 are free.  Weights
+    // (and scales) of chunk c and X chunk c have landed (waited for where they were issued); the four loads of X chunk
+    // c + 1 may still be out
+    asm volatile("s_barrier" ::: "memory");
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
       bf16x4 h, md, lw;
@@ -433,6 +445,14 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
 #pragma unroll
       for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[t][0], acc[t], 0, 0, 0);
     }
+    // the next chunk's weights, scales and X rows: everything but the four loads of the X chunk after it, if one was issued
+    if (c + 1 < nch) {
+      if (c + 2 < nch)
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    landed(std::integral_constant<int, 1 - P>{});
   };
   int stage = 0;
   for (int c = 0; c < nch; c += 2) {
@@ -442,6 +462,9 @@ __global__ __launch_bounds__(kWaves *kWave, (NT <= 4 ? 2 : 1)) void linear_ring_
     iteration(c + 1, stage, std::integral_constant<int, 1>{});
     stage = stage == 2 ? 0 : stage + 1;
   }
+  // Nothing is in flight here (the last chunk waited for everything and issued nothing); said once more in a form that
+  // the build's scan of the generated code, which does not know that the loop issues only while it goes on, can read.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
   if constexpr (NT <= 4) {
     // Output through LDS, so that rows leave as 16-byte stores (a lane's accumulators are one column of 16 rows: stored
@@ -701,10 +724,10 @@ __global__ __launch_bounds__(kResWaves *kWave, 1) void linear_resident_kernel(
 #pragma unroll
           for (int ln = 0; ln < kLines; ++ln) {
             const int j = (c * 4 + rg) * kLines + ln;
-            asm volatile("" : "+a"(land[j]));
+            asm volatile("; landed %0" : "+a"(land[j]));
             f4 v = land[j];
             if constexpr (SCALED) {
-              asm volatile("" : "+a"(sland[j]));
+              asm volatile("; landed %0" : "+a"(sland[j]));
               v *= sland[j];
             }
             *reinterpret_cast<f4 *>(stg + (8 * rg + orow) * kTLd + 32 * ln + 4 * opiece) = v;

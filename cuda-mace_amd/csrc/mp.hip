@@ -266,10 +266,13 @@ __global__ __launch_bounds__(kWave) void mp_backward_edge_kernel(
 // together and uses what iteration i - 1 issued: one memory latency per iteration instead of three.  Every load is
 // unconditional: an edge that is not to be read (beyond the list's end, beyond the cutoff, out of range) loads the row
 // of the slot's last good edge again, a cache hit, and its value is dropped by a select.  The loads are issued from
-// inline assembly and waited for once per iteration by an explicit wait, with the loaded registers passed through the
-// waiting statement so that no use can move above it: left to itself the compiler sinks each load to its first use in
+// inline assembly and waited for once per iteration by an explicit wait at the end of the iteration that issued them,
+// with the loaded registers passed through the waiting statement so that no use can move above it and every value that
+// crosses the loop's back edge has arrived: left to itself the compiler sinks each load to its first use in
 // the next iteration and waits for it there, which puts the three latencies back in a row.  Registers that are still
-// being loaded are never copied; the batches change roles after the wait.  The summation order is fixed.
+// being loaded are never copied (the build scans the generated code of this kernel for any instruction that touches
+// a register between the load issued into it and the wait); the batches change roles after the wait.  The summation
+// order is fixed.
 __device__ __forceinline__ void issue_load(int &dst, const int32_t *p) {
   asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
 }
@@ -285,13 +288,18 @@ __device__ __forceinline__ void issue_load_stream(float &dst, const float *p) {
 __device__ __forceinline__ void issue_load_stream(f4 &dst, const float *p) {
   asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(p) : "memory");
 }
+// Marks the point from which a register that a hand-issued load lands in holds the loaded value; the comment it leaves
+// in the assembly is read by the build's scan of the generated code (see the head of the sender kernel).
 template <class T>
 __device__ __forceinline__ void arrived(T &v) {
-  asm volatile("" : "+v"(v));
+  asm volatile("; landed %0" : "+v"(v));
 }
 
-template <int C, int LIVE>
-__global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
+//
+// MULTI (few senders, see parts_for): a workgroup of up to eight waves per sender, each on a part of the sender's range;
+// the parts' sums are added by the first wave in the order of the parts.
+template <int C, int LIVE, bool MULTI>
+__global__ __launch_bounds__(MULTI ? 8 * kWave : kWave) void mp_backward_sender_kernel(
     const float *__restrict__ gXe, const int32_t *__restrict__ perm,
     const int32_t *__restrict__ offsets, int nnodes, int64_t nedges, const float *__restrict__ live_by, float r_max,
     float *__restrict__ gX) {
@@ -299,13 +307,22 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
   using vec = typename K::vec;
   constexpr int B = 4;            // edges per slot and iteration
   constexpr int STEP = B * K::EPW;
+  __shared__ __attribute__((aligned(16))) float comb[MULTI ? 7 * C : 1];
   const int node = blockIdx.x;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x % kWave;
+  const int wave = MULTI ? threadIdx.x / kWave : 0;
+  const int parts = MULTI ? blockDim.x / kWave : 1;
   const int slot = lane / K::SW;
   const int cl = lane % K::SW;
   const bool active = cl < K::LPE;
-  const int k0 = offsets[node];
-  const int k1 = offsets[node + 1];
+  int k0 = offsets[node];
+  int k1 = offsets[node + 1];
+  if (MULTI) {
+    const int64_t len = k1 - k0;
+    const int lo = k0 + static_cast<int>(len * wave / parts);
+    k1 = k0 + static_cast<int>(len * (wave + 1) / parts);
+    k0 = lo;
+  }
   vec acc = zerov<vec>();
   if (active && k0 < k1 && nedges > 0) {
     const int klast = k1 - 1;
@@ -368,25 +385,9 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
       return take[j] ? r : zerov<vec>();
     };
 
-    int k = k0 + slot;
-    // prologue: indices of batches 0 and 1, then the vectors of batch 0
-    issue_indices(k, e_cur);
-    issue_indices(k + STEP, e_nxt);
-    wait_all(e_cur[0], e_cur[1], e_cur[2], e_cur[3], e_nxt[0], e_nxt[1], e_nxt[2], e_nxt[3]);
-    issue_live(e_cur);  // lands in lv_nxt / lr_nxt: the loop's first act is to move it to the current set
-    int good = min(max(e_cur[0], 0), emax);  // a row that may always be read
-#pragma unroll
-    for (int j = 0; j < B; ++j) {
-      rows4[j] = zero4();
-#pragma unroll
-      for (int q = 0; q < K::V; ++q) rowsf[j][q] = 0.f;
-      take[j] = false;
-      e_aft[j] = e_nxt[j];
-    }
-    // shift the roles once so that the loop head finds batch 0 in e_nxt / lv_nxt and batch 1 in e_aft
-#pragma unroll
-    for (int j = 0; j < B; ++j) e_nxt[j] = e_cur[j];
-    for (; k < k1; k += STEP) {
+    auto wait_for_everything = [&]() {
+      // One wait for all that is in flight; every register a load was issued into passes through this point, so that
+      // whatever the compiler does with it afterwards (a copy across the loop's back edge included) sees the loaded value.
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       arrived_rows();
 #pragma unroll
@@ -395,6 +396,25 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
         if constexpr (LIVE == 1) arrived(lv_nxt[j]);
         if constexpr (LIVE == 2) arrived(lr_nxt[j]);
       }
+    };
+
+    int k = k0 + slot;
+    // prologue: indices of batches 0 and 1, then the vectors of batch 0
+    issue_indices(k, e_cur);
+    issue_indices(k + STEP, e_aft);
+    wait_all(e_cur[0], e_cur[1], e_cur[2], e_cur[3], e_aft[0], e_aft[1], e_aft[2], e_aft[3]);
+    int good = min(max(e_cur[0], 0), emax);  // a row that may always be read
+#pragma unroll
+    for (int j = 0; j < B; ++j) {
+      rows4[j] = zero4();
+#pragma unroll
+      for (int q = 0; q < K::V; ++q) rowsf[j][q] = 0.f;
+      take[j] = false;
+      e_nxt[j] = e_cur[j];  // the loop head finds batch 0 in e_nxt / lv_nxt and batch 1 in e_aft
+    }
+    issue_live(e_nxt);  // lands in lv_nxt / lr_nxt: the loop's first act is to move it to the current set
+    wait_for_everything();
+    for (; k < k1; k += STEP) {
       // everything has arrived: rows of the previous batch, vectors of this one, indices of the next one
       acc += (row(0) + row(1)) + (row(2) + row(3));
 #pragma unroll
@@ -413,17 +433,23 @@ __global__ __launch_bounds__(kWave) void mp_backward_sender_kernel(
         good = ok ? e_cur[j] : good;
         e_cur[j] = ok ? e_cur[j] : good;
       }
-      // issue: rows of this batch, vectors of the next, indices of the one after
+      // issue: rows of this batch, vectors of the next, indices of the one after; then the iteration's one wait
       issue_rows(e_cur);
       issue_live(e_nxt);
       issue_indices(k + 2 * STEP, e_aft);
+      wait_for_everything();
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    arrived_rows();
     acc += (row(0) + row(1)) + (row(2) + row(3));
   }
 #pragma unroll
   for (int off = kWave / 2; off >= K::SW; off >>= 1) acc += shfl_downv(acc, off);
+  if (MULTI) {
+    if (wave > 0 && slot == 0 && active) K::st(comb + (wave - 1) * C + K::off(cl), acc);
+    __syncthreads();
+    if (wave > 0) return;
+    if (slot == 0 && active)
+      for (int w = 1; w < parts; ++w) acc += K::ld(comb + (w - 1) * C + K::off(cl));
+  }
   if (slot == 0 && active) K::st(gX + static_cast<int64_t>(node) * C + K::off(cl), acc);
 }
 
@@ -468,16 +494,24 @@ int launch_backward(const float *X, const float *Y, const float *R, const float 
 template <int C>
 int launch_sender(const float *gXe, const int32_t *perm, const int32_t *offsets, int64_t nnodes, int64_t nedges,
                   float *gX, hipStream_t st, const float *live_vec, const float *live_r, float r_max) {
-  const dim3 grid(static_cast<unsigned>(nnodes)), block(kWave);
+  const int parts = parts_for(nnodes, nedges);
+  const dim3 grid(static_cast<unsigned>(nnodes)), block(parts * kWave);
+#define CM_SENDER(LIVE_, by_, rmax_)                                                                                                   \
+  do {                                                                                                                                 \
+    if (parts > 1)                                                                                                                     \
+      hipLaunchKernelGGL((mp_backward_sender_kernel<C, LIVE_, true>), grid, block, 0, st, gXe, perm, offsets, static_cast<int>(nnodes), \
+                         nedges, by_, rmax_, gX);                                                                                      \
+    else                                                                                                                               \
+      hipLaunchKernelGGL((mp_backward_sender_kernel<C, LIVE_, false>), grid, block, 0, st, gXe, perm, offsets,                         \
+                         static_cast<int>(nnodes), nedges, by_, rmax_, gX);                                                            \
+  } while (0)
   if (live_vec)
-    hipLaunchKernelGGL((mp_backward_sender_kernel<C, 1>), grid, block, 0, st, gXe, perm, offsets, static_cast<int>(nnodes), nedges,
-                       live_vec, r_max, gX);
+    CM_SENDER(1, live_vec, r_max);
   else if (live_r)
-    hipLaunchKernelGGL((mp_backward_sender_kernel<C, 2>), grid, block, 0, st, gXe, perm, offsets, static_cast<int>(nnodes), nedges,
-                       live_r, r_max, gX);
+    CM_SENDER(2, live_r, r_max);
   else
-    hipLaunchKernelGGL((mp_backward_sender_kernel<C, 0>), grid, block, 0, st, gXe, perm, offsets, static_cast<int>(nnodes), nedges,
-                       static_cast<const float *>(nullptr), 0.f, gX);
+    CM_SENDER(0, static_cast<const float *>(nullptr), 0.f);
+#undef CM_SENDER
   return check_launch("cm_mp_backward (sender pass)");
 }
 

@@ -251,6 +251,16 @@ __device__ __forceinline__ float edge_length(float v0, float v1, float v2) {
   return sqrtf(fmaf(v2, v2, fmaf(v1, v1, v0 * v0)));
 }
 
+// Parts a node's edge range is cut into where one wave per node would leave most of the device idle (a 216-atom cell is
+// 216 waves for 1 024 SIMDs, each walking its ~90 edges one after the other): as many as fill about 2 048 wave slots
+// and leave a part a dozen edges on average, at most 8.
+inline int parts_for(int64_t nnodes, int64_t nedges) {
+  if (nnodes <= 0) return 1;
+  const int64_t by_slots = 2048 / nnodes, by_edges = nedges / (12 * nnodes);
+  const int64_t parts = by_slots < by_edges ? by_slots : by_edges;
+  return parts < 1 ? 1 : (parts > 8 ? 8 : static_cast<int>(parts));
+}
+
 // Sender pass of the backward, shared by both variants (defined in mp.hip).  With live_vec (edge vectors [E, 3]) or
 // live_r (edge lengths [E]) given, only the rows of edges within r_max are read: the spline-fused edge pass writes no
 // others.

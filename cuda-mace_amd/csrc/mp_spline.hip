@@ -117,16 +117,6 @@ __device__ __forceinline__ int stage_edges(const float *__restrict__ Y, const in
 // LDS of one wave's staged chunk: Y [kChunk][16], sender, knot interval, offset in it, position (floats / ints)
 constexpr int kStageBytes = kChunk * 64 + 4 * kChunk * 4;
 
-// Parts a node's edge range is cut into where one wave per node would leave most of the device idle (a 216-atom cell is
-// 216 waves for 1 024 SIMDs, each walking its ~90 edges one after the other): as many as fill about 2 048 wave slots
-// and leave a part a dozen edges on average, at most 8.
-inline int parts_for(int64_t nnodes, int64_t nedges) {
-  if (nnodes <= 0) return 1;
-  const int64_t by_slots = 2048 / nnodes, by_edges = nedges / (12 * nnodes);
-  const int64_t parts = by_slots < by_edges ? by_slots : by_edges;
-  return parts < 1 ? 1 : (parts > 8 ? 8 : static_cast<int>(parts));
-}
-
 template <int L>
 struct MRange {
   static constexpr int lo = L * L;

@@ -10,8 +10,9 @@
 //   d e[n] / d h1[n, c] = scale * w1[c]                                        (constant, not stored)
 //
 // and, on request, the [N, 2C] fp64 concatenation of the features that the model returns as "node_feats" (row n
-// optionally written to row feats_rows[n], for callers that keep their nodes in another order internally).  The
-// backward is then a scaling of those derivatives by the incoming gradient of e[n].
+// optionally written to row feats_rows[n], for callers that keep their nodes in another order internally) and the
+// node's total energy e[n] + e0[n] (e0: a given constant per node, e.g. the atomic reference energy), written to the same
+// row.  The backward is then a scaling of those derivatives by the incoming gradient of e[n].
 //
 // Work split: a workgroup of 256 threads keeps W2a and w1 in LDS and walks tiles of 16 nodes; a tile's rows of both
 // feature arrays are staged in LDS with coalesced 16-byte loads; thread (node, j) accumulates z_j over the channels,
@@ -19,6 +20,7 @@
 #include <cmath>
 
 #include "common.hpp"
+#include "readout.hpp"
 
 namespace cm {
 namespace {
@@ -36,7 +38,7 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     const float *__restrict__ h1, const float *__restrict__ h2, const double *__restrict__ w1, const double *__restrict__ W2a,
     const double *__restrict__ w2b, double act_cst, double scale, double shift, int nnodes, int C, int H,
     double *__restrict__ node_es, float *__restrict__ d2, double *__restrict__ feats64,
-    const int32_t *__restrict__ feats_rows) {
+    const int32_t *__restrict__ feats_rows, const double *__restrict__ node_e0, double *__restrict__ node_total) {
   __shared__ __attribute__((aligned(16))) double sW[kHidden * kLdW];  // W2a transposed [16, C]; rows beyond H are zero
   __shared__ double sw1[kMaxC];
   __shared__ __attribute__((aligned(16))) float s1[kNodes * kLdS];
@@ -155,7 +157,14 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     double e = e1 + e2;
 #pragma unroll
     for (int off = kHidden / 2; off > 0; off >>= 1) e += __shfl_xor(e, off);
-    if (live && j == 0) node_es[node0 + r] = scale * e + shift;
+    if (live && j == 0) {
+      const double en = scale * e + shift;
+      node_es[node0 + r] = en;
+      if (node_total) {
+        const int row = feats_rows ? feats_rows[node0 + r] : node0 + r;
+        if (static_cast<unsigned>(row) < static_cast<unsigned>(nnodes)) node_total[row] = en + (node_e0 ? node_e0[node0 + r] : 0.0);
+      }
+    }
     __syncthreads();
     // d e / d h2: a thread keeps the 16 weights of its channel in registers and serves a share of the tile's rows
     // (256 / C row groups; the rows' 16 factors are read by all lanes of a group at once)
@@ -189,22 +198,34 @@ __global__ void readout_backward_kernel(const double *__restrict__ g, const doub
 }  // namespace
 }  // namespace cm
 
-extern "C" int cm_readout_forward(const float *h1, const float *h2, const double *w1, const double *W2a, const double *w2b,
-                                  double act_cst, double scale, double shift, int64_t nnodes, int channels, int hidden,
-                                  double *node_energies, float *d_h2, double *node_feats64, const int32_t *feats_rows,
-                                  cm_stream_t stream) {
-  CM_REQUIRE(channels >= 1 && channels <= cm::kMaxC, "cm_readout_forward: channels=%d must be in [1, %d]", channels, cm::kMaxC);
-  CM_REQUIRE(hidden >= 1 && hidden <= cm::kHidden, "cm_readout_forward: hidden=%d must be in [1, %d]", hidden, cm::kHidden);
+namespace cm {
+
+int readout_forward_with_totals(const float *h1, const float *h2, const double *w1, const double *W2a, const double *w2b,
+                                double act_cst, double scale, double shift, int64_t nnodes, int channels, int hidden,
+                                double *node_energies, float *d_h2, double *node_feats64, const int32_t *rows,
+                                const double *node_e0, double *node_total, hipStream_t st) {
+  CM_REQUIRE(channels >= 1 && channels <= kMaxC, "cm_readout_forward: channels=%d must be in [1, %d]", channels, kMaxC);
+  CM_REQUIRE(hidden >= 1 && hidden <= kHidden, "cm_readout_forward: hidden=%d must be in [1, %d]", hidden, kHidden);
   CM_REQUIRE(nnodes >= 0 && nnodes < INT32_MAX / 2, "cm_readout_forward: nnodes out of range");
   if (nnodes == 0) return CM_OK;
   CM_REQUIRE(h1 && h2 && w1 && W2a && w2b && node_energies && d_h2, "cm_readout_forward: NULL pointer");
   // at most kMaxGroups workgroups (two per compute unit of a 256-unit device fit by their LDS): each stages the
   // weights once and walks several tiles
-  const int64_t tiles = cm::ceil_div(nnodes, cm::kNodes);
-  hipLaunchKernelGGL(cm::readout_forward_kernel, dim3(static_cast<unsigned>(tiles < cm::kMaxGroups ? tiles : cm::kMaxGroups)),
-                     dim3(cm::kNodes * cm::kHidden), 0, cm::as_stream(stream), h1, h2, w1, W2a, w2b, act_cst, scale, shift,
-                     static_cast<int>(nnodes), channels, hidden, node_energies, d_h2, node_feats64, feats_rows);
-  return cm::check_launch("cm_readout_forward");
+  const int64_t tiles = ceil_div(nnodes, kNodes);
+  hipLaunchKernelGGL(readout_forward_kernel, dim3(static_cast<unsigned>(tiles < kMaxGroups ? tiles : kMaxGroups)),
+                     dim3(kNodes * kHidden), 0, st, h1, h2, w1, W2a, w2b, act_cst, scale, shift, static_cast<int>(nnodes), channels,
+                     hidden, node_energies, d_h2, node_feats64, rows, node_e0, node_total);
+  return check_launch("cm_readout_forward");
+}
+
+}  // namespace cm
+
+extern "C" int cm_readout_forward(const float *h1, const float *h2, const double *w1, const double *W2a, const double *w2b,
+                                  double act_cst, double scale, double shift, int64_t nnodes, int channels, int hidden,
+                                  double *node_energies, float *d_h2, double *node_feats64, const int32_t *feats_rows,
+                                  cm_stream_t stream) {
+  return cm::readout_forward_with_totals(h1, h2, w1, W2a, w2b, act_cst, scale, shift, nnodes, channels, hidden, node_energies, d_h2,
+                                         node_feats64, feats_rows, nullptr, nullptr, cm::as_stream(stream));
 }
 
 extern "C" int cm_readout_backward(const double *grad_node_energies, const double *w1, const float *d_h2, double scale,

@@ -27,6 +27,7 @@
 #include "common.hpp"
 #include "mp_common.hpp"
 #include "node_glue.hpp"
+#include "readout.hpp"
 
 namespace cm {
 namespace {
@@ -86,6 +87,13 @@ __global__ void fill_f64_kernel(double *p, int64_t n, double value) {
     p[i] = value;
 }
 
+// p[i] = src[i], or zero without a source
+__global__ void copy_or_zero_f64_kernel(double *p, const double *src, int64_t n) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    p[i] = src ? src[i] : 0.0;
+}
+
 // g1[n, c] = -weight[n] * scale * w1[c]: the gradient of -sum(weight * node energies) with respect to the first layer's
 // features (the linear readout); without weights the same row for every node
 __global__ void seed_linear_readout_kernel(float *__restrict__ g1, const double *__restrict__ w1, double scale,
@@ -102,22 +110,38 @@ __global__ void weight_rows_kernel(float *__restrict__ x, const double *__restri
     x[i] = static_cast<float>(static_cast<double>(x[i]) * node_weights[i / C]);
 }
 
-// Edge range of every receiver node cut back to its last edge inside the cutoff: live[n] = first_occ[n],
-// live[nnodes + n] = one past the last edge e of the node with |vec[e]| <= r_max (the node's first edge if there is
-// none).  The message-passing kernels, forward and backward, skip the edges behind it: they contribute exact zeros to the
-// forward, and their vector gradients, exact zeros as well, are written by this kernel.  A Verlet list holds a third more pairs than the cutoff
-// takes in; the model orders each node's pairs with those of the skin shell last, nearest first, so that most of them
-// fall behind this mark.  The length is the one the message-passing kernels compute from the same fp32 vector.
-__global__ void live_range_kernel(const int32_t *__restrict__ first_occ, const float *__restrict__ vec, float r_max, int nnodes,
-                                  int64_t nedges, int32_t *__restrict__ live, float *__restrict__ gv1, float *__restrict__ gv2) {
-  const int n = blockIdx.x * blockDim.x + threadIdx.x;
-  if (n >= nnodes) return;
+// Edge vectors and the edge range of every receiver node cut back to its last edge inside the cutoff, one launch.
+// Thread i forms the vector of edge i (fp64 difference of the positions plus the shift, rounded once to fp32: the
+// arithmetic of cm_edge_geometry_forward) and, as node i, finds live[i] = first_occ[i], live[nnodes + i] = one past the
+// last edge e of the node with |vec[e]| <= r_max (the node's first edge if there is none).  The message-passing kernels,
+// forward and backward, skip the edges behind that mark: they contribute exact zeros to the forward, and their vector
+// gradients, exact zeros as well, are written here.  A Verlet list holds a third more pairs than the cutoff takes in; the
+// model orders each node's pairs with those of the skin shell last, nearest first, so that most of them fall behind the
+// mark.  The node's walk forms the vectors of its last edges again rather than wait for the threads that store them; the
+// length is the one the message-passing kernels compute from the same fp32 vector.
+__global__ __launch_bounds__(256) void geometry_live_range_kernel(const double *__restrict__ pos, const int32_t *__restrict__ a,
+                                                                  const int32_t *__restrict__ b, const double *__restrict__ shifts,
+                                                                  const int32_t *__restrict__ rows, const int32_t *__restrict__ first_occ,
+                                                                  float r_max, int nnodes, int64_t nedges, float *__restrict__ vec,
+                                                                  int32_t *__restrict__ live, float *__restrict__ gv1,
+                                                                  float *__restrict__ gv2) {
+  const int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  double v[3];
+  if (i < nedges) {
+    edge_vector_f64(pos, a, b, shifts, rows, i, nnodes, v);
+    vec[3 * i + 0] = static_cast<float>(v[0]);
+    vec[3 * i + 1] = static_cast<float>(v[1]);
+    vec[3 * i + 2] = static_cast<float>(v[2]);
+  }
+  if (i >= nnodes) return;
+  const int n = static_cast<int>(i);
   int e0 = first_occ[n], e1 = first_occ[nnodes + n];
   clamp_edge_range(e0, e1, nedges);
   int e = e1;
   while (e > e0) {
     const int64_t q = e - 1;
-    if (mp::edge_length(vec[3 * q + 0], vec[3 * q + 1], vec[3 * q + 2]) <= r_max) break;
+    edge_vector_f64(pos, a, b, shifts, rows, q, nnodes, v);
+    if (mp::edge_length(static_cast<float>(v[0]), static_cast<float>(v[1]), static_cast<float>(v[2])) <= r_max) break;
     // an edge behind the mark: the backward edge passes skip it as well, so its vector gradients are cleared here
     gv1[3 * q + 0] = gv1[3 * q + 1] = gv1[3 * q + 2] = 0.f;
     gv2[3 * q + 0] = gv2[3 * q + 1] = gv2[3 * q + 2] = 0.f;
@@ -131,7 +155,8 @@ __global__ void live_range_kernel(const int32_t *__restrict__ first_occ, const f
 // tree over the partials: the same order on every run.
 constexpr int kSumThreads = 1024;
 __global__ __launch_bounds__(kSumThreads) void segment_sum_f64_kernel(const double *__restrict__ x, const double *__restrict__ weights,
-                                                                     const int32_t *__restrict__ ptr, double *__restrict__ out) {
+                                                                     const int32_t *__restrict__ ptr, double *__restrict__ out,
+                                                                     const double *__restrict__ graph_e0, double *__restrict__ total) {
   __shared__ double part[kSumThreads];
   const int lo = ptr[blockIdx.x], hi = ptr[blockIdx.x + 1];
   double s = 0.0;
@@ -142,7 +167,10 @@ __global__ __launch_bounds__(kSumThreads) void segment_sum_f64_kernel(const doub
     if (threadIdx.x < d) part[threadIdx.x] += part[threadIdx.x + d];
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = part[0];
+  if (threadIdx.x == 0) {
+    out[blockIdx.x] = part[0];
+    if (total) total[blockIdx.x] = part[0] + (graph_e0 ? graph_e0[blockIdx.x] : 0.0);
+  }
 }
 
 // Virials from the per-edge gradients the backward chain ends with: under a symmetric strain every edge vector becomes
@@ -228,7 +256,7 @@ inline size_t align256(size_t n) { return (n + 255) & ~static_cast<size_t>(255);
 
 // Carves the workspace; the same walk sizes it (base == nullptr) and lays it out.
 struct Layout {
-  float *vec, *len, *gv1, *gv2, *bufM1, *bufM2, *bufA, *edge_scratch;
+  float *vec, *gv1, *gv2, *bufM1, *bufM2, *bufA, *edge_scratch;
   float *B1, *h1, *sc, *X2, *B2, *h2, *d_h2, *g1, *gB, *gX2, *gh1a, *gh1;
   int32_t *live;         // [2 N] edge ranges cut back to the last edge inside the cutoff
   double *node_virial;   // [N, 6]
@@ -243,7 +271,7 @@ struct Layout {
     };
     auto f = [&](int64_t n) { return reinterpret_cast<float *>(take(static_cast<size_t>(n) * sizeof(float))); };
     const int64_t NC = N * C;
-    vec = f(3 * E), len = f(E), gv1 = f(3 * E), gv2 = f(3 * E);
+    vec = f(3 * E), gv1 = f(3 * E), gv2 = f(3 * E);
     bufM1 = f(16 * NC), bufM2 = f(16 * NC), bufA = f(16 * NC);
     edge_scratch = f(E * C);
     B1 = f(NC), h1 = f(NC), sc = f(NC), X2 = f(NC), B2 = f(NC), h2 = f(NC), d_h2 = f(NC);
@@ -307,7 +335,8 @@ extern "C" int cm_mace_step_timing_read(double *total_ms, int64_t *launches, int
 
 extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, const double *positions, const double *shifts,
                             void *workspace, size_t workspace_bytes, double *interaction_energy, double *node_energy,
-                            double *forces, double *node_feats, double *virials, cm_stream_t stream) {
+                            double *forces, double *node_feats, double *virials, double *total_energy, double *total_node_energy,
+                            cm_stream_t stream) {
   CM_REQUIRE(w && g, "cm_mace_step: NULL weights or graph");
   const int64_t N = g->nnodes, E = g->nedges;
   const int C = w->channels, ne = w->nelements;
@@ -330,9 +359,12 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
     hipLaunchKernelGGL(cm::fill_f64_kernel, dim3(1), dim3(64), 0, st, interaction_energy, static_cast<int64_t>(g->ngraphs), 0.0);
     if (virials)
       hipLaunchKernelGGL(cm::fill_f64_kernel, dim3(1), dim3(64), 0, st, virials, static_cast<int64_t>(9) * g->ngraphs, 0.0);
+    if (total_energy)
+      hipLaunchKernelGGL(cm::copy_or_zero_f64_kernel, dim3(1), dim3(64), 0, st, total_energy, g->graph_e0, static_cast<int64_t>(g->ngraphs));
     return cm::check_launch("cm_mace_step");
   }
   CM_REQUIRE(positions && node_energy && forces, "cm_mace_step: NULL positions or output");
+  CM_REQUIRE(N < INT32_MAX / 4 && E < INT32_MAX, "cm_mace_step: sizes out of range");
   CM_REQUIRE(E == 0 || shifts, "cm_mace_step: NULL shifts");
   CM_REQUIRE(g->first_occ && g->sender_offsets && g->elem_perm && g->elem_offsets && g->onehot_perm && g->onehot_offsets && g->X1,
              "cm_mace_step: NULL graph structure");
@@ -353,13 +385,11 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   const float *none = nullptr;
 
   // ---- forward ----
-  {
+  if (E > 0) {
     cm::StageTimer timer_(st, 0, timing_mask);
-    const int rc_ = cm_edge_geometry_forward(positions, g->receiver, g->sender, shifts, g->node_rows, N, E, L.vec, L.len, stream);
-    if (rc_ != CM_OK) return rc_;
-    if (E > 0)
-      hipLaunchKernelGGL(cm::live_range_kernel, dim3(static_cast<unsigned>(cm::ceil_div(N, 256))), dim3(256), 0, st, g->first_occ,
-                         L.vec, w->r_max, static_cast<int>(N), E, L.live, L.gv1, L.gv2);
+    hipLaunchKernelGGL(cm::geometry_live_range_kernel, dim3(static_cast<unsigned>(cm::ceil_div(std::max(N, E), 256))), dim3(256), 0, st,
+                       positions, g->receiver, g->sender, shifts, g->node_rows, g->first_occ, w->r_max, static_cast<int>(N), E, L.vec,
+                       L.live, L.gv1, L.gv2);
   }
   const int32_t *fo_live = E > 0 ? L.live : g->first_occ;
   const float *X[2] = {g->X1, L.X2};
@@ -391,12 +421,12 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
     else
       CM_STAGE(t == 0 ? 4 : 10, cm_linear(B[t], w->prod_WT[t], nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, t == 1 ? L.sc : none, h[t], stream));
   }
-  CM_STAGE(11, cm_readout_forward(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden, node_energy,
-                             L.d_h2, node_feats, g->node_rows, stream));
+  CM_STAGE(11, cm::readout_forward_with_totals(L.h1, L.h2, w->w1, w->W2a, w->w2b, w->act_cst, w->scale, w->shift, N, C, w->hidden,
+                                               node_energy, L.d_h2, node_feats, g->node_rows, g->node_e0, total_node_energy, st));
   if (!glue) {  // with the chained kernels the sums ride in the backward chain's launch
     cm::StageTimer timer_(st, 12, timing_mask);
     hipLaunchKernelGGL(cm::segment_sum_f64_kernel, dim3(g->ngraphs), dim3(cm::kSumThreads), 0, st, node_energy, g->node_weights,
-                       g->graph_ptr, interaction_energy);
+                       g->graph_ptr, interaction_energy, g->graph_e0, total_energy);
   }
 
   // ---- backward: d(-sum of node energies) / d positions ----
@@ -422,7 +452,7 @@ extern "C" int cm_mace_step(const cm_mace_weights *w, const cm_mace_graph *g, co
   if (glue) {
     CM_STAGE(17, cm::node_glue_backward_with_energy_sums(L.gX2, L.d_h2, w->up_W, w->skip_W, w->prod_W[0], w->w1, w->scale, g->node_weights,
                                                          oh_perm, oh_off, N, ne + 1, C, w->skip_scale, L.gB, node_energy, g->graph_ptr,
-                                                         g->ngraphs, interaction_energy, st));
+                                                         g->ngraphs, interaction_energy, g->graph_e0, total_energy, st));
   } else {
     CM_STAGE(17, cm_linear(L.gX2, w->up_W, nullptr, nullptr, N, 1, 0, 1, C, C, 1.0f, none, L.g1, L.gh1a, stream));
     CM_STAGE(18, cm_linear(L.d_h2, w->skip_W, oh_perm, oh_off, N, ne + 1, 1, 1, C, C, -w->skip_scale, none, L.gh1a, L.gh1, stream));

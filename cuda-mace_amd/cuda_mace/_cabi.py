@@ -78,7 +78,7 @@ SIGNATURES = {
     "cm_probe_fma": (_i32, [_p, _i32, _i32, _p]),
     "cm_mace_step_timing_read": (_i32, [_p, _p, _i32]),
     "cm_mace_step_workspace": (_sz, [_i64, _i64, _i32]),
-    "cm_mace_step": (_i32, [_p, _p, _p, _p, _p, _sz, _p, _p, _p, _p, _p, _p]),
+    "cm_mace_step": (_i32, [_p, _p, _p, _p, _p, _sz, _p, _p, _p, _p, _p, _p, _p, _p]),
     # fp64 instantiations: same argument lists, floating-point buffers in double
     "cm_mp_forward_f64": (_i32, [_p, _p, _p, _p, _p, _i64, _i64, _i32, _p, _p]),
     "cm_mp_backward_f64": (_i32, [_p] * 8 + [_i64, _i64, _i32] + [_p] * 5),

@@ -538,19 +538,15 @@ class OptimizedInvariantMACE(torch.nn.Module):
             t = data["node_weights"]
             inner["node_weights"] = _cached_for(data["edge_index"], "_cm_spatial_node_weights", t, lambda: t.index_select(0, perm))
         rows = _cached(data["edge_index"], "_cm_spatial_rows32", None, lambda: (perm.int(), inverse))
-        out = self._forward_ordered(inner, training, compute_force, compute_virials, compute_stress, compute_displacement,
-                                    node_rows=rows, positions_in_caller_order=direct)
-        # node_feats is already written in the caller's order, and so are the forces on the direct path
-        for name in ("node_energy",) if direct else ("forces", "node_energy"):
-            if out.get(name) is not None:
-                out[name] = out[name].index_select(0, inverse)
-        return out
+        # per-node outputs come back in the caller's order (node_rows)
+        return self._forward_ordered(inner, training, compute_force, compute_virials, compute_stress, compute_displacement,
+                                     node_rows=rows, positions_in_caller_order=direct)
 
     def _forward_ordered(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
                          compute_virials: bool = False, compute_stress: bool = False, compute_displacement: bool = False,
                          node_rows=None, positions_in_caller_order: bool = False) -> Dict[str, Optional[torch.Tensor]]:
-        """node_rows = (rows int32 [N], inverse int64 [N]): node n of `data` is node rows[n] of the caller; the
-        returned node_feats is written in the caller's order (every other per-node output stays in the order of `data`).
+        """node_rows = (rows int32 [N], inverse int64 [N]): node n of `data` is node rows[n] of the caller, and the
+        per-node outputs (forces, node_energy, node_feats) are returned in the caller's order.
         positions_in_caller_order: data["positions"] (and hence the forces) are rows of the caller, read through rows."""
         data["positions"].requires_grad_(True)
         positions = data["positions"]
@@ -588,12 +584,17 @@ class OptimizedInvariantMACE(torch.nn.Module):
         node_weights = data.get("node_weights")
         if node_weights is not None:
             node_weights = node_weights.detach().to(torch.float64)
-            e0 = scatter_sum(src=node_e0 * node_weights, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
-        elif num_graphs == 1 and node_heads is None:
-            # one graph: the sum of the atomic reference energies is a function of the species tensor alone, too
-            e0 = _cached_for(node_attrs, "_cm_e0_sum", self._weights_token, lambda: node_e0.sum(dim=0, keepdim=True))
-        else:
-            e0 = scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
+
+        def graph_e0(weights=node_weights):
+            """(Weighted) sum of the atomic reference energies per graph.  The one-call step evaluates it once per
+            list (it rides in the step's graph handle); the autograd path evaluates it per call."""
+            if weights is not None:
+                return scatter_sum(src=node_e0 * weights, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
+            if num_graphs == 1 and node_heads is None:
+                # one graph: the sum of the atomic reference energies is a function of the species tensor alone, too
+                return _cached_for(node_attrs, "_cm_e0_sum", self._weights_token, lambda: node_e0.sum(dim=0, keepdim=True))
+            return scatter_sum(src=node_e0, index=batch, dim=0, dim_size=num_graphs, ptr=data["ptr"])
+
         node_feats = None
 
         # index structures shared by both layers, cached on the caller's tensors so that they are rebuilt only when
@@ -611,11 +612,11 @@ class OptimizedInvariantMACE(torch.nn.Module):
             # X1, which depends on this model's weights)
             handle = _cached_per(edge_index, "_cm_native_graphs", self._weights_token, node_attrs,
                                  lambda: native.graph(edge_index, receiver, sender, node_attrs32, atom_types, data["ptr"],
-                                                      node_feats_up, rows32))
+                                                      node_feats_up, rows32, node_e0, graph_e0(None)))
             if node_weights is not None:
                 plain = handle
                 handle = _cached_per(data["node_weights"], "_cm_native_graphs_weighted", self._weights_token, plain,
-                                     lambda: plain.with_node_weights(node_weights))
+                                     lambda: plain.with_node_weights(node_weights, graph_e0()))
             want_virials = compute_virials or compute_stress
             res = native(handle, positions, shifts, want_virials=want_virials)
             inter_e = res["interaction_energy"]
@@ -625,8 +626,10 @@ class OptimizedInvariantMACE(torch.nn.Module):
                 c3 = cell.view(-1, 3, 3).to(virials.dtype)  # the volume as a triple product: a few element-wise launches
                 volume = (c3[:, 0] * torch.linalg.cross(c3[:, 1], c3[:, 2], dim=-1)).sum(dim=-1).abs()
                 stress = -virials / volume.view(-1, 1, 1)
+            # energy = e0 + interaction energy and node_energy = node_e0 + its interaction part (already in the caller's
+            # order) are written by the step's own kernels: the atomic reference energies ride in the handle
             return {
-                "energy": e0 + inter_e, "node_energy": node_e0 + res["node_energy"], "interaction_energy": inter_e,
+                "energy": res["energy"], "node_energy": res["node_energy"], "interaction_energy": inter_e,
                 "forces": res["forces"].to(data["positions"].dtype), "virials": virials, "stress": stress, "hessian": None,
                 "displacement": displacement, "node_feats": res["node_feats"], "edge_forces": None,
             }
@@ -679,12 +682,16 @@ class OptimizedInvariantMACE(torch.nn.Module):
         weighted_es = node_inter_es.double() if node_weights is None else node_inter_es.double() * node_weights
         inter_e = scatter_sum(src=weighted_es, index=batch, dim=-1, dim_size=num_graphs, ptr=data["ptr"])
 
-        total_energy = e0 + inter_e
+        total_energy = graph_e0() + inter_e
         node_energy = node_e0 + node_inter_es
+        if node_rows is not None:  # node_feats is already written in the caller's order
+            node_energy = node_energy.index_select(0, node_rows[1])
 
         forces, virials, stress, hessian, edge_forces = get_outputs(
             energy=inter_e, positions=data["positions"], displacement=displacement, cell=cell, training=training,
             compute_force=compute_force, compute_virials=compute_virials, compute_stress=compute_stress)
+        if node_rows is not None and not positions_in_caller_order and forces is not None:
+            forces = forces.index_select(0, node_rows[1])
 
         return {
             "energy": total_energy, "node_energy": node_energy, "interaction_energy": inter_e, "forces": forces,

@@ -37,7 +37,7 @@ class _Graph(ctypes.Structure):
         ("nnodes", ctypes.c_int64), ("nedges", ctypes.c_int64), ("ngraphs", ctypes.c_int),
         ("receiver", _fp), ("sender", _fp), ("first_occ", _fp), ("sender_perm", _fp), ("sender_offsets", _fp),
         ("elem_perm", _fp), ("elem_offsets", _fp), ("onehot_perm", _fp), ("onehot_offsets", _fp),
-        ("node_rows", _fp), ("graph_ptr", _fp), ("X1", _fp), ("node_weights", _fp),
+        ("node_rows", _fp), ("graph_ptr", _fp), ("X1", _fp), ("node_weights", _fp), ("node_e0", _fp), ("graph_e0", _fp),
     ]
 
 
@@ -99,8 +99,11 @@ class NativeStep:
         self.weights, self._keep, self.channels, self.nelements = w, keep, C, w.nelements
         self._workspace = None
 
-    def graph(self, edge_index, receiver, sender, node_attrs32, atom_types, ptr, X1, node_rows) -> "_GraphHandle":
-        """Struct of the index structures of one neighbour list + species tensor (all cached on those tensors)."""
+    def graph(self, edge_index, receiver, sender, node_attrs32, atom_types, ptr, X1, node_rows, node_e0=None,
+              graph_e0=None) -> "_GraphHandle":
+        """Struct of the index structures of one neighbour list + species tensor (all cached on those tensors).
+        node_e0 fp64 [N] (order of the lists) / graph_e0 fp64 [ngraphs]: what the step adds to the interaction part in its
+        "energy" and (caller-ordered) "node_energy" outputs; None counts as zeros."""
         N = int(node_attrs32.shape[0])
         g = _Graph()
         I32 = torch.int32
@@ -118,7 +121,19 @@ class NativeStep:
         g.node_rows = _ptr(node_rows, I32, "node_rows") if node_rows is not None else None
         g.graph_ptr, g.X1 = _ptr(ptr32, I32, "graph_ptr"), _ptr(X1, torch.float32, "X1")
         g.node_weights = None
-        return _GraphHandle(g, (receiver, sender, first_occ, sperm, soff, eperm, eoff, operm, ooff, ptr32, X1, node_rows))
+        F64 = torch.float64
+        if node_e0 is not None:
+            node_e0 = node_e0.detach().to(F64).contiguous()
+            if node_e0.shape != (N,):
+                raise cabi.CudaMaceError("native step: node_e0 must be [%d]" % N)
+        if graph_e0 is not None:
+            graph_e0 = graph_e0.detach().to(F64).contiguous()
+            if graph_e0.shape != (int(g.ngraphs),):
+                raise cabi.CudaMaceError("native step: graph_e0 must be [%d]" % int(g.ngraphs))
+        g.node_e0 = _ptr(node_e0, F64, "node_e0") if node_e0 is not None else None
+        g.graph_e0 = _ptr(graph_e0, F64, "graph_e0") if graph_e0 is not None else None
+        return _GraphHandle(g, (receiver, sender, first_occ, sperm, soff, eperm, eoff, operm, ooff, ptr32, X1, node_rows, node_e0,
+                                graph_e0))
 
     def __call__(self, handle: "_GraphHandle", positions: torch.Tensor, shifts: torch.Tensor, want_feats: bool = True,
                  want_virials: bool = False) -> Dict[str, torch.Tensor]:
@@ -145,26 +160,37 @@ class NativeStep:
         forces = torch.empty(N, 3, dtype=F64, device=dev)
         feats = torch.empty(N, 2 * C, dtype=F64, device=dev) if want_feats else None
         virials = torch.empty(int(g.ngraphs), 3, 3, dtype=F64, device=dev) if want_virials else None
+        total = torch.empty(int(g.ngraphs), dtype=F64, device=dev)
+        node_total = torch.empty(N, dtype=F64, device=dev)
         cabi._check(cabi.lib.cm_mace_step(
             ctypes.addressof(self.weights), ctypes.addressof(g), _ptr(pos64, F64, "positions"), _ptr(sh64, F64, "shifts"),
             ws.data_ptr(), ws.numel(), _ptr(energy, F64, "energy"), _ptr(node_energy, F64, "node_energy"),
             _ptr(forces, F64, "forces"), _ptr(feats, F64, "node_feats") if want_feats else None,
-            _ptr(virials, F64, "virials") if want_virials else None, cabi._stream()))
-        return {"interaction_energy": energy, "node_energy": node_energy, "forces": forces, "node_feats": feats,
-                "virials": virials}
+            _ptr(virials, F64, "virials") if want_virials else None, _ptr(total, F64, "total_energy"),
+            _ptr(node_total, F64, "total_node_energy"), cabi._stream()))
+        # energy / node_energy: the interaction part plus the handle's graph_e0 / node_e0, node_energy in the caller's
+        # order (rows node_rows of the handle); interaction_node_energy: the interaction part alone, in list order
+        return {"interaction_energy": energy, "interaction_node_energy": node_energy, "energy": total, "node_energy": node_total,
+                "forces": forces, "node_feats": feats, "virials": virials}
 
 
 class _GraphHandle:
     def __init__(self, struct, keep):
         self.struct, self._keep = struct, keep
 
-    def with_node_weights(self, weights: torch.Tensor) -> "_GraphHandle":
+    def with_node_weights(self, weights: torch.Tensor, graph_e0: Optional[torch.Tensor] = None) -> "_GraphHandle":
         """The same index structures with a weight per node energy (fp64 [nnodes], in the order of the lists): the step
-        then returns sum_n weights[n] * node_energy[n] per graph and minus its gradient."""
+        then returns sum_n weights[n] * node_energy[n] per graph and minus its gradient.  graph_e0: the constant per
+        graph that goes with these weights (None keeps the handle's)."""
         if weights.shape != (int(self.struct.nnodes),):
             raise cabi.CudaMaceError("node weights must be [%d]" % int(self.struct.nnodes))
         g = _Graph()
         ctypes.memmove(ctypes.addressof(g), ctypes.addressof(self.struct), ctypes.sizeof(_Graph))
         w = weights.detach().to(torch.float64).contiguous()
         g.node_weights = _ptr(w, torch.float64, "node_weights")
-        return _GraphHandle(g, (self._keep, w))
+        if graph_e0 is not None:
+            graph_e0 = graph_e0.detach().to(torch.float64).contiguous()
+            if graph_e0.shape != (int(g.ngraphs),):
+                raise cabi.CudaMaceError("graph_e0 must be [%d]" % int(g.ngraphs))
+            g.graph_e0 = _ptr(graph_e0, torch.float64, "graph_e0")
+        return _GraphHandle(g, (self._keep, w, graph_e0))

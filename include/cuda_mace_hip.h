@@ -495,13 +495,18 @@ int cm_node_glue_backward(const float *gX2, const float *d_h2, const float *up_W
  *     and in the quantity the forces derive from, sum_n node_weights[n] * node_energy[n]; what the rank of a
  *     domain-decomposed MD code needs (1 for its own atoms, 0 for ghost copies: upstream MACE's LAMMPS wrapper,
  *     mace/calculators/lammps_mace.py; the reference has no counterpart).  NULL is all ones, bit for bit.
+ *   node_e0 fp64 [nnodes] (in the order of the lists) / graph_e0 fp64 [ngraphs], or NULL = zeros: what total_node_energy /
+ *     total_energy add to the interaction part, i.e. the atomic reference energies of the species and their (weighted)
+ *     sum per graph (models/InvariantMACE.py:287-293 computes them per call; they depend on the species alone)
  * Per call: positions fp64 [nnodes, 3], shifts fp64 [nedges, 3]; outputs interaction_energy fp64 [ngraphs] ((weighted) sum
  * of the node energies of each graph, in a fixed order), node_energy fp64 [nnodes] (interaction part, unweighted, in
  * list order), forces fp64 [nnodes, 3] = -d(sum of interaction_energy)/d positions (rows of the caller when node_rows is given), node_feats fp64
  * [nnodes, 2C] or NULL, virials fp64 [ngraphs, 3, 3] or NULL = minus the derivative of each graph's energy with respect to a
  * symmetric strain of its positions and cell (what models/InvariantMACE.py:273-285 obtains by differentiating through
  * get_symmetric_displacement), formed from the per-edge gradients as 1/2 sum_e (vec_e (x) g_e + g_e (x) vec_e), g_e =
- * -dE/d vec_e.  workspace: cm_mace_step_workspace(nnodes, nedges, channels) bytes, 256-byte aligned; its
+ * -dE/d vec_e.  total_energy fp64 [ngraphs] or NULL = interaction_energy + graph_e0; total_node_energy fp64 [nnodes] or NULL
+ * = node_energy + node_e0, atom n of the lists written to row node_rows[n] (what the reference returns as "energy" and
+ * "node_energy", models/InvariantMACE.py:350-352, without a launch of their own).  workspace: cm_mace_step_workspace(nnodes, nedges, channels) bytes, 256-byte aligned; its
  * contents are scratch.  Nothing is allocated, so the call can be captured into a HIP graph.
  */
 typedef struct cm_mace_weights {
@@ -530,6 +535,7 @@ typedef struct cm_mace_graph {
   const int32_t *node_rows, *graph_ptr;
   const float *X1;
   const double *node_weights;
+  const double *node_e0, *graph_e0;
 } cm_mace_graph;
 
 /* Per-stage timing of cm_mace_step (off by default): with bit s of stage_mask set, stage s of every later step is
@@ -551,7 +557,7 @@ int cm_mace_step_timing_read(double *total_ms, int64_t *launches, int capacity);
 size_t cm_mace_step_workspace(int64_t nnodes, int64_t nedges, int channels);
 int cm_mace_step(const cm_mace_weights *weights, const cm_mace_graph *graph, const double *positions, const double *shifts,
                  void *workspace, size_t workspace_bytes, double *interaction_energy, double *node_energy, double *forces,
-                 double *node_feats, double *virials, cm_stream_t stream);
+                 double *node_feats, double *virials, double *total_energy, double *total_node_energy, cm_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -146,6 +146,58 @@ def test_build_refuses_copies_into_landing_registers():
         build._scan_landing_registers("linear.hip", ok[:4] + ok[5:])
 
 
+def test_build_refuses_use_of_a_register_before_its_load_has_landed():
+    """Kernels that issue loads from inline assembly and wait for them later: the build walks their generated code with
+    the hardware's rule (vector-memory operations retire in order; s_waitcnt vmcnt(n) leaves the newest n out) and fails
+    on any instruction that touches a register while a load into it is in flight -- the copy a compiler may place where
+    such a register crosses a loop's back edge, which reads the register before the data is there."""
+    import importlib.util
+
+    import pytest
+
+    spec = importlib.util.spec_from_file_location("_cm_build", os.path.join(ROOT, "cuda-mace_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    head = ["_ZN2cm13other_kernelEv:  ; @x", "\tglobal_load_dword v5, v[2:3], off", "\tv_mov_b32_e32 v6, v5", ".Lfunc_end0:",
+            "_ZN2cm25mp_backward_sender_kernelILi128ELi1ELb0EEE:  ; @y"]
+    tail = ["\ts_endpgm", ".Lfunc_end1:"]
+    ok = ["\tglobal_load_dword v5, v[2:3], off", "\tv_add_u32_e32 v9, v8, v7", "\ts_waitcnt vmcnt(0)", "\tv_mov_b32_e32 v6, v5",
+          ".LBB1_1:  ; loop", "\tv_add_f32_e32 v10, v6, v10",
+          "\tglobal_load_dword v5, v[2:3], off", "\tglobal_load_lds_dwordx4 v[20:21], off nt", "\tglobal_load_dword v12, v[2:3], off",
+          "\tv_add_u32_e32 v20, 4, v20",                       # the address of a load that lands in LDS is free at once
+          "\ts_waitcnt vmcnt(1) lgkmcnt(0)", "\tv_mov_b32_e32 v6, v5",  # the older load has landed, the newest may be out
+          "\t;;#ASMSTART", "\t; landed v12", "\t;;#ASMEND", "\tv_mov_b32_e32 v13, v12",  # the source says so: taken at its word
+          "\ts_cbranch_scc1 .LBB1_1"]
+    assert build._scan_in_flight_registers("mp.hip", head + ok + tail) == 1  # kernels not named may do as they like
+
+    def scan(body):
+        build._scan_in_flight_registers("mp.hip", head + body + tail)
+
+    with pytest.raises(RuntimeError, match="v_mov_b32_e32 v14, v12.*touches v12"):  # newest load still out at vmcnt(1)
+        scan(ok[:12] + ["\tv_mov_b32_e32 v14, v12"] + ok[12:])
+    with pytest.raises(RuntimeError, match="touches v5"):  # written, not read: the load would land on top of it
+        scan(ok[:7] + ["\tv_mov_b32_e32 v5, 0"] + ok[7:])
+    with pytest.raises(RuntimeError, match="touches v5"):  # used as an address
+        scan(ok[:7] + ["\tglobal_load_dword v30, v[4:5], off"] + ok[7:])
+    # issued at the bottom of the loop, waited for at its top: the copy across the back edge reads too early ...
+    loop = [".LBB1_1:", "\ts_waitcnt vmcnt(0)", "\tv_add_f32_e32 v10, v38, v10", "\tglobal_load_dword v46, v[2:3], off",
+            "\tv_mov_b32_e32 v38, v46", "\ts_cbranch_scc1 .LBB1_1"]
+    with pytest.raises(RuntimeError, match="v_mov_b32_e32 v38, v46.*touches v46"):
+        scan(loop)
+    scan(loop[:4] + loop[5:])  # ... without it the register is first read behind the wait at the top
+    # ... and a use that only the way round the back edge makes too early is found as well
+    with pytest.raises(RuntimeError, match="v_add_f32_e32 v10, v46, v10.*touches v46"):
+        scan([".LBB1_1:", "\tv_add_f32_e32 v10, v46, v10", "\ts_waitcnt vmcnt(0)", "\tglobal_load_dword v46, v[2:3], off",
+              "\ts_cbranch_scc1 .LBB1_1"])
+    # a wait on one side of a branch only does not count for the other side
+    with pytest.raises(RuntimeError, match="touches v5"):
+        scan(["\tglobal_load_dword v5, v[2:3], off", "\ts_cbranch_scc1 .LBB1_2", "\ts_waitcnt vmcnt(0)", ".LBB1_2:", "\tv_mov_b32_e32 v6, v5"])
+    scan(["\tglobal_load_dword v5, v[2:3], off", "\ts_cbranch_scc1 .LBB1_2", "\ts_waitcnt vmcnt(0)", "\ts_branch .LBB1_3", ".LBB1_2:",
+          "\ts_waitcnt vmcnt(0)", ".LBB1_3:", "\tv_mov_b32_e32 v6, v5"])
+    with pytest.raises(RuntimeError, match="no code found"):
+        build._scan_in_flight_registers("mp.hip", head[:4])
+
+
 def test_header_is_valid_c_and_cpp(tmp_path):
     """The boundary is a C ABI: the header must compile as plain C (what cgo, a Fortran binding generator or LAMMPS'
     C glue would include) and as C++, on its own."""
