@@ -226,6 +226,146 @@ __global__ __launch_bounds__(kWaves *kWave) void linear_kernel(const float *__re
 }
 
 // -----------------------------------------------------------------------------------------------
+// Few tiles (a system of a few hundred atoms): the launch is over in a few microseconds, most of which a workgroup of the
+// kernel above spends waiting for one K chunk after the other, with next to nothing to multiply in between.  Here a
+// workgroup (one tile, one component, 32 output columns) requests every K chunk of both operands, the row scales and
+// the residual values at once and waits for memory once; K = 32 KCH.  Staging, operand split, piece products and their
+// order, and the epilogue's roundings are those of the kernel above: the same bits.
+template <int KCH, bool SCALED>
+__global__ __launch_bounds__(kWaves *kWave) void linear_few_tiles_kernel(const float *__restrict__ X, const float *__restrict__ WT,
+                                                                         const int32_t *__restrict__ node_perm,
+                                                                         const int32_t *__restrict__ group_offsets, int nnodes,
+                                                                         int ngroups, int zero_last_group, int ncomp, float scale,
+                                                                         const float *__restrict__ row_scale, const float *residual,
+                                                                         float *OUT, int nout_total) {
+  constexpr int K = kKC * KCH;
+  constexpr int NOUT = 32;
+  const int col0 = blockIdx.y * NOUT;
+  __shared__ __attribute__((aligned(16))) __bf16 sAp[3 * kTileNodes * kLdH];
+  __shared__ __attribute__((aligned(16))) __bf16 sBp[3 * NOUT * kLdH];
+  __shared__ int sNode[kTileNodes];
+
+  const int tid = threadIdx.x;
+  const int lane = tid % kWave;
+  const int wave = tid / kWave;
+  const int m = blockIdx.x % ncomp;
+  const int l = ncomp == 1 ? 0 : l_of_m(m);
+  const int nblocks = ncomp == 1 ? 1 : 4;
+
+  int g, pos0, gend;
+  if (!locate_group_tile(group_offsets, ngroups, nnodes, blockIdx.x / ncomp, kTileNodes, g, pos0, gend)) return;
+  const int nrows = min(kTileNodes, gend - pos0);
+  if (tid < kTileNodes) {
+    int node = -1;
+    if (tid < nrows) {
+      node = node_perm ? node_perm[pos0 + tid] : pos0 + tid;
+      if (static_cast<unsigned>(node) >= static_cast<unsigned>(nnodes)) node = -1;
+    }
+    sNode[tid] = node;
+  }
+  __syncthreads();
+
+  if (zero_last_group && g == ngroups - 1) {
+    for (int i = tid; i < kTileNodes * NOUT; i += kWaves * kWave) {
+      const int node = sNode[i / NOUT];
+      if (node >= 0) {
+        const int64_t at = (static_cast<int64_t>(node) * ncomp + m) * nout_total + col0 + i % NOUT;
+        OUT[at] = residual ? residual[at] : 0.f;
+      }
+    }
+    return;
+  }
+  const float *Wg = WT + ((static_cast<int64_t>(g) * nblocks + l) * nout_total + col0) * K;  // [NOUT, K] of [nout_total, K]
+
+  constexpr int kTPR = kKC / 4;
+  constexpr int kRPP = kWaves * kWave / kTPR;
+  static_assert(kRPP == NOUT, "one pass of the staging map covers the 32 weight rows");
+  constexpr int A_PASSES = kTileNodes / kRPP;
+  const int srow = tid / kTPR;
+  const int scol = (tid % kTPR) * 4;
+  const int mrow = lane % 32;
+  const int half = lane / 32;
+
+  // everything this workgroup reads, requested before anything is waited for
+  f4 pa[KCH][A_PASSES], pb[KCH], ps[SCALED ? KCH : 1][A_PASSES];
+#pragma unroll
+  for (int i = 0; i < A_PASSES; ++i) {
+    const int node = sNode[kRPP * i + srow];
+    const float *xp = X + (static_cast<int64_t>(node >= 0 ? node : 0) * ncomp + m) * K + scol;
+    const float *sp = SCALED ? row_scale + static_cast<int64_t>(node >= 0 ? node : 0) * K + scol : nullptr;
+#pragma unroll
+    for (int c = 0; c < KCH; ++c) {
+      pa[c][i] = node >= 0 ? ld4_stream(xp + kKC * c) : zero4();
+      if constexpr (SCALED) ps[c][i] = node >= 0 ? ld4(sp + kKC * c) : zero4();
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < KCH; ++c) pb[c] = ld4(Wg + static_cast<int64_t>(srow) * K + kKC * c + scol);
+  float res[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int node = sNode[32 * wave + 8 * (r / 4) + 4 * half + (r % 4)];
+    res[r] = (residual && node >= 0) ? residual[(static_cast<int64_t>(node) * ncomp + m) * nout_total + col0 + mrow] : 0.f;
+  }
+
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+  for (int c = 0; c < KCH; ++c) {
+    if (c > 0) __syncthreads();  // previous chunk fully consumed
+#pragma unroll
+    for (int i = 0; i < A_PASSES; ++i) {
+      f4 v = pa[c][i];
+      if constexpr (SCALED) v *= ps[c][i];
+      bf16x4 h, md, lw;
+      split3(v, h, md, lw);
+      const int at = (kRPP * i + srow) * kLdH + scol;
+      *reinterpret_cast<bf16x4 *>(sAp + at) = h;
+      *reinterpret_cast<bf16x4 *>(sAp + kTileNodes * kLdH + at) = md;
+      *reinterpret_cast<bf16x4 *>(sAp + 2 * kTileNodes * kLdH + at) = lw;
+    }
+    {
+      bf16x4 h, md, lw;
+      split3(pb[c], h, md, lw);
+      const int at = srow * kLdH + scol;
+      *reinterpret_cast<bf16x4 *>(sBp + at) = h;
+      *reinterpret_cast<bf16x4 *>(sBp + NOUT * kLdH + at) = md;
+      *reinterpret_cast<bf16x4 *>(sBp + 2 * NOUT * kLdH + at) = lw;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < kKC; ks += 16) {
+      const int aoff = (32 * wave + mrow) * kLdH + ks + 8 * half;
+      bf16x8 a[3], b[3];
+#pragma unroll
+      for (int p = 0; p < 3; ++p) {
+        a[p] = *reinterpret_cast<const bf16x8 *>(sAp + p * kTileNodes * kLdH + aoff);
+        b[p] = *reinterpret_cast<const bf16x8 *>(sBp + p * NOUT * kLdH + mrow * kLdH + ks + 8 * half);
+      }
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[2], b[0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[2], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[1], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[1], b[0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[1], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[0], acc, 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int node = sNode[32 * wave + 8 * (r / 4) + 4 * half + (r % 4)];
+    if (node < 0) continue;
+    float *op = OUT + (static_cast<int64_t>(node) * ncomp + m) * nout_total + col0 + mrow;
+    {
+#pragma clang fp contract(off)  // the product is rounded before the residual is added, as everywhere
+      const float v = acc[r] * scale;
+      *op = residual ? v + res[r] : v;
+    }
+  }
+}
+
+// -----------------------------------------------------------------------------------------------
 // Variant with the feature rows on a ring of raw fp32 chunks in LDS, filled by direct global -> LDS loads.
 //
 // What bounds the kernel above is the amount of X that a workgroup has in flight: one 16 KB chunk, and only while it
@@ -857,6 +997,19 @@ int launch(const float *X, const float *WT, const int32_t *perm, const int32_t *
   // few tiles (less than half a workgroup per compute unit): 32 columns per workgroup
   if (NT > 1 && tiles * ncomp * 2 <= device_compute_units()) {
     const dim3 split(grid.x, NT);
+    if (K <= 4 * kKC) {  // every chunk requested at once (registers for four of them)
+#define CM_FEW(KCH_, SCALED_)                                                                                                       \
+  hipLaunchKernelGGL((linear_few_tiles_kernel<KCH_, SCALED_>), split, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups, \
+                     zero_last_group, ncomp, scale, row_scale, residual, OUT, NOUT)
+      switch (K / kKC) {
+        case 1: if (row_scale) CM_FEW(1, true); else CM_FEW(1, false); break;
+        case 2: if (row_scale) CM_FEW(2, true); else CM_FEW(2, false); break;
+        case 3: if (row_scale) CM_FEW(3, true); else CM_FEW(3, false); break;
+        default: if (row_scale) CM_FEW(4, true); else CM_FEW(4, false); break;
+      }
+#undef CM_FEW
+      return check_launch("cm_linear");
+    }
     if (row_scale)
       hipLaunchKernelGGL((linear_kernel<1, true>), split, block, 0, st, X, WT, perm, offs, static_cast<int>(nnodes), ngroups,
                          zero_last_group, ncomp, K, scale, row_scale, residual, OUT, NOUT);

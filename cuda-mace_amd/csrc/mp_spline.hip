@@ -128,7 +128,7 @@ struct MRange {
 // -----------------------------------------------------------------------------------------------
 // MULTI: a workgroup of up to eight waves per node, each on a part of the node's edge range (launched for few nodes)
 template <int C, bool FROM_VEC, bool MULTI>
-__global__ __launch_bounds__(MULTI ? 8 * kWave : kWave, (Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVES)) void mp_spline_forward_kernel(const float *__restrict__ X,
+__global__ __launch_bounds__(MULTI ? 8 * kWave : kWave, (MULTI || Cfg<C, true>::V > 5 ? 2 : CM_FUSED_FWD_WAVES)) void mp_spline_forward_kernel(const float *__restrict__ X,
                                                                  const float *__restrict__ Y, Spline sp,
                                                                  const int32_t *__restrict__ sender,
                                                                  const int32_t *__restrict__ first_occ, int nnodes,
@@ -172,37 +172,87 @@ __global__ __launch_bounds__(MULTI ? 8 * kWave : kWave, (Cfg<C, true>::V > 5 ? 2
                                             [](int, int, unsigned long long, bool) {});
     wave_lds_fence();
     if (active) {
-      for (int j = slot; j < nlive; j += K::EPW) {
+      // what one edge brings in: the sender's row piece, the 16 coefficient pieces of its knot interval, its harmonics
+      struct Edge {
+        vec x, coef[16];
+        float y[16], xr;
+      };
+      auto fetch = [&](int j, Edge &e) {
         const int s = sS[j];
         const int idx = sIdx[j];
-        const float xr = sXr[j];
-        const vec x = K::ld(X + (static_cast<unsigned>(s) * C + unsigned(K::off(cl))));
-        float y[16];
-        {
-          const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
+        e.xr = sXr[j];
+        e.x = K::ld(X + (static_cast<unsigned>(s) * C + unsigned(K::off(cl))));
+        const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const f4 v = yp[q];
-            y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
-          }
+        for (int q = 0; q < 4; ++q) {
+          const f4 v = yp[q];
+          e.y[4 * q] = v.x, e.y[4 * q + 1] = v.y, e.y[4 * q + 2] = v.z, e.y[4 * q + 3] = v.w;
         }
         const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(K::off(cl));  // 32-bit offset from the uniform table base
-        const float *__restrict__ tab = sp.coeffs;
+        // addressed from the middle of the interval's 16C-float row: all 16 pieces lie within +-8C floats of it, which
+        // up to C = 128 fits the signed immediate offset of a load, so one address serves them all
+        const float *mid = sp.coeffs + (co + 8 * C);
+#pragma unroll
+        for (int q = 0; q < 16; ++q) e.coef[q] = K::ld(mid + (q * C - 8 * C));  // piece q: coefficient q / 4 of degree q % 4
+      };
+      auto accumulate = [&](const Edge &e) {
         auto per_l = [&](auto lc) {
           constexpr int L = decltype(lc)::value;
-          // addressed from the middle of the interval's 16C-float row: all 16 pieces lie within +-8C floats of it, which
-          // up to C = 128 fits the signed immediate offset of a load, so one address serves them all
-          const float *mid = tab + (co + 8 * C);
-          const vec a = K::ld(mid + (L * C - 8 * C)), b = K::ld(mid + (L * C - 4 * C)), c = K::ld(mid + L * C),
-                    d = K::ld(mid + (L * C + 4 * C));
-          const vec t = x * (a + xr * (b + xr * (c + xr * d)));
+          const vec t = e.x * (e.coef[L] + e.xr * (e.coef[4 + L] + e.xr * (e.coef[8 + L] + e.xr * e.coef[12 + L])));
 #pragma unroll
-          for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) acc[m] += y[m] * t;
+          for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) acc[m] += e.y[m] * t;
         };
         per_l(std::integral_constant<int, 0>{});
         per_l(std::integral_constant<int, 1>{});
         per_l(std::integral_constant<int, 2>{});
         per_l(std::integral_constant<int, 3>{});
+      };
+      if constexpr (MULTI && K::V <= 4) {
+        // few nodes: a wave's part is a dozen edges, and what it waits for is one memory round trip per trip of this
+        // loop, so two edges per slot are requested per trip (same order of the sums; registers for it up to four
+        // channels per lane)
+        for (int j = slot; j < nlive; j += 2 * K::EPW) {
+          Edge e0, e1;
+          const bool two = j + K::EPW < nlive;
+          fetch(j, e0);
+          fetch(two ? j + K::EPW : j, e1);
+          __builtin_amdgcn_sched_barrier(0);  // both edges' loads stay ahead of the first edge's arithmetic
+          accumulate(e0);
+          if (two) accumulate(e1);
+        }
+      } else {
+        // one edge per trip; per degree the four coefficient pieces are loaded, used and dropped (16 registers of
+        // radial data live at a time)
+        for (int j = slot; j < nlive; j += K::EPW) {
+          const int s = sS[j];
+          const int idx = sIdx[j];
+          const float xr = sXr[j];
+          const vec x = K::ld(X + (static_cast<unsigned>(s) * C + unsigned(K::off(cl))));
+          float y[16];
+          {
+            const f4 *yp = reinterpret_cast<const f4 *>(sY + j * 16);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const f4 v = yp[q];
+              y[4 * q] = v.x, y[4 * q + 1] = v.y, y[4 * q + 2] = v.z, y[4 * q + 3] = v.w;
+            }
+          }
+          const unsigned co = static_cast<unsigned>(idx) * (16u * C) + unsigned(K::off(cl));
+          const float *__restrict__ tab = sp.coeffs;
+          auto per_l = [&](auto lc) {
+            constexpr int L = decltype(lc)::value;
+            const float *mid = tab + (co + 8 * C);
+            const vec a = K::ld(mid + (L * C - 8 * C)), b = K::ld(mid + (L * C - 4 * C)), c = K::ld(mid + L * C),
+                      d = K::ld(mid + (L * C + 4 * C));
+            const vec t = x * (a + xr * (b + xr * (c + xr * d)));
+#pragma unroll
+            for (int m = MRange<L>::lo; m < MRange<L>::hi; ++m) acc[m] += y[m] * t;
+          };
+          per_l(std::integral_constant<int, 0>{});
+          per_l(std::integral_constant<int, 1>{});
+          per_l(std::integral_constant<int, 2>{});
+          per_l(std::integral_constant<int, 3>{});
+        }
       }
     }
   }

@@ -45,11 +45,6 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
   __shared__ __attribute__((aligned(16))) float s2[kNodes * kLdS];
   __shared__ double sD[kNodes * kHidden];  // w2b[j] * act'(z_j) per node
   const int t = threadIdx.x;
-  for (int i = t; i < C * kHidden; i += blockDim.x) {
-    const int c = i / kHidden, j = i % kHidden;
-    sW[j * kLdW + c] = j < H ? W2a[c * H + j] : 0.0;
-  }
-  for (int c = t; c < C; c += blockDim.x) sw1[c] = w1[c];
   // a workgroup stages the weights once and then walks tiles of 16 nodes; the rows of its next tile are requested
   // before the current one is worked on (one element per trip, each waited for, would cost a memory latency per trip)
   const int ntiles = (nnodes + kNodes - 1) / kNodes;
@@ -68,6 +63,25 @@ __global__ __launch_bounds__(kNodes *kHidden) void readout_forward_kernel(
     }
   };
   if (wide && static_cast<int>(blockIdx.x) < ntiles) request(blockIdx.x);
+  {
+    // the weights: every element this thread stages is requested before the first is stored (one trip after the other,
+    // each waiting for its load, is a memory latency per trip -- most of the launch for a few hundred nodes)
+    constexpr int kWTrips = kMaxC * kHidden / (kNodes * kHidden);
+    double wv[kWTrips];
+#pragma unroll
+    for (int u = 0; u < kWTrips; ++u) {
+      const int i = t + u * (kNodes * kHidden);
+      const int c = i / kHidden, j = i % kHidden;
+      wv[u] = (c < C && j < H) ? W2a[c * H + j] : 0.0;
+    }
+    const double w1v = t < C ? w1[t] : 0.0;
+#pragma unroll
+    for (int u = 0; u < kWTrips; ++u) {
+      const int i = t + u * (kNodes * kHidden);
+      if (i < C * kHidden) sW[(i % kHidden) * kLdW + i / kHidden] = wv[u];
+    }
+    if (t < C) sw1[t] = w1v;
+  }
   for (int tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
     const int node0 = tile * kNodes;
     const int rows = min(kNodes, nnodes - node0);
