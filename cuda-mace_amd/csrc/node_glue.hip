@@ -34,7 +34,6 @@ constexpr int kGlSmallTile = 32;   // where 128-node tiles would occupy less tha
 constexpr int kGlKC = 32;          // K columns staged per step
 constexpr int kGlLdH = kGlKC + 8;  // padded row stride of a bf16 plane (elements)
 constexpr int kGlTPR = kGlKC / 4;  // threads that cover the 32 columns of a staged row, 16 bytes each
-constexpr int kGlSumThreads = 256; // threads that take part in a graph's energy sum (fewer in a smaller workgroup)
 
 // A workgroup has (ROWS / 32) * NT waves (C = 32 NT): wave w owns the 32 x 32 block of the tile's output at rows
 // 32 (w % (ROWS / 32)), columns 32 (w / (ROWS / 32)).  With one wave per block a product's matrix instructions, operand reads and staging
@@ -231,7 +230,8 @@ __global__ __launch_bounds__(ROWS / 32 * NT *kWave) void node_glue_forward_kerne
 }
 
 // Energies per graph, riding in the backward launch (its tiles do not depend on them): out[g] = sum over the graph's nodes
-// of weight[n] * node_es[n], strided partial sums of 256 threads and a tree over them: a fixed order.
+// of weight[n] * node_es[n], strided partial sums of the workgroup's threads (the largest power of two of them) and a tree
+// over them: a fixed order.
 struct EnergySums {
   const double *node_es, *node_weights;
   const int32_t *graph_ptr;
@@ -245,9 +245,17 @@ __device__ __forceinline__ void graph_energy(const EnergySums &q, int graph, dou
   const int tid = threadIdx.x;
   if (tid < THREADS) {
     const int lo = q.graph_ptr[graph], hi = q.graph_ptr[graph + 1];
-    double sum = 0.0;
-    for (int i = lo + tid; i < hi; i += THREADS) sum += q.node_weights ? q.node_weights[i] * q.node_es[i] : q.node_es[i];
-    part[tid] = sum;
+    auto term = [&](int i) { return q.node_weights ? q.node_weights[i] * q.node_es[i] : q.node_es[i]; };
+    // four strided partial sums per thread, their loads requested together: one sum after the other waits for memory
+    // once per node, and this workgroup would outlast the tiles of the launch
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+    int i = lo + tid;
+    for (; i + 3 * THREADS < hi; i += 4 * THREADS) {
+      const double t0 = term(i), t1 = term(i + THREADS), t2 = term(i + 2 * THREADS), t3 = term(i + 3 * THREADS);
+      s0 += t0, s1 += t1, s2 += t2, s3 += t3;
+    }
+    for (; i < hi; i += THREADS) s0 += term(i);
+    part[tid] = (s0 + s1) + (s2 + s3);
   }
   __syncthreads();
   for (int d = THREADS / 2; d > 0; d >>= 1) {
@@ -272,7 +280,7 @@ __global__ __launch_bounds__(ROWS / 32 * NT *kWave) void node_glue_backward_kern
   __shared__ __attribute__((aligned(16))) S s;
   if (static_cast<int>(blockIdx.x) < first_tile) {
     // workgroups ahead of the tiles: the energy of one graph each, from node energies an earlier launch wrote
-    constexpr int kSum = S::kThreads >= kGlSumThreads ? kGlSumThreads : (S::kThreads >= 128 ? 128 : 64);
+    constexpr int kSum = S::kThreads >= 1024 ? 1024 : (S::kThreads >= 512 ? 512 : (S::kThreads >= 256 ? 256 : (S::kThreads >= 128 ? 128 : 64)));
     static_assert(sizeof(s.tile) >= kSum * sizeof(double), "the tile holds the partial sums");
     graph_energy<kSum>(sums, blockIdx.x, reinterpret_cast<double *>(s.tile));
     return;
