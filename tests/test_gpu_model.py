@@ -410,6 +410,30 @@ def test_native_step_on_a_list_with_a_skin(cabi, relabel):
     torch.testing.assert_close(a["forces"], c["forces"], rtol=0, atol=2e-6 * fscale)
 
 
+@pytest.mark.parametrize("natoms,channels", [(60, 64), (700, 128), (3000, 96)])
+def test_step_with_chained_node_kernels_equals_the_separate_launches(cabi, natoms, channels, monkeypatch):
+    """Up to 128 channels the one-call step runs the three [N,C] products between the layers, and their transposes, as one
+    chained launch per direction (on 32-node tiles for few nodes, 128-node tiles otherwise) and sums the energies in that
+    launch; the library's switch for the separate launches (CM_STEP_GLUE=-1, read per call) gives the same step as the
+    same kernels beyond 128 channels run it.  Same operand split, piece order and rounding points: node energies, node
+    features and forces agree bit for bit; the graph energy is a sum in another (fixed) order."""
+    if natoms < 130:  # too few for a periodic box of twice the cutoff: a cluster
+        data = make_system(natoms, 4, seed=5, density=None, cluster_box=10.0)
+    else:
+        data = make_system(natoms, 4, seed=5, density=0.1)
+    _, model = _build(channels, (1, 6, 7, 8), data, seed=6)
+    dev = to_device(data, "cuda")
+    monkeypatch.delenv("CM_STEP_GLUE", raising=False)
+    a = model(dict(dev))
+    monkeypatch.setenv("CM_STEP_GLUE", "-1")
+    b = model(dict(dev))
+    monkeypatch.delenv("CM_STEP_GLUE")
+    assert model._native not in (None, False)
+    assert torch.equal(a["node_energy"], b["node_energy"]) and torch.equal(a["node_feats"], b["node_feats"])
+    assert torch.equal(a["forces"], b["forces"])
+    torch.testing.assert_close(a["energy"], b["energy"], rtol=1e-13, atol=1e-13)
+
+
 def test_a_second_model_on_the_same_tensors_gets_its_own_graph_handle(cabi):
     """Model A evaluated on a batch and deleted, model B (other weights) built and evaluated on the very same tensors,
     several times over so that B's cache token can land on A's freed address: B's one-call step must use B's own first-layer
