@@ -338,6 +338,12 @@ def other_configs(torch, make_system, to_device, OptimizedInvariantMACE, Synthet
                     tuple(range(1, 11)), 10, 50)
     res["c5"] = run("100 000-atom periodic box, 192x0e, 10 elements", make_system(100000, 10, seed=0, density=0.1), 192,
                     tuple(range(1, 11)), 3, 10)
+    # sixteen times the headline size on the one GPU (29 GB of its 288): the list from the device neighbour search
+    from cuda_mace.utils.synthetic import make_large_system
+
+    big = make_large_system(400000, 10, seed=0, density=0.1)
+    res["c4_x16"] = run("400 000-atom periodic box (jittered lattice, 0.1 atoms/A^3), 128x0e, 10 elements",
+                        {k: v for k, v in big.items()}, 128, tuple(range(1, 11)), 2, 5)
     return res
 
 

@@ -111,3 +111,23 @@ def collate(systems) -> Dict[str, torch.Tensor]:
 
 def to_device(data: Dict[str, torch.Tensor], device) -> Dict[str, torch.Tensor]:
     return {k: v.to(device) for k, v in data.items()}
+
+
+def make_large_system(n_atoms: int, num_elements: int, seed: int = 0, density: float = 0.1, cutoff: float = 5.0,
+                      device="cuda") -> Dict[str, torch.Tensor]:
+    """A periodic box of `n_atoms` at `density` atoms / A^3 for sizes at which `make_system`'s rejection sampling and
+    host-side neighbour search take minutes: atoms on randomly chosen sites of a cubic lattice, each moved by up to 0.3
+    lattice spacings per axis (no close pairs), the neighbour list from the device search (utils/neighbour_list.py)."""
+    from .neighbour_list import neighbour_data
+
+    g = torch.Generator().manual_seed(seed)
+    box = (n_atoms / density) ** (1.0 / 3.0)
+    m = int(round(n_atoms ** (1.0 / 3.0))) + 1
+    site = torch.randperm(m ** 3, generator=g)[:n_atoms]
+    grid = torch.stack([site // (m * m), (site // m) % m, site % m], dim=1).double()
+    positions = (grid + 0.5 + 0.6 * (torch.rand(n_atoms, 3, generator=g, dtype=torch.float64) - 0.5)) * (box / m)
+    species = torch.randint(0, num_elements, (n_atoms,), generator=g)
+    node_attrs = torch.nn.functional.one_hot(species, num_elements).double()
+    cell = torch.eye(3, dtype=torch.float64) * box
+    return neighbour_data(positions.to(device), node_attrs.to(device), cutoff=cutoff, pbc=(True, True, True), cell=cell.to(device))
+
