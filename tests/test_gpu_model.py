@@ -468,6 +468,28 @@ def test_step_with_chained_node_kernels_equals_the_separate_launches(cabi, natom
     torch.testing.assert_close(a["energy"], b["energy"], rtol=1e-13, atol=1e-13)
 
 
+@pytest.mark.parametrize("channels", [32, 64, 96, 128, 160, 192, 224, 256])
+def test_repeated_evaluations_agree_bit_for_bit_at_every_width(cabi, channels):
+    """Every kernel sums in a fixed order and reads nothing it (or an earlier kernel of the same step) has not written:
+    the same input gives the same bits again, also after an evaluation of another size has left other values in the
+    shared workspace.  Two sizes per width: with one wave per node and with a node's edges cut into parts (few nodes).
+    (A kernel whose hand-issued loads were read before they had landed once passed every tolerance test and failed
+    only this kind.)"""
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+
+    boxes = {"large": to_device(make_system(2100, 4, seed=12, density=0.1), "cuda"),
+             "small": to_device(make_system(260, 4, seed=11, density=0.1), "cuda")}
+    up = SyntheticInvariantMACE(channels=channels, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=52.0, seed=13)
+    model = OptimizedInvariantMACE(up, device="cuda")  # one model: both boxes share its workspace
+    first = {k: model(dict(d)) for k, d in boxes.items()}
+    assert model._native not in (None, False)
+    for _ in range(2):
+        for k, d in boxes.items():  # the other size ran in between: the workspace holds its leftovers
+            again = model(dict(d))
+            for key in ("energy", "node_energy", "forces", "node_feats"):
+                assert torch.equal(again[key], first[k][key]), "%s of the %s box differs between evaluations at C=%d" % (key, k, channels)
+
+
 def test_a_second_model_on_the_same_tensors_gets_its_own_graph_handle(cabi):
     """Model A evaluated on a batch and deleted, model B (other weights) built and evaluated on the very same tensors,
     several times over so that B's cache token can land on A's freed address: B's one-call step must use B's own first-layer
