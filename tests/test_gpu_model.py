@@ -490,6 +490,60 @@ def test_repeated_evaluations_agree_bit_for_bit_at_every_width(cabi, channels):
                 assert torch.equal(again[key], first[k][key]), "%s of the %s box differs between evaluations at C=%d" % (key, k, channels)
 
 
+def test_step_total_energies_through_the_library_call(cabi):
+    """cm_mace_step's total_energy / total_node_energy: the interaction parts plus the constants handed over in the graph
+    struct (graph_e0 per graph, node_e0 per atom in list order), the per-atom total written to the caller's rows; without
+    the constants the totals are the interaction parts; an empty system returns the constants alone."""
+    import ctypes
+
+    from cuda_mace.models import OptimizedInvariantMACE, SyntheticInvariantMACE
+    from cuda_mace.ops._autograd import groups_of, groups_of_one_hot
+    from cuda_mace.ops.native_step import NativeStep
+    from cuda_mace.utils.synthetic import collate
+
+    data = to_device(collate([make_system(n, 4, seed=40 + k, density=0.1) for k, n in enumerate((140, 170))]), "cuda")
+    n = data["positions"].shape[0]
+    up = SyntheticInvariantMACE(channels=64, atomic_numbers=(1, 6, 7, 8), avg_num_neighbors=data["edge_index"].shape[1] / n, seed=41)
+    model = OptimizedInvariantMACE(up, device="cuda", spatial_order_min_atoms=None)
+    model(dict(data))  # builds the model's own step object and the caches on the tensors
+    step = model._native
+    assert isinstance(step, NativeStep)
+    recv, send = data["edge_index"][0].int().contiguous(), data["edge_index"][1].int().contiguous()
+    attrs32, types = data["node_attrs"].float(), data["node_attrs"].argmax(dim=-1).int()
+    with torch.no_grad():
+        X1 = model.interactions[0].linear_up(model.node_embedding(data["node_attrs"].double()).float())
+    g = torch.Generator().manual_seed(42)
+    rows = torch.randperm(n, generator=g).int().cuda()  # atom k of the lists is row rows[k] of the caller
+    pos_rows = torch.empty_like(data["positions"])
+    pos_rows[rows.long()] = data["positions"]
+    node_e0 = torch.randn(n, generator=g, dtype=torch.float64).cuda()
+    graph_e0 = torch.tensor([3.25, -1.5], dtype=torch.float64, device="cuda")
+    plain = step.graph(data["edge_index"], recv, send, attrs32, types, data["ptr"], X1, rows)
+    full = step.graph(data["edge_index"], recv, send, attrs32, types, data["ptr"], X1, rows, node_e0, graph_e0)
+    a = step(plain, pos_rows, data["shifts"])
+    b = step(full, pos_rows, data["shifts"])
+    assert torch.equal(a["forces"], b["forces"]) and torch.equal(a["interaction_energy"], b["interaction_energy"])
+    assert torch.equal(a["energy"], a["interaction_energy"])
+    assert torch.equal(b["energy"], b["interaction_energy"] + graph_e0)
+    expect = torch.empty(n, dtype=torch.float64, device="cuda")
+    expect[rows.long()] = a["interaction_node_energy"]
+    assert torch.equal(a["node_energy"], expect)
+    expect[rows.long()] = b["interaction_node_energy"] + node_e0
+    assert torch.equal(b["node_energy"], expect)
+    # no atoms: zeros, or the constants
+    lib = cabi.lib
+    empty = ctypes.create_string_buffer(bytes(full.struct))
+    from cuda_mace.ops.native_step import _Graph
+
+    g0 = _Graph.from_buffer(empty)
+    g0.nnodes, g0.nedges = 0, 0
+    out_i = torch.full((2,), 7.0, dtype=torch.float64, device="cuda")
+    out_t = torch.full((2,), 7.0, dtype=torch.float64, device="cuda")
+    cabi._check(lib.cm_mace_step(ctypes.addressof(step.weights), ctypes.addressof(g0), None, None, None, 0, out_i.data_ptr(), None, None,
+                                 None, None, out_t.data_ptr(), None, cabi._stream()))
+    assert torch.equal(out_i, torch.zeros_like(out_i)) and torch.equal(out_t, graph_e0)
+
+
 def test_a_second_model_on_the_same_tensors_gets_its_own_graph_handle(cabi):
     """Model A evaluated on a batch and deleted, model B (other weights) built and evaluated on the very same tensors,
     several times over so that B's cache token can land on A's freed address: B's one-call step must use B's own first-layer
