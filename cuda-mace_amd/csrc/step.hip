@@ -159,9 +159,16 @@ __global__ __launch_bounds__(kSumThreads) void segment_sum_f64_kernel(const doub
                                                                      const double *__restrict__ graph_e0, double *__restrict__ total) {
   __shared__ double part[kSumThreads];
   const int lo = ptr[blockIdx.x], hi = ptr[blockIdx.x + 1];
-  double s = 0.0;
-  for (int i = lo + threadIdx.x; i < hi; i += kSumThreads) s += weights ? weights[i] * x[i] : x[i];
-  part[threadIdx.x] = s;
+  auto term = [&](int i) { return weights ? weights[i] * x[i] : x[i]; };
+  // four strided partial sums per thread, their loads requested together (one sum waits for memory once per element)
+  double s0 = 0.0, s1 = 0.0, s2 = 0.0, s3 = 0.0;
+  int i = lo + threadIdx.x;
+  for (; i + 3 * kSumThreads < hi; i += 4 * kSumThreads) {
+    const double t0 = term(i), t1 = term(i + kSumThreads), t2 = term(i + 2 * kSumThreads), t3 = term(i + 3 * kSumThreads);
+    s0 += t0, s1 += t1, s2 += t2, s3 += t3;
+  }
+  for (; i < hi; i += kSumThreads) s0 += term(i);
+  part[threadIdx.x] = (s0 + s1) + (s2 + s3);
   __syncthreads();
   for (int d = kSumThreads / 2; d > 0; d >>= 1) {
     if (threadIdx.x < d) part[threadIdx.x] += part[threadIdx.x + d];
