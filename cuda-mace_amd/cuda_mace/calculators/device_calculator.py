@@ -52,6 +52,8 @@ class DeviceCalculator:
             use_graph = (not one_call) and node_attrs.shape[0] <= 8192
         self.use_graph = bool(use_graph) and (one_call or not self.compute_stress)
         self.run_ahead = bool(run_ahead)
+        # an MD step reads energy, forces and stress only: a model that can skip the per-node feature output is told to
+        self._forward_kwargs = {"compute_node_feats": False} if one_call else {}
         self.builds = 0
         self.steps = 0
         self.dropped = 0  # steps enqueued on a list that turned out stale, and enqueued again
@@ -79,7 +81,7 @@ class DeviceCalculator:
         self._graph = None
         if self.use_graph:
             self._graph = GraphedStep(self.model, self._data, warmup=1, compute_virials=self.compute_stress,
-                                      compute_stress=self.compute_stress)
+                                      compute_stress=self.compute_stress, **self._forward_kwargs)
         self._moved = 0.0
         self.builds += 1
 
@@ -89,7 +91,7 @@ class DeviceCalculator:
             return self._graph(positions)
         data = dict(self._data)
         data["positions"] = positions.detach()  # an alias: the model marks its own handle as differentiable, not the caller's
-        out = self.model(data, compute_virials=self.compute_stress, compute_stress=self.compute_stress)
+        out = self.model(data, compute_virials=self.compute_stress, compute_stress=self.compute_stress, **self._forward_kwargs)
         return {k: v.detach() for k, v in out.items() if isinstance(v, torch.Tensor)}
 
     def compute(self, positions: torch.Tensor) -> Dict[str, torch.Tensor]:

@@ -508,10 +508,14 @@ class OptimizedInvariantMACE(torch.nn.Module):
 
     def forward(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
                 compute_virials: bool = False, compute_stress: bool = False,
-                compute_displacement: bool = False) -> Dict[str, Optional[torch.Tensor]]:
+                compute_displacement: bool = False, compute_node_feats: bool = True) -> Dict[str, Optional[torch.Tensor]]:
+        """compute_node_feats=False (no counterpart in the reference, which always returns the [N, 2C] fp64 features):
+        "node_feats" may come back as None; the one-call step then skips that output (51 MB at 25 000 atoms x 128
+        channels), which an MD driver never reads."""
         n = data["positions"].shape[0]
         if self.spatial_order_min_atoms is None or n < self.spatial_order_min_atoms or training:
-            return self._forward_ordered(data, training, compute_force, compute_virials, compute_stress, compute_displacement)
+            return self._forward_ordered(data, training, compute_force, compute_virials, compute_stress, compute_displacement,
+                                         compute_node_feats=compute_node_feats)
         # Same step on the relabelled graph.  Everything that depends only on the neighbour list or the species is
         # derived once per tensor object; per call the positions are gathered into the new order and forces, node
         # energies and node features gathered back (fixed-order gathers: results stay reproducible bit for bit).
@@ -540,11 +544,12 @@ class OptimizedInvariantMACE(torch.nn.Module):
         rows = _cached(data["edge_index"], "_cm_spatial_rows32", None, lambda: (perm.int(), inverse))
         # per-node outputs come back in the caller's order (node_rows)
         return self._forward_ordered(inner, training, compute_force, compute_virials, compute_stress, compute_displacement,
-                                     node_rows=rows, positions_in_caller_order=direct)
+                                     node_rows=rows, positions_in_caller_order=direct, compute_node_feats=compute_node_feats)
 
     def _forward_ordered(self, data: Dict[str, torch.Tensor], training: bool = False, compute_force: bool = True,
                          compute_virials: bool = False, compute_stress: bool = False, compute_displacement: bool = False,
-                         node_rows=None, positions_in_caller_order: bool = False) -> Dict[str, Optional[torch.Tensor]]:
+                         node_rows=None, positions_in_caller_order: bool = False,
+                         compute_node_feats: bool = True) -> Dict[str, Optional[torch.Tensor]]:
         """node_rows = (rows int32 [N], inverse int64 [N]): node n of `data` is node rows[n] of the caller, and the
         per-node outputs (forces, node_energy, node_feats) are returned in the caller's order.
         positions_in_caller_order: data["positions"] (and hence the forces) are rows of the caller, read through rows."""
@@ -618,7 +623,7 @@ class OptimizedInvariantMACE(torch.nn.Module):
                 handle = _cached_per(data["node_weights"], "_cm_native_graphs_weighted", self._weights_token, plain,
                                      lambda: plain.with_node_weights(node_weights, graph_e0()))
             want_virials = compute_virials or compute_stress
-            res = native(handle, positions, shifts, want_virials=want_virials)
+            res = native(handle, positions, shifts, want_feats=compute_node_feats, want_virials=want_virials)
             inter_e = res["interaction_energy"]
             virials = res["virials"].to(positions.dtype) if want_virials else None
             stress = None

@@ -544,6 +544,20 @@ def test_step_total_energies_through_the_library_call(cabi):
     assert torch.equal(out_i, torch.zeros_like(out_i)) and torch.equal(out_t, graph_e0)
 
 
+def test_step_without_the_feature_output(cabi):
+    """compute_node_feats=False (what the MD calculators pass): the step skips the [N, 2C] fp64 output and nothing else
+    changes."""
+    data = make_system(500, 4, seed=7, density=0.1)
+    _, model = _build(64, (1, 6, 7, 8), data, seed=8)
+    dev = to_device(data, "cuda")
+    a = model(dict(dev))
+    b = model(dict(dev), compute_node_feats=False)
+    assert model._native not in (None, False)
+    assert a["node_feats"] is not None and b["node_feats"] is None
+    for key in ("energy", "node_energy", "forces", "interaction_energy"):
+        assert torch.equal(a[key], b[key])
+
+
 def test_a_second_model_on_the_same_tensors_gets_its_own_graph_handle(cabi):
     """Model A evaluated on a batch and deleted, model B (other weights) built and evaluated on the very same tensors,
     several times over so that B's cache token can land on A's freed address: B's one-call step must use B's own first-layer
