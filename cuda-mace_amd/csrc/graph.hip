@@ -26,6 +26,7 @@ namespace {
 
 constexpr int kBoxThreads = 1024;
 constexpr int kScanThreads = 1024;
+constexpr int kScanStage = 32 * 1024;  // values staged in LDS at a time (128 KB)
 constexpr int kSegLds = 1024;  // keys of a segment that a wave keeps in LDS
 
 // box[0..2] = smallest coordinate per axis, box[3] = largest extent over the axes (one workgroup; a fixed order)
@@ -101,25 +102,13 @@ __global__ void relabel_nodes_kernel(const int32_t *__restrict__ perm, const int
 __global__ __launch_bounds__(kScanThreads) void degree_scan_kernel(const int32_t *__restrict__ degree, int n,
                                                                    int32_t *__restrict__ first_occ) {
   __shared__ int part[kScanThreads];
-  const int t = threadIdx.x;
-  const int per = (n + kScanThreads - 1) / kScanThreads;
-  const int lo = min(t * per, n), hi = min(lo + per, n);
-  int sum = 0;
-  for (int k = lo; k < hi; ++k) sum += degree[k];
-  part[t] = sum;
-  __syncthreads();
-  for (int d = 1; d < kScanThreads; d <<= 1) {
-    const int v = t >= d ? part[t - d] : 0;
-    __syncthreads();
-    part[t] += v;
-    __syncthreads();
-  }
-  int run = part[t] - sum;
-  for (int k = lo; k < hi; ++k) {
-    first_occ[k] = run;
-    run += degree[k];
-    first_occ[n + k] = run;
-  }
+  __shared__ int stage[kScanStage];
+  workgroup_exclusive_scan<kScanThreads, kScanStage, int>(
+      n, stage, part, [&](int k) { return degree[k]; },
+      [&](int k, int before, int value) {
+        first_occ[k] = before;
+        first_occ[n + k] = before + value;
+      });
 }
 
 // Sort key of an edge inside its segment: pairs within the cutoff by the new label of atom j, the others behind them

@@ -23,6 +23,7 @@ namespace cm {
 namespace {
 
 constexpr int kGridThreads = 1024;
+constexpr int kOffsetsStage = 16 * 1024;  // values staged in LDS at a time by the offsets scan (128 KB)
 constexpr double kBinSlack = 1.0 + 1e-9;
 constexpr int kMaxScan = 32;  // most images of the cell scanned on each side of an atom
 
@@ -324,25 +325,11 @@ __global__ __launch_bounds__(256) void nl_scan_kernel(const double *__restrict__
 __global__ __launch_bounds__(kGridThreads) void nl_offsets_kernel(const int32_t *__restrict__ degree, int n,
                                                                   int32_t *__restrict__ offsets) {
   __shared__ long long part[kGridThreads];
-  const int t = threadIdx.x;
-  const int per = (n + kGridThreads - 1) / kGridThreads;
-  const int lo = min(t * per, n), hi = min(lo + per, n);
-  long long sum = 0;
-  for (int k = lo; k < hi; ++k) sum += degree[k];
-  part[t] = sum;
-  __syncthreads();
-  for (int d = 1; d < kGridThreads; d <<= 1) {
-    const long long v = t >= d ? part[t - d] : 0;
-    __syncthreads();
-    part[t] += v;
-    __syncthreads();
-  }
-  long long run = part[t] - sum;
-  for (int k = lo; k < hi; ++k) {
-    offsets[k] = static_cast<int32_t>(run > INT32_MAX ? INT32_MAX : run);
-    run += degree[k];
-  }
-  if (t == kGridThreads - 1) offsets[n] = static_cast<int32_t>(part[t] > INT32_MAX ? INT32_MAX : part[t]);
+  __shared__ long long stage[kOffsetsStage];
+  const long long total = workgroup_exclusive_scan<kGridThreads, kOffsetsStage, long long>(
+      n, stage, part, [&](int k) { return degree[k]; },
+      [&](int k, long long before, long long) { offsets[k] = static_cast<int32_t>(before > INT32_MAX ? INT32_MAX : before); });
+  if (threadIdx.x == 0) offsets[n] = static_cast<int32_t>(total > INT32_MAX ? INT32_MAX : total);
 }
 
 __device__ __forceinline__ bool key_less(int ja, const int32_t *Sa, int jb, const int32_t *Sb) {

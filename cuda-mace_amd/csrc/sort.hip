@@ -14,6 +14,7 @@ namespace cm {
 namespace {
 
 constexpr int kScanThreads = 1024;
+constexpr int kScanStage = 32 * 1024;  // values staged in LDS at a time (128 KB)
 
 __global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t value) {
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
@@ -35,27 +36,14 @@ __global__ __launch_bounds__(kScanThreads) void scan_kernel(const int32_t *__res
                                                             int32_t *__restrict__ offsets,
                                                             int32_t *__restrict__ cursor) {
   __shared__ int part[kScanThreads];
-  const int t = threadIdx.x;
-  const int per = (nkeys + kScanThreads - 1) / kScanThreads;
-  const int lo = min(t * per, nkeys);
-  const int hi = min(lo + per, nkeys);
-  int sum = 0;
-  for (int k = lo; k < hi; ++k) sum += counts[k];
-  part[t] = sum;
-  __syncthreads();
-  for (int d = 1; d < kScanThreads; d <<= 1) {
-    const int v = t >= d ? part[t - d] : 0;
-    __syncthreads();
-    part[t] += v;
-    __syncthreads();
-  }
-  int run = part[t] - sum;  // exclusive prefix of this thread's run
-  for (int k = lo; k < hi; ++k) {
-    offsets[k] = run;
-    if (cursor) cursor[k] = run;
-    run += counts[k];
-  }
-  if (t == kScanThreads - 1) offsets[nkeys] = part[t];
+  __shared__ int stage[kScanStage];
+  const int total = workgroup_exclusive_scan<kScanThreads, kScanStage, int>(
+      nkeys, stage, part, [&](int k) { return counts[k]; },
+      [&](int k, int before, int) {
+        offsets[k] = before;
+        if (cursor) cursor[k] = before;
+      });
+  if (threadIdx.x == 0) offsets[nkeys] = total;
 }
 
 __global__ void bucket_fill_kernel(const int32_t *__restrict__ keys, int64_t n, int nkeys,

@@ -112,13 +112,42 @@ __global__ void weight_rows_kernel(float *__restrict__ x, const double *__restri
 
 // Edge vectors and the edge range of every receiver node cut back to its last edge inside the cutoff, one launch.
 // Thread i forms the vector of edge i (fp64 difference of the positions plus the shift, rounded once to fp32: the
-// arithmetic of cm_edge_geometry_forward) and, as node i, finds live[i] = first_occ[i], live[nnodes + i] = one past the
-// last edge e of the node with |vec[e]| <= r_max (the node's first edge if there is none).  The message-passing kernels,
-// forward and backward, skip the edges behind that mark: they contribute exact zeros to the forward, and their vector
-// gradients, exact zeros as well, are written here.  A Verlet list holds a third more pairs than the cutoff takes in; the
-// model orders each node's pairs with those of the skin shell last, nearest first, so that most of them fall behind the
-// mark.  The node's walk forms the vectors of its last edges again rather than wait for the threads that store them; the
-// length is the one the message-passing kernels compute from the same fp32 vector.
+// arithmetic of cm_edge_geometry_forward) and clears the vector gradients of an edge beyond the cutoff (the backward edge
+// passes skip the edges behind a node's mark, and write the same zeros for those before it).  The thread of a receiver's
+// last edge closes the receiver's range: live[n] = first_occ[n], live[nnodes + n] = one past the last edge e of the node
+// with |vec[e]| <= r_max (the node's first edge if there is none).  The message-passing kernels, forward and backward,
+// skip the edges behind that mark, which contribute exact zeros.  A Verlet list holds a third more pairs than the cutoff
+// takes in; the model orders each node's pairs with those of the skin shell last, nearest first, so that most of them
+// fall behind the mark.  The closing thread reads the mark off the workgroup's ballots of "inside the cutoff" where the
+// node's edges up to the mark lie among the workgroup's 256; otherwise it walks back from the workgroup's first edge,
+// forming those vectors again (a walk over all of a node's tail, one line of memory per lane and access, cost a list
+// with a skin 60 us per step).  The length is the one the message-passing kernels compute from the same fp32 vector.
+__device__ __forceinline__ int walk_back_to_live_edge(const double *__restrict__ pos, const int32_t *__restrict__ a,
+                                                      const int32_t *__restrict__ b, const double *__restrict__ shifts,
+                                                      const int32_t *__restrict__ rows, int nnodes, float r_max, int e0, int e) {
+  constexpr int kAhead = 4;  // edges per trip, their operands requested together
+  bool found = false;
+  while (e > e0 && !found) {
+    float len[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int64_t q = max(e - 1 - u, e0);  // below the range: the first edge again, never looked at
+      double w[3];
+      edge_vector_f64(pos, a, b, shifts, rows, q, nnodes, w);
+      len[u] = mp::edge_length(static_cast<float>(w[0]), static_cast<float>(w[1]), static_cast<float>(w[2]));
+    }
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      if (found || e <= e0) continue;
+      if (len[u] <= r_max)
+        found = true;
+      else
+        --e;
+    }
+  }
+  return e;
+}
+
 __global__ __launch_bounds__(256) void geometry_live_range_kernel(const double *__restrict__ pos, const int32_t *__restrict__ a,
                                                                   const int32_t *__restrict__ b, const double *__restrict__ shifts,
                                                                   const int32_t *__restrict__ rows, const int32_t *__restrict__ first_occ,
@@ -126,29 +155,65 @@ __global__ __launch_bounds__(256) void geometry_live_range_kernel(const double *
                                                                   int32_t *__restrict__ live, float *__restrict__ gv1,
                                                                   float *__restrict__ gv2) {
   const int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
-  double v[3];
+  const int lane = threadIdx.x % kWave;
+  bool inside = false;
+  int recv = -1, next_recv = -2;
   if (i < nedges) {
+    double v[3];
     edge_vector_f64(pos, a, b, shifts, rows, i, nnodes, v);
-    vec[3 * i + 0] = static_cast<float>(v[0]);
-    vec[3 * i + 1] = static_cast<float>(v[1]);
-    vec[3 * i + 2] = static_cast<float>(v[2]);
+    const float v0 = static_cast<float>(v[0]), v1 = static_cast<float>(v[1]), v2 = static_cast<float>(v[2]);
+    vec[3 * i + 0] = v0;
+    vec[3 * i + 1] = v1;
+    vec[3 * i + 2] = v2;
+    inside = mp::edge_length(v0, v1, v2) <= r_max;
+    if (!inside) {
+      gv1[3 * i + 0] = gv1[3 * i + 1] = gv1[3 * i + 2] = 0.f;
+      gv2[3 * i + 0] = gv2[3 * i + 1] = gv2[3 * i + 2] = 0.f;
+    }
+    recv = a[i];
+    next_recv = i + 1 < nedges ? a[i + 1] : -2;
   }
-  if (i >= nnodes) return;
-  const int n = static_cast<int>(i);
-  int e0 = first_occ[n], e1 = first_occ[nnodes + n];
-  clamp_edge_range(e0, e1, nedges);
-  int e = e1;
-  while (e > e0) {
-    const int64_t q = e - 1;
-    edge_vector_f64(pos, a, b, shifts, rows, q, nnodes, v);
-    if (mp::edge_length(static_cast<float>(v[0]), static_cast<float>(v[1]), static_cast<float>(v[2])) <= r_max) break;
-    // an edge behind the mark: the backward edge passes skip it as well, so its vector gradients are cleared here
-    gv1[3 * q + 0] = gv1[3 * q + 1] = gv1[3 * q + 2] = 0.f;
-    gv2[3 * q + 0] = gv2[3 * q + 1] = gv2[3 * q + 2] = 0.f;
-    --e;
+  // "inside the cutoff" of the workgroup's 256 consecutive edges, one word per wave (every thread arrives here)
+  __shared__ unsigned long long s_inside[4];
+  const int wave = threadIdx.x / kWave;
+  const unsigned long long inside_mask = __ballot(inside);
+  if (lane == 0) s_inside[wave] = inside_mask;
+  __syncthreads();
+  if (i < nedges && recv != next_recv && static_cast<unsigned>(recv) < static_cast<unsigned>(nnodes)) {
+    int e0 = first_occ[recv], e1 = first_occ[nnodes + recv];
+    clamp_edge_range(e0, e1, nedges);
+    int e;
+    if (e1 == i + 1) {  // this is the last edge of the receiver's range, as in every sorted list
+      const int64_t group_first = i - threadIdx.x;  // first edge of the workgroup
+      e = -1;
+      // the node's edges in this workgroup, from this wave down: the highest one inside the cutoff
+      for (int w = wave; w >= 0 && e < 0; --w) {
+        const int64_t wave_first = group_first + w * kWave;
+        if (wave_first + kWave <= e0) break;  // the node's range begins above this wave
+        const int hi = w == wave ? lane : kWave - 1;
+        const int lo = e0 > wave_first ? static_cast<int>(e0 - wave_first) : 0;
+        const unsigned long long upto = hi == kWave - 1 ? ~0ull : (1ull << (hi + 1)) - 1ull;
+        const unsigned long long mine = s_inside[w] & upto & ~((1ull << lo) - 1ull);
+        if (mine != 0) e = static_cast<int>(wave_first) + (63 - __clzll(static_cast<long long>(mine))) + 1;
+      }
+      if (e < 0)
+        e = e0 >= group_first ? e0
+                              : walk_back_to_live_edge(pos, a, b, shifts, rows, nnodes, r_max, e0, static_cast<int>(group_first));
+    } else {
+      e = walk_back_to_live_edge(pos, a, b, shifts, rows, nnodes, r_max, e0, e1);
+    }
+    live[recv] = e0;
+    live[nnodes + recv] = e;
   }
-  live[n] = e0;
-  live[nnodes + n] = e;
+  if (i < nnodes) {  // a node without edges: an empty range
+    const int n = static_cast<int>(i);
+    int e0 = first_occ[n], e1 = first_occ[nnodes + n];
+    clamp_edge_range(e0, e1, nedges);
+    if (e0 >= e1) {
+      live[n] = e0;
+      live[nnodes + n] = e0;
+    }
+  }
 }
 
 // out[g] = sum of x over the nodes ptr[g] .. ptr[g + 1]: one workgroup per graph, every thread a strided partial sum, a
