@@ -12,9 +12,11 @@
 // Inside a workgroup a quad of four lanes serves one receiver node, four channels per lane, so a wave works on 16 nodes
 // at once.  Edges are taken four at a time: lane k of the quad loads edge k of the block, computes its length, knot
 // interval, offset and the eight harmonics, and in step j of the block the whole quad handles edge j: the X row piece of
-// its sender is one contiguous 64 bytes over the quad, and the edge's values come from lane j through a quad permutation
-// of the DPP operand, once per value and step (an instruction with a DPP operand occupies the SIMD 2.4 times as long as a
-// plain one on this device, measured, so the multiply-adds themselves take plain operands).
+// its sender is one contiguous 64 bytes over the quad.  The edge's values reach the other lanes once per block: the
+// offset inside the interval and the eight harmonics of the block's four edges are gathered over the quad by one matrix
+// instruction each (quad_gather below), after which every lane holds them for all four steps in plain registers; the two
+// byte offsets of an edge (table row, X row) come from lane j through a quad permutation of the DPP operand of the
+// address addition, once per step.
 //
 // LDS layout of the table slice: interval idx at 512 idx bytes; inside it the (a, b, c, d) of degree li (0 / 1: first /
 // second of the pair), channel 4 k + 2 p + b of the slice at 256 li + 64 (p + 2 b) + 16 k: the four lanes of a quad read
@@ -70,12 +72,17 @@ typedef float f2 __attribute__((ext_vector_type(2)));
 
 // value of `v` in lane J of the reader's quad of four lanes (quad permutation of the DPP operand)
 template <int J>
-__device__ __forceinline__ float quadf(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), J * 0x55, 0xf, 0xf, true));
-}
-template <int J>
 __device__ __forceinline__ unsigned quadu(unsigned v) {
   return static_cast<unsigned>(__builtin_amdgcn_mov_dpp(static_cast<int>(v), J * 0x55, 0xf, 0xf, true));
+}
+
+// The value of `v` in each of the four lanes of the reader's quad: element i is lane i's.  One matrix instruction: the
+// 4x4x1 form works on 16 independent blocks of four lanes, D_b[i][j] = A_b[i] B_b[j] + C_b[i][j], with A_b[i] taken from
+// lane i of the block and row i of D in register i of every lane; B = 1 and C = 0 make it a copy (exact for every
+// normal number).  It runs on the matrix pipe, which this kernel does not use otherwise, in place of four moves with a
+// DPP operand on the vector pipe, which is the one that bounds the kernel.
+__device__ __forceinline__ f4 quad_gather(float v) {
+  return __builtin_amdgcn_mfma_f32_4x4x1f32(v, 1.0f, f4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 }
 
 // the two degrees of pair P and their component counts
@@ -106,6 +113,18 @@ struct Prepared {
   float xr;
   float y[8];
 };
+// offset inside the interval and harmonics of the four edges of a block, in every lane of the quad
+struct Gathered {
+  f4 xr;
+  f4 y[8];
+};
+__device__ __forceinline__ Gathered gather(const Prepared &o) {
+  Gathered g;
+  g.xr = quad_gather(o.xr);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) g.y[i] = quad_gather(o.y[i]);
+  return g;
+}
 struct Raw {  // what a lane loads for its edge of a block
   int s;
   float v0, v1, v2;
@@ -142,15 +161,15 @@ __device__ __forceinline__ void request_row(const float *__restrict__ X, unsigne
 // Steps J .. 3 of a block: `cur` is the block, xin[j] the X values of the edge of step j; as soon as step j has taken
 // them, the values of step j of the block after next (`fut`) are requested into xout[j].
 template <int P, int J>
-__device__ __forceinline__ void edge_step(const float *__restrict__ X, const char *tab, const Prepared &cur, const Prepared &fut,
-                                          const LaneMap &m, const f2 (&xin)[4][2], f2 (&xout)[4][2], f4 (&q)[8],
-                                          float (&acc)[8][4]) {
+__device__ __forceinline__ void edge_step(const float *__restrict__ X, const char *tab, const Prepared &cur, const Gathered &all,
+                                          const Prepared &fut, const LaneMap &m, const f2 (&xin)[4][2], f2 (&xout)[4][2],
+                                          f4 (&q)[8], float (&acc)[8][4]) {
   const float xs[4] = {xin[J][0].x, xin[J][0].y, xin[J][1].x, xin[J][1].y};
   request_row<J>(X, fut.xo, m, xout[J]);
-  const float xr = quadf<J>(cur.xr);
+  const float xr = all.xr[J];
   float y[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) y[i] = quadf<J>(cur.y[i]);
+  for (int i = 0; i < 8; ++i) y[i] = all.y[i][J];
   float t[2][4];
 #pragma unroll
   for (int li = 0; li < 2; ++li)
@@ -166,7 +185,7 @@ __device__ __forceinline__ void edge_step(const float *__restrict__ X, const cha
 #pragma unroll
     for (int d = 0; d < 4; ++d) acc[i][d] = fmaf(y[i], t[i < Pair<P>::M0 ? 0 : 1][d], acc[i][d]);
   __builtin_amdgcn_sched_barrier(0);
-  if constexpr (J + 1 < 4) edge_step<P, J + 1>(X, tab, cur, fut, m, xin, xout, q, acc);
+  if constexpr (J + 1 < 4) edge_step<P, J + 1>(X, tab, cur, all, fut, m, xin, xout, q, acc);
 }
 
 // the rounds of one sorted sub-range: nodes lo + order[0 .. cnt)
@@ -248,6 +267,7 @@ __device__ __forceinline__ void run_rounds(const SlicedArgs &p, const float *sTa
     Prepared p0 = prepare(r0, 0), p1 = prepare(r1, 1), p2;
     f2 x0[4][2], x1[4][2], x2[4][2];
     f4 q[8];
+    Gathered all;
     rows(p0, x0);
     rows(p1, x1);
     for (int blk = 0;; blk += 3) {
@@ -255,22 +275,25 @@ __device__ __forceinline__ void run_rounds(const SlicedArgs &p, const float *sTa
       __builtin_amdgcn_sched_barrier(0);
       p2 = prepare(r2, blk + 2);
       read_pieces<0>(tab, p0.io, m, q);
+      all = gather(p0);
       __builtin_amdgcn_sched_barrier(0);
-      edge_step<P, 0>(p.X, tab, p0, p2, m, x0, x2, q, acc);
+      edge_step<P, 0>(p.X, tab, p0, all, p2, m, x0, x2, q, acc);
       if (!__any(blk + 1 < nblk)) break;
       r1 = request(blk + 4);
       __builtin_amdgcn_sched_barrier(0);
       p0 = prepare(r0, blk + 3);
       read_pieces<0>(tab, p1.io, m, q);
+      all = gather(p1);
       __builtin_amdgcn_sched_barrier(0);
-      edge_step<P, 0>(p.X, tab, p1, p0, m, x1, x0, q, acc);
+      edge_step<P, 0>(p.X, tab, p1, all, p0, m, x1, x0, q, acc);
       if (!__any(blk + 2 < nblk)) break;
       r2 = request(blk + 5);
       __builtin_amdgcn_sched_barrier(0);
       p1 = prepare(r1, blk + 4);
       read_pieces<0>(tab, p2.io, m, q);
+      all = gather(p2);
       __builtin_amdgcn_sched_barrier(0);
-      edge_step<P, 0>(p.X, tab, p2, p1, m, x2, x1, q, acc);
+      edge_step<P, 0>(p.X, tab, p2, all, p1, m, x2, x1, q, acc);
       if (!__any(blk + 3 < nblk)) break;
     }
 
