@@ -97,9 +97,9 @@ struct Pair {
 
 // the eight harmonics of pair P (the unused ones of the full evaluation fall away at compile time)
 template <int P>
-__device__ __forceinline__ void harmonics(float v0, float v1, float v2, float (&y)[8]) {
+__device__ __forceinline__ void harmonics(float v0, float v1, float v2, float inv_len, float (&y)[8]) {
   float all[16];
-  sh::eval(sh::direction(v0, v1, v2), all);
+  sh::eval(sh::Direction{v2 * inv_len, v0 * inv_len, v1 * inv_len, inv_len}, all);
 #pragma unroll
   for (int i = 0; i < 8; ++i) y[i] = all[Pair<P>::row(i)];
 }
@@ -206,6 +206,7 @@ __device__ __forceinline__ void run_rounds(const SlicedArgs &p, const float *sTa
   const int C = p.C;
   const int last_edge = static_cast<int>(p.nedges) - 1;  // the launcher does not come here without edges
   const unsigned zero_row = static_cast<unsigned>(p.nknots - 1) * 512u;
+  const float inv_width = 1.0f / p.r_width;
 
   for (;;) {
     int base = 0;
@@ -237,20 +238,26 @@ __device__ __forceinline__ void run_rounds(const SlicedArgs &p, const float *sTa
     auto prepare = [&](const Raw &r, int blk) {
       Prepared o;
       const bool valid = e0 + 4 * blk + k < e1;
-      const float len = edge_length(r.v0, r.v1, r.v2);
-      int idx = -1;
-      o.xr = 0.f;
-      if (valid && len <= p.r_max) {
-        idx = static_cast<int>(len / p.r_width);
-        idx = idx < 0 ? 0 : (idx > p.nknots - 2 ? p.nknots - 2 : idx);
-        o.xr = len - sKnots[idx];
-      }
-      const bool live = idx >= 0 && static_cast<unsigned>(r.s) < static_cast<unsigned>(p.nnodes);
-      harmonics<P>(r.v0, r.v1, r.v2, o.y);
+      // Length and direction from one reciprocal square root (the hardware's, one Newton step: within an ulp) and the
+      // interval from a product with 1 / width: the correctly rounded square root and the two divisions they stand for
+      // are 40 instructions per edge, and every one of the 16 workgroup types of a piece of the node range prepares
+      // every edge.  An edge within rounding of a knot may land in the neighbouring interval, whose cubic continues
+      // the spline there (value and two derivatives agree at the knot).
+      const float r2 = fmaf(r.v2, r.v2, fmaf(r.v1, r.v1, r.v0 * r.v0));
+      float ir = __builtin_amdgcn_rsqf(r2);
+      ir = ir * fmaf(-0.5f * r2 * ir, ir, 1.5f);
+      const float len = r2 * ir;  // NaN for a vector of zeros: such an edge does not count
+      // without a branch (the interval of an edge that does not count is looked up and dropped): under a branch the
+      // knot's way from LDS is waited for on the spot, here it arrives while the harmonics are formed
+      int idx = static_cast<int>(len * inv_width);
+      idx = idx < 0 ? 0 : (idx > p.nknots - 2 ? p.nknots - 2 : idx);
+      const float knot = sKnots[idx];
+      const bool live = valid && len <= p.r_max && static_cast<unsigned>(r.s) < static_cast<unsigned>(p.nnodes);
+      harmonics<P>(r.v0, r.v1, r.v2, ir, o.y);
 #pragma unroll
       for (int i = 0; i < 8; ++i) o.y[i] = live ? o.y[i] : 0.f;
-      o.xr = live ? o.xr : 0.f;
-      o.xo = live ? static_cast<unsigned>(r.s) * static_cast<unsigned>(4 * C) : own_row;
+      o.xr = live ? len - knot : 0.f;
+      o.xo = live ? __umul24(static_cast<unsigned>(r.s), static_cast<unsigned>(4 * C)) : own_row;  // both below 2^24
       o.io = live ? static_cast<unsigned>(idx) * 512u : zero_row;
       return o;
     };
@@ -394,7 +401,7 @@ __global__ __launch_bounds__(kSlThreads) void mp_edge_forward_sliced_kernel(cons
 }  // namespace
 
 bool sliced_forward_applies(int64_t nnodes, int channels, int nknots) {
-  return nnodes >= kSlMinNodes && nnodes * channels < (int64_t{1} << 30) && channels % 16 == 0 && nknots >= 2 &&
+  return nnodes >= kSlMinNodes && nnodes < (1 << 24) && nnodes * channels < (int64_t{1} << 30) && channels % 16 == 0 && nknots >= 2 &&
          nknots - 1 < kSlMaxIntervals && device_compute_units() / (2 * (channels / 16)) >= 2;
 }
 
