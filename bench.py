@@ -81,7 +81,7 @@ def traffic_of(table, kernels):
 def forward_kernel_name(C, N):
     """Kernel that runs the fused forward from edge vectors at this shape (csrc/mp_spline.hip: cm_mp_edge_forward; the
     benchmark's spline table has 256 knots)."""
-    if N >= 2048 and C % 16 == 0 and N * C < 2**30:
+    if 2048 <= N < 2**24 and C % 16 == 0 and N * C < 2**30:
         return "mp_edge_forward_sliced_kernel"
     return "mp_spline_forward_kernel<%d,true>" % C
 
@@ -148,7 +148,7 @@ def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=
         ("mp_backward gY,gR (tabulated R)", "mp_backward_edge_kernel<%d,true,true,false>" % C, bwd_b,
          lambda: cabi.mp_backward(X, Y, R, G, snd, fo, None, None, N, need_gX=False)),
         ("mp_backward gX,gY,gR (tabulated R): edge pass + sender pass",
-         "mp_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,0>" % (C, C), bwd_full_b,
+         "mp_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,0,false>" % (C, C), bwd_full_b,
          lambda: cabi.mp_backward(X, Y, R, G, snd, fo, perm, off, N)),
     ]
     if with_per_component:
@@ -158,7 +158,7 @@ def op_cases(torch, cabi, N, E, C, ne, rcv, snd, with_fused=True, with_node_ops=
             ("mp_forward (R per component [E,16,C])", "mp_per_m_forward_kernel<%d>" % C,
              4 * (16 * E * C + 16 * E + 17 * N * C) + 8 * E, lambda: cabi.mp_forward(X, Y, R16, snd, fo, N)),
             ("mp_backward gX,gY,gR (R per component): edge pass + sender pass",
-             "mp_per_m_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,0>" % (C, C),
+             "mp_per_m_backward_edge_kernel<%d,true,true,true> + mp_backward_sender_kernel<%d,0,false>" % (C, C),
              4 * (32 * E * C + 32 * E + 18 * N * C) + 8 * E, lambda: cabi.mp_backward(X, Y, R16, G, snd, fo, perm, off, N)),
         ]
     if with_fused:
