@@ -46,14 +46,24 @@ struct Spline {
   float r_max;
 };
 
-// Knot interval (or -1 beyond the cutoff) and offset inside it for one edge length.
-__device__ __forceinline__ void locate(const Spline &sp, float re, int &idx, float &x) {
+// Knot interval (or -1 beyond the cutoff) and offset inside it for one edge length.  lds_knots: a copy of the knots in LDS,
+// read instead of the one in memory if use_lds.
+__device__ __forceinline__ void locate(const Spline &sp, float re, int &idx, float &x, const float *lds_knots = nullptr,
+                                       bool use_lds = false) {
   idx = -1;
   x = 0.f;
   if (re <= sp.r_max) {
     idx = static_cast<int>(re / sp.r_width);
     idx = idx < 0 ? 0 : (idx > sp.nknots - 2 ? sp.nknots - 2 : idx);
-    x = re - sp.knots[idx];
+    // The markers keep each read and its use inside its branch: merged, the two become one read through a generic
+    // address, or one subtraction behind a wait for the read of memory, on the path that reads LDS as well.
+    if (use_lds) {
+      x = re - lds_knots[idx];
+      asm volatile("; offset from the knot in LDS" : "+v"(x));
+    } else {
+      x = re - sp.knots[idx];
+      asm volatile("; offset from the knot in memory" : "+v"(x));
+    }
   }
 }
 
@@ -65,13 +75,24 @@ __device__ __forceinline__ void locate(const Spline &sp, float re, int &idx, flo
 // was consumed; `dead(pass_base, consumed, live_mask, lane_is_dead)` is called once per pass for the consumed edges that
 // are not live (the backward writes their zeros there).  Returns the number of staged edges (the same in every lane).
 // FROM_VEC: Y and the length come from the edge vector; otherwise from the Y and r arrays.
-template <bool FROM_VEC, class DeadFn>
+// `ahead` (AHEAD, FROM_VEC only): sender and vector of edge base + lane, which the caller asked for before it
+// called (so that loads it issued in between do not stand in front of them in the queue); used by the first pass.
+struct RawEdge {
+  int s;
+  float v0, v1, v2;
+};
+template <bool FROM_VEC, bool AHEAD = false, class DeadFn>
 __device__ __forceinline__ int stage_edges(const float *__restrict__ Y, const int32_t *__restrict__ sender, const Spline &sp,
                                            int nnodes, int64_t nedges, int &base, int e1, int lane, float *sY, int *sS,
-                                           int *sIdx, float *sXr, int *sOrig, DeadFn dead) {
+                                           int *sIdx, float *sXr, int *sOrig, DeadFn dead,
+                                           RawEdge ahead = RawEdge{-1, 0.f, 0.f, 0.f}, const float *lds_knots = nullptr,
+                                           bool use_lds_knots = false) {
+  static_assert(FROM_VEC || !AHEAD, "raw edges are handed in for the edge-vector variant only");
   const int first = base;
   int nlive = 0;
-  while (nlive < kChunk && base < e1) {
+  // one pass over up to kChunk raw edges; the first one is written out on its own where its raw edges are handed in, so
+  // that its waits are not those of a pass that has just issued its loads
+  auto pass = [&](auto use_ahead) {
     const int cnt = min(kChunk, e1 - base);
     int s = -1, idx = -1;
     float x = 0.f;
@@ -80,13 +101,18 @@ __device__ __forceinline__ int stage_edges(const float *__restrict__ Y, const in
     for (int m = 0; m < 16; ++m) y[m] = 0.f;
     if (lane < cnt) {
       const int64_t e = base + lane;
-      s = sender[e];
       if constexpr (FROM_VEC) {
-        const float v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
-        locate(sp, edge_length(v0, v1, v2), idx, x);
+        float v0, v1, v2;
+        if constexpr (decltype(use_ahead)::value) {
+          s = ahead.s, v0 = ahead.v0, v1 = ahead.v1, v2 = ahead.v2;
+        } else {
+          s = sender[e], v0 = sp.vec[3 * e + 0], v1 = sp.vec[3 * e + 1], v2 = sp.vec[3 * e + 2];
+        }
+        locate(sp, edge_length(v0, v1, v2), idx, x, lds_knots, use_lds_knots);
         sh::eval(sh::direction(v0, v1, v2), y);
       } else {
-        locate(sp, sp.r[e], idx, x);
+        s = sender[e];
+        locate(sp, sp.r[e], idx, x, lds_knots, use_lds_knots);
 #pragma unroll
         for (int m = 0; m < 16; ++m) y[m] = Y[m * nedges + e];
       }
@@ -110,9 +136,15 @@ __device__ __forceinline__ int stage_edges(const float *__restrict__ Y, const in
     dead(base, consumed, live_mask, lane < consumed && !live);
     nlive = min(kChunk, nlive + nlive_pass);
     base += consumed;
+  };
+  if constexpr (AHEAD) {
+    if (base < e1) pass(std::true_type{});
   }
+  while (nlive < kChunk && base < e1) pass(std::false_type{});
   return nlive;
 }
+
+constexpr int kKnotsInLds = 512;  // knots the backward edge pass keeps in LDS (more are read from memory)
 
 // LDS of one wave's staged chunk: Y [kChunk][16], sender, knot interval, offset in it, position (floats / ints)
 constexpr int kStageBytes = kChunk * 64 + 4 * kChunk * 4;
@@ -304,6 +336,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   __shared__ int sOrig[kChunk];
   __shared__ float sGY[16 * kChunk];  // [m][edge]
   __shared__ float sGr[kChunk];
+  // The knots, where there are at most kKnotsInLds of them: the staging looks one up per edge, and a lookup in memory is
+  // waited for behind everything the wave has in flight (the gradient rows from HBM first of all).
+  __shared__ float sKnots[kKnotsInLds];
 
   // one wave per node, or (few nodes: parts_for) per part of a node's edge range: every output of this pass belongs to
   // one edge, so the parts share nothing but the node's gradient rows, which each of them reads
@@ -313,6 +348,11 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   const int cl = lane % K::SW;
   const bool active = cl < K::LPE;
   const unsigned cla = active ? cl : 0;  // lanes beyond the channel count read lane 0's addresses; their g is zero
+  const bool knots_in_lds = sp.nknots <= kKnotsInLds;
+  float knot[kKnotsInLds / kWave];
+#pragma unroll
+  for (int q = 0; q < kKnotsInLds / kWave; ++q) knot[q] = sp.knots[min(lane + kWave * q, sp.nknots - 1)];
+  __builtin_amdgcn_sched_barrier(0);
   int e0 = first_occ[node];
   int e1 = first_occ[nnodes + node];
   clamp_edge_range(e0, e1, nedges);
@@ -325,16 +365,37 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
   }
   if (e0 >= e1) return;
 
+  // Order of the first requests: the raw edges of the first chunk (from L2, and the staging waits for them), then the
+  // node's gradient rows (from HBM, read once, not needed before the first edge's arithmetic).  Memory operations retire
+  // in issue order, so with the rows in front the staging would wait for them as well.
+  RawEdge ahead{-1, 0.f, 0.f, 0.f};
+  if constexpr (FROM_VEC) {
+    const int64_t e = min(static_cast<int64_t>(e0) + lane, nedges - 1);  // unconditional; lanes beyond the range drop it
+    ahead.s = sender[e];
+    ahead.v0 = sp.vec[3 * e + 0], ahead.v1 = sp.vec[3 * e + 1], ahead.v2 = sp.vec[3 * e + 2];
+    __builtin_amdgcn_sched_barrier(0);
+  }
   vec g[16];
   {
     const float *gp = G + static_cast<int64_t>(node) * (16 * C) + K::off(cl);
 #pragma unroll
     for (int m = 0; m < 16; ++m) g[m] = active ? K::ld_stream(gp + m * C) : zerov<vec>();  // read once
   }
+  __builtin_amdgcn_sched_barrier(0);
+  if (knots_in_lds) {
+#pragma unroll
+    for (int q = 0; q < kKnotsInLds / kWave; ++q) sKnots[lane + kWave * q] = knot[q];
+  }
 
-  for (int cursor = e0; cursor < e1;) {
+  // The first chunk is written out ahead of the loop over the others (most nodes have no others): at a loop's head the
+  // compiler has to assume that the loads a previous iteration left in flight (a slot's last, unused look-ahead) are still
+  // on their way into registers the staging reuses, and waits for everything, the gradient rows included.
+  int cursor = e0;
+  auto chunk = [&](auto first_chunk) {
     const int base = cursor;  // sOrig counts from here
-    __syncthreads();
+    // (the workgroup is this one wave: ordering its own LDS traffic is all that is needed, and a workgroup barrier would
+    // wait for everything in flight first, the gradient rows and the previous chunk's stores included)
+    wave_lds_fence();
     // consumed edges that are not live: their gradients are zeros (their rows of gXe stay unwritten: the sender pass
     // reads the rows of live edges only)
     auto dead = [&](int pass_base, int, unsigned long long, bool lane_is_dead) {
@@ -355,8 +416,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
         }
       }
     };
-    const int nlive = stage_edges<FROM_VEC>(Y, sender, sp, nnodes, nedges, cursor, e1, lane, sY, sS, sIdx, sXr, sOrig, dead);
-    __syncthreads();
+    const int nlive = stage_edges<FROM_VEC, FROM_VEC && decltype(first_chunk)::value>(
+        Y, sender, sp, nnodes, nedges, cursor, e1, lane, sY, sS, sIdx, sXr, sOrig, dead, ahead, sKnots, knots_in_lds);
+    wave_lds_fence();
     // Every lane of a slot takes part in the reductions, so the loop bound is slot-uniform; only live edges are staged.
     // The loop is rotated: the sender row and the 16 coefficient pieces of the NEXT edge are requested right after the
     // arithmetic of the current one, so they travel while the cross-lane reductions (a chain of dependent lane
@@ -449,7 +511,7 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
       edge(opb, j + K::EPW, opa);
     }
     if constexpr (WANT_GY || WANT_GR) {
-      __syncthreads();
+      wave_lds_fence();
       // lane k < nlive finishes the k-th staged edge
       if (lane < nlive) {
         const int64_t e = base + sOrig[lane];
@@ -483,7 +545,9 @@ __global__ __launch_bounds__(kWave, CM_FUSED_BWD_WAVES) void mp_spline_backward_
         }
       }
     }
-  }
+  };
+  chunk(std::true_type{});
+  while (cursor < e1) chunk(std::false_type{});
 }
 
 template <int C, bool FROM_VEC>
