@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kWave) void mp_per_m_forward_kernel(const float *__
     stage_chunk(Y, sender, nedges, base, cnt, lane, sY, sS);
     __syncthreads();
     if (active) {
-      for (int j = slot; j < cnt; j += K::EPW) {
+      auto one = [&](int j) {
         const int64_t e = base + j;
         const int s = sS[j];
         const float *rp = R + e * (16 * C) + K::off(cl);
@@ -53,7 +53,14 @@ __global__ __launch_bounds__(kWave) void mp_per_m_forward_kernel(const float *__
         const float *yp = sY + j * 16;
 #pragma unroll
         for (int m = 0; m < 16; ++m) acc[m] += (yp[m] * x) * r[m];
+      };
+      // two edges per slot at a time, their 2 x 16 rows requested together
+      int j = slot;
+      for (; j + K::EPW < cnt; j += 2 * K::EPW) {
+        one(j);
+        one(j + K::EPW);
       }
+      if (j < cnt) one(j);
     }
   }
 #pragma unroll
