@@ -131,18 +131,22 @@ __global__ __launch_bounds__(kWave) void mp_forward_kernel(
         acc[15] += yd.w * t3;
       };
       // Edges in blocks of eight (from 128 channels on), four, two, one per slot: the loads of a block are requested
-      // together (8 x 4 rows of R in flight per wave keep the stream at 5.8 TB/s where 2 x 4 give 5.5), and a node's
-      // last edges take the largest block that still fits instead of one edge at a time.
+      // together (8 x 4 rows of R in flight per wave keep the stream at 5.9 TB/s where 2 x 4 give 5.5), and a node's
+      // last edges take the largest block that still fits instead of one edge at a time.  A block's rows and the 16
+      // accumulators have to fit the register file: 5 V and 16 V registers for V channels per lane, so five channels
+      // per lane (160 channels) stop at blocks of four and seven (224 channels) at blocks of two.
       int j = slot;
-      if constexpr (C >= 128) {
+      if constexpr (C >= 128 && K::V <= 4) {
         for (; j + 7 * K::EPW < cnt; j += 8 * K::EPW) {
 #pragma unroll
           for (int u = 0; u < 8; ++u) one(j + u * K::EPW);
         }
       }
-      for (; j + 3 * K::EPW < cnt; j += 4 * K::EPW) {
+      if constexpr (K::V <= 5) {
+        for (; j + 3 * K::EPW < cnt; j += 4 * K::EPW) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) one(j + u * K::EPW);
+          for (int u = 0; u < 4; ++u) one(j + u * K::EPW);
+        }
       }
       for (; j + K::EPW < cnt; j += 2 * K::EPW) {
         one(j);
