@@ -325,16 +325,23 @@ __global__ __launch_bounds__(kSlThreads) void mp_edge_forward_sliced_kernel(cons
 
   const int tid = threadIdx.x;
   // Which (pair, slice) and which piece j of the node range.  Consecutive workgroups go to consecutive XCDs (eight of
-  // them, each with its own L2): where the pieces divide evenly among the XCDs, all workgroups of a piece sit on one XCD,
-  // so that the edge data and the X rows of a piece are fetched into one L2 only.
+  // them, each with its own L2): all workgroups of a piece sit on one XCD, so that the edge data and the X rows of the
+  // piece are fetched into one L2 only, for as many pieces as divide evenly among the XCDs (all of them at 64, 128 and
+  // 256 channels).
   int type, j;
-  if (p.share % 8 == 0) {
-    const int xcd = blockIdx.x % 8, q = blockIdx.x / 8;
-    type = q % (2 * p.nslices);
-    j = xcd + 8 * (q / (2 * p.nslices));
-  } else {
-    type = blockIdx.x % (2 * p.nslices);
-    j = blockIdx.x / (2 * p.nslices);
+  {
+    const int types = 2 * p.nslices;
+    const int aligned = (p.share / 8) * 8;  // pieces that go to one XCD each; the others are spread over all of them
+    const int b = blockIdx.x;
+    if (b < aligned * types) {
+      const int xcd = b % 8, q = b / 8;
+      type = q % types;
+      j = xcd + 8 * (q / types);
+    } else {
+      const int rest = b - aligned * types;
+      type = rest % types;
+      j = aligned + rest / types;
+    }
   }
   const int slice = type >> 1;
   const int pair = type & 1;
