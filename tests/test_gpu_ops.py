@@ -128,6 +128,32 @@ def test_mp_forward(cabi, case):
     close(out, ref, RTOL, ATOL)
 
 
+@pytest.mark.parametrize("C", [64, 96, 128, 160, 224])
+def test_mp_forward_every_edge_count(cabi, C):
+    """Node i receives i edges, i = 0 .. 140: the forward takes a slot's edges in blocks of eight, four, two and one (which
+    of them depends on the channels per lane), so every remainder of every block size occurs, in one chunk of 64 staged
+    edges and across chunks; per-component weights take two edges at a time."""
+    import numpy as np
+
+    _say("mp_forward every edge count", C)
+    nnodes = 141
+    rng = np.random.default_rng(C)
+    rcv = torch.from_numpy(np.repeat(np.arange(nnodes), np.arange(nnodes)).astype(np.int32))
+    E = rcv.numel()
+    snd = torch.from_numpy(rng.integers(0, nnodes, E).astype(np.int32))
+    X, v, R, _ = mp_inputs(nnodes, E, C, C)
+    Y = O.spherical_harmonics(v).contiguous()
+    fo = cabi.first_occurences(rcv.to(DEV), nnodes)
+    out = cabi.mp_forward(X.float().to(DEV), Y.float().to(DEV), R.float().to(DEV), snd.to(DEV), fo, nnodes)
+    close(out, O.mp_forward(X, Y, R, snd, rcv, nnodes), RTOL, ATOL)
+    assert float(out[0].abs().max()) == 0.0  # the node without edges
+    if C <= 128:
+        g = torch.Generator().manual_seed(C + 1)
+        R16 = torch.randn(E, 16, C, generator=g, dtype=torch.float64)
+        out16 = cabi.mp_forward(X.float().to(DEV), Y.float().to(DEV), R16.float().to(DEV), snd.to(DEV), fo, nnodes)
+        close(out16, O.mp_forward(X, Y, R16, snd, rcv, nnodes), RTOL, ATOL)
+
+
 @pytest.mark.parametrize("case", MP_CASES, ids=lambda c: "N%d_d%d_C%d_%s_s%d" % (c[0], c[1], c[2], c[3], c[5]))
 def test_mp_backward(cabi, case):
     _say("mp_backward", case)
