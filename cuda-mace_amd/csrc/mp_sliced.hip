@@ -242,7 +242,9 @@ __device__ __forceinline__ void run_rounds(const SlicedArgs &p, const float *sTa
       // interval from a product with 1 / width: the correctly rounded square root and the two divisions they stand for
       // are 40 instructions per edge, and every one of the 16 workgroup types of a piece of the node range prepares
       // every edge.  An edge within rounding of a knot may land in the neighbouring interval, whose cubic continues
-      // the spline there (value and two derivatives agree at the knot).
+      // the spline there (value and two derivatives agree at the knot); one within rounding of the cutoff may be kept
+      // or dropped, where the tabulated functions of a model end in zero (their envelope) and a table that does not
+      // is cut off at a length that is only known to that rounding anyway.
       const float r2 = fmaf(r.v2, r.v2, fmaf(r.v1, r.v1, r.v0 * r.v0));
       float ir = __builtin_amdgcn_rsqf(r2);
       ir = ir * fmaf(-0.5f * r2 * ir, ir, 1.5f);
